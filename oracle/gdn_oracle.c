@@ -7,7 +7,7 @@
  * Follows qwen35/batch.py:36-125 (deltanet_b), qwen35/kernels.py:476-541 (deltanet), qwen35/mslib.py:7-27
  * (bf16 rounding structure of sigmoid / silu / softplus) and qwen35/gated_delta.py:75-126 (the recurrence).
  * The arithmetic contract is the one of gdn_oracle.py: exp/log are the double-precision libm results rounded
- * to float, sums of squares are exact (double) and rounded once, rsqrt = 1/sqrtf, and the dot products of the
+ * to float, sums of squares are exact (double) and rounded once, rsqrt = (float)(1/sqrt) in double, and the dot products of the
  * recurrence are accumulated in double (acc64 != 0) or in float, sequentially (acc64 == 0).
  *
  * Build: gcc -O2 -fopenmp -ffp-contract=off -shared -fPIC gdn_oracle.c -o libgdn_oracle.so -lm
@@ -63,7 +63,7 @@ static void norm_scale(float* u, float sc) { /* kernels.py:504-510 */
     const float e2 = (1e-6f * inv_scale) * inv_scale;
     double ss = 0.0;
     for (int i = 0; i < DK; i++) ss += (double)u[i] * (double)u[i];
-    float r = 1.0f / sqrtf((float)ss / (float)DK + e2);
+    float r = (float)(1.0 / sqrt((double)((float)ss / (float)DK + e2)));
     for (int i = 0; i < DK; i++) u[i] = BF(BF(u[i] * r) * sc);
 }
 

@@ -11,7 +11,7 @@ Arithmetic contract shared with the HIP kernels (so that the elementwise prologu
     for all practical purposes); the reference uses metal::precise::exp / log, whose last-ulp behaviour is
     not available off Apple hardware.
   * sums of squares of bf16 values are exact (accumulated in float64) and then rounded to float32 once.
-  * rsqrt(x) = 1 / sqrt(x) with IEEE float32 sqrt and divide.
+  * rsqrt(x) = 1 / sqrt(x) evaluated in float64 and rounded to float32 once.
   * the recurrence itself (dot products over Dk) is accumulated in `acc` precision (float64 by default);
     the kernels accumulate in float32, which is what the 1e-4 tolerance covers.
 
@@ -58,8 +58,7 @@ def log32(x):
 
 
 def rsqrt32(x):
-    x = np.asarray(x, dtype=np.float32)
-    return (F32(1.0) / np.sqrt(x)).astype(np.float32)
+    return (1.0 / np.sqrt(np.asarray(x, dtype=np.float32).astype(np.float64))).astype(np.float32)
 
 
 def log1p_mx(x):

@@ -1,0 +1,91 @@
+"""ctypes binding of csrc/libqwen_tailor_hip.so (the C ABI declared in include/qwen_tailor_hip.h).
+
+There is no CPU fallback: every operator of this package runs a HIP kernel or raises."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+from . import _build
+
+_lib = None
+_vp, _i, _l, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
+
+ERRORS = {-1: "bad dimension", -2: "misaligned pointer", -3: "null pointer", -4: "unsupported shape", -5: "kernel launch failed",
+          -6: "workspace too small"}
+
+_SIGS = {
+    "qt_gdn_decode_step": [_vp] * 9 + [_i, _i, _i, _vp],
+    "qt_gdn_verify_step": [_vp] * 10 + [_i, _i, _i, _i, _vp],
+    "qt_gdn_deltanet": [_vp] * 10 + [_i, _i, _i, _vp],
+    "qt_gdn_gates": [_vp, _vp, _l, _l, _vp, _vp, _vp, _vp, _vp, _l, _i, _vp],
+    "qt_normalize_qk": [_vp, _vp, _vp, _vp, _l, _i, _vp],
+    "qt_gdn_conv_prep": [_vp] * 6 + [_i, _vp],
+    "qt_gated_rmsnorm": [_vp, _vp, _vp, _vp, _l, _f, _vp],
+    "qt_gdn_recurrent": [_vp] * 8 + [_i] * 6 + [_vp],
+}
+
+
+def lib():
+    """The loaded library.  Builds it first if no built library is present; raises if that is impossible."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_build.SO):
+            _build.build()
+        L = ctypes.CDLL(_build.SO)
+        for name, args in _SIGS.items():
+            fn = getattr(L, name)
+            fn.argtypes, fn.restype = args, ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def declare(name, args):
+    """Register the signature of one more entry point (used by the modules that own it)."""
+    _SIGS[name] = args
+    if _lib is not None:
+        fn = getattr(_lib, name)
+        fn.argtypes, fn.restype = args, ctypes.c_int
+
+
+def call(name, *args):
+    rc = getattr(lib(), name)(*args)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed: {ERRORS.get(rc, rc)}")
+
+
+def stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def dev(t, dtype, name, shape=None):
+    """Check that `t` is a contiguous device tensor of `dtype` (and of `shape`, None entries free); return it."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError(f"{name}: expected a tensor on the GPU")
+    if t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
+    if shape is not None:
+        if t.dim() != len(shape) or any(s is not None and s != d for s, d in zip(shape, t.shape)):
+            raise ValueError(f"{name}: expected shape {shape}, got {tuple(t.shape)}")
+    return t
+
+
+def f32(t, name, shape=None):
+    """Per-head parameter vectors (A_log, dt_bias, norm weight) are consumed as float32."""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError(f"{name}: expected a tensor on the GPU")
+    if t.dtype != torch.float32 or not t.is_contiguous():
+        t = t.float().contiguous()
+    return dev(t, torch.float32, name, shape)
+
+
+def i32(t, name, n=None):
+    return dev(t, torch.int32, name, None if n is None else (n,))

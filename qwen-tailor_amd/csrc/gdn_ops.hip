@@ -1,0 +1,220 @@
+// Stand-alone pieces of the GatedDeltaNet layer core for gfx950: gates, q/k norm, conv4+SiLU+norm over S tokens, gated
+// RMSNorm and the sequential recurrence.  Arithmetic contract: see qt_common.h.
+#include "qt_common.h"
+
+using namespace qt;
+
+namespace {
+
+// compute_g + beta (qwen35/gated_delta.py:16-18,158; rounding points of qwen35/kernels.py:511-515).
+// a, b are read with a row stride so they can be taken straight out of the 8224-wide projection row.
+__global__ __launch_bounds__(256) void gates_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ b, long a_stride,
+                                                    long b_stride, const float* __restrict__ A_log,
+                                                    const float* __restrict__ dt_bias, float* __restrict__ g,
+                                                    float* __restrict__ lg, bf16_t* __restrict__ beta, long rows, int hv) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * hv) return;
+    const long r = i / hv;
+    const int h = (int)(i % hv);
+    const float av = BF(bf2f(a[r * a_stride + h]) + dt_bias[h]);
+    const float l = -exp32(A_log[h]) * softplus_bf16(av);
+    if (g) g[i] = exp32(l);
+    if (lg) lg[i] = l;
+    if (beta) beta[i] = f2bf(sigmoid_bf16(bf2f(b[r * b_stride + h])));
+}
+
+// normalize_qk (qwen35/gated_delta.py:21-30) on rows of 128: one wavefront per row, two elements per lane
+__global__ __launch_bounds__(256) void normalize_qk_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                           bf16_t* __restrict__ qo, bf16_t* __restrict__ ko, long rows) {
+    const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
+    const uint32_t wq = reinterpret_cast<const uint32_t*>(q + row * DK)[lane];
+    const uint32_t wk = reinterpret_cast<const uint32_t*>(k + row * DK)[lane];
+    const float q0 = lo_bf(wq), q1 = hi_bf(wq), k0 = lo_bf(wk), k1 = hi_bf(wk);
+    const float qs = (float)wave_sum_d((double)q0 * q0 + (double)q1 * q1);
+    const float ks = (float)wave_sum_d((double)k0 * k0 + (double)k1 * k1);
+    const float qr = rsqrt_rn(qs / (float)DK + qk_eps()), kr = rsqrt_rn(ks / (float)DK + qk_eps());
+    reinterpret_cast<uint32_t*>(qo + row * DK)[lane] = pack_bf(BF(BF(q0 * qr) * scq), BF(BF(q1 * qr) * scq));
+    reinterpret_cast<uint32_t*>(ko + row * DK)[lane] = pack_bf(BF(BF(k0 * kr) * sck), BF(BF(k1 * kr) * sck));
+}
+
+// conv_prep (qwen35/prefill.py:96-134, 228-238): one workgroup of 128 threads per (token, head); thread i owns channel i
+// of the head's q, k and v.  proj [S,8224], cs [3,6144] -> q, k, v [S,16,128].
+__global__ __launch_bounds__(128) void conv_prep_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs,
+                                                        const bf16_t* __restrict__ cw, bf16_t* __restrict__ q,
+                                                        bf16_t* __restrict__ k, bf16_t* __restrict__ v, int S) {
+    __shared__ double red[2][2];
+    const int t = blockIdx.x / HV, h = blockIdx.x % HV, i = threadIdx.x, w = i >> 6;
+    float u[3];
+#pragma unroll
+    for (int part = 0; part < 3; part++) {
+        const int ch = part * KD + h * DK + i;
+        float x[4];
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const int tt = t - 3 + d;
+            x[d] = tt < 0 ? bf2f(cs[(tt + 3) * CD + ch]) : bf2f(proj[(size_t)tt * PW + ch]);
+        }
+        u[part] = conv_silu(x[0], x[1], x[2], x[3], *reinterpret_cast<const uint2*>(cw + (size_t)ch * 4));
+    }
+    const double sq = wave_sum_d((double)u[0] * u[0]), sk = wave_sum_d((double)u[1] * u[1]);
+    if ((i & 63) == 0) {
+        red[0][w] = sq;
+        red[1][w] = sk;
+    }
+    __syncthreads();
+    const float qr = rsqrt_rn((float)(red[0][0] + red[0][1]) / (float)DK + qk_eps());
+    const float kr = rsqrt_rn((float)(red[1][0] + red[1][1]) / (float)DK + qk_eps());
+    const size_t o = ((size_t)t * HV + h) * DK + i;
+    q[o] = f2bf(BF(BF(u[0] * qr) * BF(INV_SCALE * INV_SCALE)));
+    k[o] = f2bf(BF(BF(u[1] * kr) * BF(INV_SCALE)));
+    v[o] = f2bf(u[2]);
+}
+
+// gated RMSNorm (qwen35/batch.py:304-343, qwen35/prefill.py:137-157): 16 lanes per (row, head), 8 elements per lane.
+__global__ __launch_bounds__(256) void gated_norm_kernel(const bf16_t* __restrict__ y, const bf16_t* __restrict__ proj,
+                                                         const float* __restrict__ gw, bf16_t* __restrict__ out, long rows,
+                                                         float eps) {
+    const long grp = (long)blockIdx.x * 16 + (threadIdx.x >> 4);       // (row, head)
+    const int c = threadIdx.x & 15;
+    if (grp >= rows * HV) return;
+    const long row = grp / HV;
+    const int h = (int)(grp % HV);
+    const uint4 yv = reinterpret_cast<const uint4*>(y + row * KD + h * DV)[c];
+    const uint4 zv = reinterpret_cast<const uint4*>(proj + row * PW + CD + h * DV)[c];
+    const uint32_t yw[4] = {yv.x, yv.y, yv.z, yv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
+    float yy[8], zz[8];
+    double ss = 0.0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        yy[2 * j] = lo_bf(yw[j]);
+        yy[2 * j + 1] = hi_bf(yw[j]);
+        zz[2 * j] = lo_bf(zw[j]);
+        zz[2 * j + 1] = hi_bf(zw[j]);
+        ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
+    }
+    const float inv = rsqrt_rn((float)row16_sum_d(ss) / 128.f + eps);
+    float o[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float n = gw[c * 8 + j] * (yy[j] * inv);
+        const float sig = __fdiv_rn(zz[j], 1.0f + exp32(-zz[j]));
+        o[j] = sig * n;
+    }
+    uint4 ov = make_uint4(pack_bf(o[0], o[1]), pack_bf(o[2], o[3]), pack_bf(o[4], o[5]), pack_bf(o[6], o[7]));
+    reinterpret_cast<uint4*>(out + row * KD + h * DV)[c] = ov;
+}
+
+// gated_delta_update's kernel (qwen35/gated_delta.py:33-137): T sequential tokens with q, k, v, g, beta given.
+// One workgroup of 256 threads per (batch, value head, 16-row block); a 16-lane group owns one value row, a lane 8 of its
+// 128 columns; no LDS, no barriers.  q, k [B,T,Hk,128], v, y [B,T,Hv,Dv], g f32 / beta bf16 [B,T,Hv], state [B,Hv,Dv,128].
+__global__ __launch_bounds__(256) void recurrent_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                        const bf16_t* __restrict__ v, const float* __restrict__ g,
+                                                        const bf16_t* __restrict__ beta, const float* st_in,
+                                                        float* st_out, bf16_t* __restrict__ y, int T, int Hk, int Hv,
+                                                        int Dv) {
+    const int nblk = Dv / 16;
+    const int blk = blockIdx.x % nblk, n = blockIdx.x / nblk;             // n = b*Hv + hv
+    const int b = n / Hv, hv = n % Hv, hk = hv / (Hv / Hk);              // gated_delta.py:43-46
+    const int tid = threadIdx.x, c = tid & 15;
+    const int row = blk * 16 + (tid >> 4);
+    const size_t so = ((size_t)n * Dv + row) * DK;
+    float sv[8];
+    {
+        const float4 a = reinterpret_cast<const float4*>(st_in + so)[c], d = reinterpret_cast<const float4*>(st_in + so)[16 + c];
+        sv[0] = a.x; sv[1] = a.y; sv[2] = a.z; sv[3] = a.w; sv[4] = d.x; sv[5] = d.y; sv[6] = d.z; sv[7] = d.w;
+    }
+    const bf16_t* qp = q + ((size_t)b * T * Hk + hk) * DK;
+    const bf16_t* kp = k + ((size_t)b * T * Hk + hk) * DK;
+    const bf16_t* vp = v + ((size_t)b * T * Hv + hv) * Dv + row;
+    bf16_t* yp = y + ((size_t)b * T * Hv + hv) * Dv + row;
+    const float* gp = g + (size_t)b * T * Hv + hv;
+    const bf16_t* bp = beta + (size_t)b * T * Hv + hv;
+    for (int t = 0; t < T; t++) {
+        const uint2 qa = reinterpret_cast<const uint2*>(qp)[c], qb = reinterpret_cast<const uint2*>(qp)[16 + c];
+        const uint2 ka = reinterpret_cast<const uint2*>(kp)[c], kb = reinterpret_cast<const uint2*>(kp)[16 + c];
+        const float q8[8] = {lo_bf(qa.x), hi_bf(qa.x), lo_bf(qa.y), hi_bf(qa.y), lo_bf(qb.x), hi_bf(qb.x), lo_bf(qb.y), hi_bf(qb.y)};
+        const float k8[8] = {lo_bf(ka.x), hi_bf(ka.x), lo_bf(ka.y), hi_bf(ka.y), lo_bf(kb.x), hi_bf(kb.x), lo_bf(kb.y), hi_bf(kb.y)};
+        const float kq = dot8_row16(k8, q8);
+        const float yv = gdn_row_step(sv, k8, q8, bf2f(*vp), *gp, bf2f(*bp), kq);
+        if (c == 0) *yp = f2bf(yv);
+        qp += (size_t)Hk * DK;
+        kp += (size_t)Hk * DK;
+        vp += (size_t)Hv * Dv;
+        yp += (size_t)Hv * Dv;
+        gp += Hv;
+        bp += Hv;
+    }
+    reinterpret_cast<float4*>(st_out + so)[c] = make_float4(sv[0], sv[1], sv[2], sv[3]);
+    reinterpret_cast<float4*>(st_out + so)[16 + c] = make_float4(sv[4], sv[5], sv[6], sv[7]);
+}
+
+inline bool al(const void* p, unsigned a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+int qt_gdn_gates(const void* a, const void* b, long a_stride, long b_stride, const float* A_log, const float* dt_bias,
+                 float* g, float* log_g, void* beta, long rows, int hv, hipStream_t stream) {
+    if (!a || !A_log || !dt_bias || (beta && !b)) return QT_ERR_NULL;
+    if (rows < 0 || hv <= 0) return QT_ERR_DIM;
+    if (rows == 0) return QT_OK;
+    const long n = rows * hv;
+    hipLaunchKernelGGL(gates_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, (const bf16_t*)a, (const bf16_t*)b,
+                       a_stride, b_stride, A_log, dt_bias, g, log_g, (bf16_t*)beta, rows, hv);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_normalize_qk(const void* q, const void* k, void* q_out, void* k_out, long rows, int dk, hipStream_t stream) {
+    if (!q || !k || !q_out || !k_out) return QT_ERR_NULL;
+    if (dk != DK) return QT_ERR_UNSUPPORTED;
+    if (rows < 0) return QT_ERR_DIM;
+    if (rows == 0) return QT_OK;
+    if (!al(q, 4) || !al(k, 4) || !al(q_out, 4) || !al(k_out, 4)) return QT_ERR_ALIGN;
+    hipLaunchKernelGGL(normalize_qk_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, (const bf16_t*)q,
+                       (const bf16_t*)k, (bf16_t*)q_out, (bf16_t*)k_out, rows);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_gdn_conv_prep(const void* proj, const void* conv_state, const void* conv_w, void* q, void* k, void* v, int S,
+                     hipStream_t stream) {
+    if (!proj || !conv_state || !conv_w || !q || !k || !v) return QT_ERR_NULL;
+    if (S < 0) return QT_ERR_DIM;
+    if (S == 0) return QT_OK;
+    if (!al(conv_w, 8)) return QT_ERR_ALIGN;
+    hipLaunchKernelGGL(conv_prep_kernel, dim3((unsigned)S * HV), dim3(128), 0, stream, (const bf16_t*)proj,
+                       (const bf16_t*)conv_state, (const bf16_t*)conv_w, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, S);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_gated_rmsnorm(const void* y, const void* proj, const float* gw, void* out, long rows, float eps, hipStream_t stream) {
+    if (!y || !proj || !gw || !out) return QT_ERR_NULL;
+    if (rows < 0) return QT_ERR_DIM;
+    if (rows == 0) return QT_OK;
+    if (!al(y, 16) || !al(proj, 16) || !al(out, 16)) return QT_ERR_ALIGN;
+    hipLaunchKernelGGL(gated_norm_kernel, dim3((unsigned)rows), dim3(256), 0, stream, (const bf16_t*)y, (const bf16_t*)proj, gw,
+                       (bf16_t*)out, rows, eps);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_gdn_recurrent(const void* q, const void* k, const void* v, const float* g, const void* beta, const float* state_in,
+                     float* state_out, void* y, int B, int T, int Hk, int Hv, int Dk, int Dv, hipStream_t stream) {
+    if (!q || !k || !v || !g || !beta || !state_in || !state_out || !y) return QT_ERR_NULL;
+    if (Dk != DK || Dv <= 0 || Dv % 16 || Hk <= 0 || Hv <= 0 || Hv % Hk) return QT_ERR_UNSUPPORTED;   // gated_delta.py:164-166
+    if (B < 0 || T < 0) return QT_ERR_DIM;
+    if (B == 0) return QT_OK;
+    if (!al(q, 8) || !al(k, 8) || !al(state_in, 16) || !al(state_out, 16)) return QT_ERR_ALIGN;
+    hipLaunchKernelGGL(recurrent_kernel, dim3((unsigned)(B * Hv * (Dv / 16))), dim3(256), 0, stream, (const bf16_t*)q,
+                       (const bf16_t*)k, (const bf16_t*)v, g, (const bf16_t*)beta, state_in, state_out, (bf16_t*)y, T, Hk, Hv, Dv);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+}  // extern "C"

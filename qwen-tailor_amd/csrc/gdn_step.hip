@@ -1,0 +1,289 @@
+// Fused GatedDeltaNet decode / speculative-verify step for gfx950.
+//
+// One workgroup (256 threads = 4 wavefronts of 64) owns ROWS = RS*16 value rows of one (sequence, head) and streams them
+// HBM -> registers -> HBM exactly once: conv4 + SiLU, q/k L2 norm, gates, then for every value row r
+//     s = S[r,:] * g;  kv = s.k;  delta = (v_r - kv) * beta;  s += k * delta;  y_r = s.q
+// (qwen35/kernels.py:518-530).  Replaces the Metal kernels deltanet_b (qwen35/batch.py:36-135), deltanet_bm
+// (qwen35/batch_spec.py:45-150) and deltanet_m{M} (qwen35/kernels.py:461-567).
+//
+// Memory layout (slot-major, as qwen35/batch.py:1-12): ssm pool [S+1][16][128][128] f32, one head = 64 KiB contiguous;
+// a 16-lane group reads 256 contiguous bytes of a row per load, a wavefront 4 rows, the workgroup 16 rows = 8 KiB per
+// load slot.  Both dot products of a row are taken from the state as loaded,
+//     kv = g * (S_r . k),   y_r = g * (S_r . q) + delta * (k . q),
+// so the two 16-lane DPP reductions of a row are independent and the row is touched once.
+#include "qt_common.h"
+
+using namespace qt;
+
+namespace {
+
+struct RawIn {          // the un-convolved inputs one prologue thread needs for one token
+    float w0, w1, w2, x;
+    uint2 c;
+};
+
+// input row t of channel ch for the chained tokens of one sequence: t < 0 reads the stored window (kernels.py:477-479)
+__device__ __forceinline__ float inp(const bf16_t* __restrict__ cs_in, const bf16_t* __restrict__ proj, int t, int ch) {
+    return t < 0 ? bf2f(cs_in[(t + 3) * CD + ch]) : bf2f(proj[(size_t)t * PW + ch]);
+}
+__device__ __forceinline__ RawIn load_raw(const bf16_t* __restrict__ cs_in, const bf16_t* __restrict__ proj,
+                                          const bf16_t* __restrict__ cw, int j, int ch) {
+    RawIn r;
+    r.w0 = inp(cs_in, proj, j - 3, ch);
+    r.w1 = inp(cs_in, proj, j - 2, ch);
+    r.w2 = inp(cs_in, proj, j - 1, ch);
+    r.x = inp(cs_in, proj, j, ch);
+    r.c = *reinterpret_cast<const uint2*>(cw + (size_t)ch * 4);
+    return r;
+}
+__device__ __forceinline__ void store_window(bf16_t* __restrict__ cs_out, const RawIn& r, int ch) {
+    cs_out[ch] = f2bf(r.w1);            // kernels.py:531: the new window is the last three input rows
+    cs_out[CD + ch] = f2bf(r.w2);
+    cs_out[2 * CD + ch] = f2bf(r.x);
+}
+
+// M chained tokens of one (sequence, head, row split).  Snapshot j of the state goes to st_out + j*st_stride and of the
+// conv window to cs_out + j*cs_stride (strides 0 = update in place).
+template <int RS>
+__device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs_in,
+                                           bf16_t* __restrict__ cs_out, size_t cs_stride,
+                                           const bf16_t* __restrict__ cw, const float* __restrict__ A_log,
+                                           const float* __restrict__ dt_bias, const float* st_in,
+                                           float* st_out, size_t st_stride, bf16_t* __restrict__ y, int M, int h,
+                                           int split) {
+    constexpr int ROWS = RS * 16;
+    __shared__ double red[4];
+    __shared__ __align__(16) float qk_s[2][DK];
+    __shared__ float v_s[ROWS];
+    __shared__ float gb_s[2];
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, grp = lane >> 4, c = lane & 15;
+    const int row0 = split * ROWS;
+    const int which = tid >> 7;                                  // 0: a q channel, 1: a k channel
+    const int ch_qk = which * KD + h * DK + (tid & 127);
+    const bool has_v = tid < ROWS;
+    const int ch_v = 2 * KD + h * DV + row0 + tid;
+    const bool gate_thread = tid == 192;
+
+    // ---- token 0's prologue inputs first, then the state: the prologue runs while the state is in flight
+    RawIn rq = load_raw(cs_in, proj, cw, 0, ch_qk);
+    RawIn rv;
+    if (has_v) rv = load_raw(cs_in, proj, cw, 0, ch_v);
+    float ga = 0.f, gbv = 0.f, gA = 0.f, gdt = 0.f;
+    if (gate_thread) {
+        ga = bf2f(proj[CD + KD + HV + h]);
+        gbv = bf2f(proj[CD + KD + h]);
+        gA = A_log[h];
+        gdt = dt_bias[h];
+    }
+
+    float4 s[RS][2];
+    {
+        const float4* sin4 = reinterpret_cast<const float4*>(st_in + ((size_t)h * DV + row0) * DK);
+#pragma unroll
+        for (int i = 0; i < RS; i++) {
+            const int row = i * 16 + w * 4 + grp;
+            s[i][0] = sin4[row * (DK / 4) + c];
+            s[i][1] = sin4[row * (DK / 4) + 16 + c];
+        }
+    }
+
+    const float sc = which == 0 ? BF(INV_SCALE * INV_SCALE) : BF(INV_SCALE);       // kernels.py:492
+    for (int j = 0; j < M; j++) {
+        if (j > 0) {
+            rq = load_raw(cs_in, proj, cw, j, ch_qk);
+            if (has_v) rv = load_raw(cs_in, proj, cw, j, ch_v);
+            if (gate_thread) {
+                ga = bf2f(proj[(size_t)j * PW + CD + KD + HV + h]);
+                gbv = bf2f(proj[(size_t)j * PW + CD + KD + h]);
+            }
+        }
+        bf16_t* cso = cs_out + (size_t)j * cs_stride;
+        // conv + silu, exact sum of squares over the head's 128 q (waves 0,1) / k (waves 2,3) channels
+        const float u = conv_silu(rq.w0, rq.w1, rq.w2, rq.x, rq.c);
+        const double tot = wave_sum_d((double)u * (double)u);
+        if (lane == 0) red[w] = tot;
+        if (split == 0) store_window(cso, rq, ch_qk);
+        float vv = 0.f;
+        if (has_v) {
+            vv = conv_silu(rv.w0, rv.w1, rv.w2, rv.x, rv.c);
+            store_window(cso, rv, ch_v);
+        }
+        float g = 0.f, beta = 0.f;
+        if (gate_thread) {                                                       // kernels.py:511-515
+            const float av = BF(ga + gdt);
+            g = exp32(-exp32(gA) * softplus_bf16(av));
+            beta = sigmoid_bf16(gbv);
+        }
+        __syncthreads();
+        {
+            const float ss = (float)(red[which * 2] + red[which * 2 + 1]);
+            const float r = rsqrt_rn(ss / (float)DK + qk_eps());
+            qk_s[which][tid & 127] = BF(BF(u * r) * sc);                         // kernels.py:507-510
+            if (has_v) v_s[tid] = vv;
+            if (gate_thread) {
+                gb_s[0] = g;
+                gb_s[1] = beta;
+            }
+        }
+        __syncthreads();
+
+        // ---- the recurrence over this thread's 8 columns of RS rows
+        float q8[8], k8[8];
+        {
+            const float4 a = reinterpret_cast<const float4*>(qk_s[0])[c], b = reinterpret_cast<const float4*>(qk_s[0])[16 + c];
+            const float4 d = reinterpret_cast<const float4*>(qk_s[1])[c], e = reinterpret_cast<const float4*>(qk_s[1])[16 + c];
+            q8[0] = a.x; q8[1] = a.y; q8[2] = a.z; q8[3] = a.w; q8[4] = b.x; q8[5] = b.y; q8[6] = b.z; q8[7] = b.w;
+            k8[0] = d.x; k8[1] = d.y; k8[2] = d.z; k8[3] = d.w; k8[4] = e.x; k8[5] = e.y; k8[6] = e.z; k8[7] = e.w;
+        }
+        const float gg = gb_s[0], bb = gb_s[1];
+        const float kq = dot8_row16(k8, q8);
+
+        float4* so4 = reinterpret_cast<float4*>(st_out + (size_t)j * st_stride + ((size_t)h * DV + row0) * DK);
+        bf16_t* yo = y + (size_t)j * KD + h * DV + row0;
+#pragma unroll
+        for (int i = 0; i < RS; i++) {
+            const int row = i * 16 + w * 4 + grp;
+            float sv[8] = {s[i][0].x, s[i][0].y, s[i][0].z, s[i][0].w, s[i][1].x, s[i][1].y, s[i][1].z, s[i][1].w};
+            const float yv = gdn_row_step(sv, k8, q8, v_s[row], gg, bb, kq);
+            s[i][0] = make_float4(sv[0], sv[1], sv[2], sv[3]);
+            s[i][1] = make_float4(sv[4], sv[5], sv[6], sv[7]);
+            so4[row * (DK / 4) + c] = s[i][0];
+            so4[row * (DK / 4) + 16 + c] = s[i][1];
+            if (c == 0) yo[row] = f2bf(yv);
+        }
+    }
+}
+
+template <int RS>
+__device__ __forceinline__ void split_id(int& b, int& h, int& split) {
+    constexpr int NSPLIT = 8 / RS;
+    const unsigned id = xcd_remap(blockIdx.x, gridDim.x);
+    b = id / (HV * NSPLIT);
+    const unsigned rem = id % (HV * NSPLIT);
+    h = rem / NSPLIT;
+    split = rem % NSPLIT;
+}
+
+// batch.deltanet_b (qwen35/batch.py:128-135): one token per row, pools updated in place
+template <int RS>
+__global__ __launch_bounds__(256) void gdn_decode_kernel(const bf16_t* __restrict__ proj, bf16_t* conv_pool,
+                                                         const bf16_t* __restrict__ cw, const float* __restrict__ A_log,
+                                                         const float* __restrict__ dt_bias, float* ssm_pool,
+                                                         const int* __restrict__ slots, const int* __restrict__ pos,
+                                                         bf16_t* __restrict__ y, int n_slots) {
+    int b, h, split;
+    split_id<RS>(b, h, split);
+    const int slot = slots[b];
+    if ((unsigned)slot >= (unsigned)n_slots) return;             // never touch memory outside the pools
+    const int par = pos[b] & 1;                                  // batch.py:49-52: read buffer pos&1, write the other
+    float* st = ssm_pool + (size_t)slot * HV * DV * DK;
+    gdn_tokens<RS>(proj + (size_t)b * PW, conv_pool + (size_t)(slot * 2 + par) * 3 * CD,
+                   conv_pool + (size_t)(slot * 2 + (par ^ 1)) * 3 * CD, 0, cw, A_log, dt_bias, st, st, 0,
+                   y + (size_t)b * KD, 1, h, split);
+}
+
+// batch_spec.deltanet_bm (qwen35/batch_spec.py:142-150): M chained tokens per sequence, snapshot pools in place
+template <int RS>
+__global__ __launch_bounds__(256) void gdn_verify_kernel(const bf16_t* __restrict__ proj, bf16_t* conv_pool,
+                                                         const bf16_t* __restrict__ cw, const float* __restrict__ A_log,
+                                                         const float* __restrict__ dt_bias, float* ssm_pool,
+                                                         const int* __restrict__ sslots, const int* __restrict__ sels,
+                                                         const int* __restrict__ pars, bf16_t* __restrict__ y, int M,
+                                                         int n_entries) {
+    int b, h, split;
+    split_id<RS>(b, h, split);
+    const int ss = sslots[b], sl = sels[b];
+    if ((unsigned)ss >= (unsigned)n_entries || (unsigned)sl >= (unsigned)M) return;
+    const int par = pars[b] & 1;
+    const size_t hs = (size_t)HV * DV * DK;
+    gdn_tokens<RS>(proj + (size_t)b * M * PW, conv_pool + ((size_t)(ss * 2 + par) * M + sl) * 3 * CD,
+                   conv_pool + (size_t)(ss * 2 + (par ^ 1)) * M * 3 * CD, (size_t)3 * CD, cw, A_log, dt_bias,
+                   ssm_pool + ((size_t)ss * M + sl) * hs, ssm_pool + (size_t)ss * M * hs, hs, y + (size_t)b * M * KD, M,
+                   h, split);
+}
+
+// kernels.deltanet (qwen35/kernels.py:555-567): one sequence, starts from snapshot sel[0], writes M fresh snapshots
+template <int RS>
+__global__ __launch_bounds__(256) void gdn_solo_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs_snap,
+                                                       const bf16_t* __restrict__ cw, const float* __restrict__ A_log,
+                                                       const float* __restrict__ dt_bias, const float* __restrict__ st_snap,
+                                                       const int* __restrict__ sel, bf16_t* __restrict__ y,
+                                                       bf16_t* __restrict__ cs_out, float* __restrict__ st_out, int M,
+                                                       int n_snap) {
+    int b, h, split;
+    split_id<RS>(b, h, split);
+    const int sl = sel[0];
+    if ((unsigned)sl >= (unsigned)n_snap) return;
+    const size_t hs = (size_t)HV * DV * DK;
+    gdn_tokens<RS>(proj, cs_snap + (size_t)sl * 3 * CD, cs_out, (size_t)3 * CD, cw, A_log, dt_bias, st_snap + sl * hs,
+                   st_out, hs, y, M, h, split);
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// rows per workgroup: few sequences -> split a head over more workgroups so the chip still fills
+inline int pick_rs(int nseq, int rows_split) {
+    if (rows_split == 128 || rows_split == 64 || rows_split == 32 || rows_split == 16) return rows_split / 16;
+    if (nseq >= 32) return 8;
+    if (nseq >= 8) return 4;
+    if (nseq >= 4) return 2;
+    return 1;
+}
+
+}  // namespace
+
+#define QT_DISPATCH_RS(rs, KERNEL, nseq, stream, ...)                                                  \
+    switch (rs) {                                                                                       \
+        case 8: hipLaunchKernelGGL(KERNEL<8>, dim3((nseq) * HV * 1), dim3(256), 0, stream, __VA_ARGS__); break; \
+        case 4: hipLaunchKernelGGL(KERNEL<4>, dim3((nseq) * HV * 2), dim3(256), 0, stream, __VA_ARGS__); break; \
+        case 2: hipLaunchKernelGGL(KERNEL<2>, dim3((nseq) * HV * 4), dim3(256), 0, stream, __VA_ARGS__); break; \
+        default: hipLaunchKernelGGL(KERNEL<1>, dim3((nseq) * HV * 8), dim3(256), 0, stream, __VA_ARGS__); break; \
+    }
+
+extern "C" {
+
+int qt_gdn_decode_step(const void* proj, void* conv_pool, const void* conv_w, const float* A_log, const float* dt_bias,
+                       float* ssm_pool, const int32_t* slots, const int32_t* pos, void* y, int B, int n_slots,
+                       int rows_per_wg, hipStream_t stream) {
+    if (!proj || !conv_pool || !conv_w || !A_log || !dt_bias || !ssm_pool || !slots || !pos || !y) return QT_ERR_NULL;
+    if (B < 0 || n_slots <= 0) return QT_ERR_DIM;
+    if (B == 0) return QT_OK;
+    if (!aligned16(ssm_pool) || (reinterpret_cast<uintptr_t>(conv_w) & 7u)) return QT_ERR_ALIGN;
+    const int rs = pick_rs(B, rows_per_wg);
+    QT_DISPATCH_RS(rs, gdn_decode_kernel, B, stream, (const bf16_t*)proj, (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log,
+                   dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_gdn_verify_step(const void* proj, void* conv_pool, const void* conv_w, const float* A_log, const float* dt_bias,
+                       float* ssm_pool, const int32_t* sslots, const int32_t* sels, const int32_t* pars, void* y, int B,
+                       int M, int n_entries, int rows_per_wg, hipStream_t stream) {
+    if (!proj || !conv_pool || !conv_w || !A_log || !dt_bias || !ssm_pool || !sslots || !sels || !pars || !y) return QT_ERR_NULL;
+    if (B < 0 || n_entries <= 0) return QT_ERR_DIM;
+    if (M < 1 || M > 16) return QT_ERR_UNSUPPORTED;
+    if (B == 0) return QT_OK;
+    if (!aligned16(ssm_pool) || (reinterpret_cast<uintptr_t>(conv_w) & 7u)) return QT_ERR_ALIGN;
+    const int rs = pick_rs(B, rows_per_wg);
+    QT_DISPATCH_RS(rs, gdn_verify_kernel, B, stream, (const bf16_t*)proj, (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log,
+                   dt_bias, ssm_pool, sslots, sels, pars, (bf16_t*)y, M, n_entries);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_gdn_deltanet(const void* proj, const void* conv_snap, const void* conv_w, const float* A_log, const float* dt_bias,
+                    const float* ssm_snap, const int32_t* sel, void* y, void* cs_out, float* st_out, int M, int n_snap,
+                    int rows_per_wg, hipStream_t stream) {
+    if (!proj || !conv_snap || !conv_w || !A_log || !dt_bias || !ssm_snap || !sel || !y || !cs_out || !st_out) return QT_ERR_NULL;
+    if (n_snap <= 0) return QT_ERR_DIM;
+    if (M < 1 || M > 16) return QT_ERR_UNSUPPORTED;
+    if (!aligned16(ssm_snap) || !aligned16(st_out) || (reinterpret_cast<uintptr_t>(conv_w) & 7u)) return QT_ERR_ALIGN;
+    const int rs = pick_rs(1, rows_per_wg);
+    QT_DISPATCH_RS(rs, gdn_solo_kernel, 1, stream, (const bf16_t*)proj, (const bf16_t*)conv_snap, (const bf16_t*)conv_w, A_log,
+                   dt_bias, ssm_snap, sel, (bf16_t*)y, (bf16_t*)cs_out, st_out, M, n_snap);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,160 @@
+// Device helpers shared by every kernel of the GatedDeltaNet / GQA-hd256 hot path (gfx950 only).
+//
+// Arithmetic contract of the elementwise prologue (conv + SiLU, q/k norm, gates, gated RMSNorm).  It keeps the
+// reference's bf16 rounding points (qwen35/mslib.py:7-27, qwen35/kernels.py:476-515) and fixes the last-place
+// behaviour so that a CPU restatement reproduces every bf16 value bit for bit:
+//   exp32 / log32 : double-precision libm result rounded to float
+//   sum of squares: exact (double), rounded to float once
+//   rsqrt         : 1 / sqrt evaluated in double precision and rounded to float once
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace qt {
+
+constexpr int HV = 16, DK = 128, DV = 128, KD = 2048, CD = 6144, PW = 8224;   // qwen35/batch.py:29
+constexpr int AH = 8, AKV = 2, AD = 256;                                        // qwen35/model.py:43-45
+
+typedef uint16_t bf16_t;   // raw bf16 bits
+
+__device__ __forceinline__ float bf2f(bf16_t b) { return __uint_as_float((uint32_t)b << 16); }
+
+__device__ __forceinline__ bf16_t f2bf(float f) {   // round to nearest even; NaN stays NaN
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float BF(float f) { return bf2f(f2bf(f)); }          // `#define BF(v)`, mslib.py:8-10
+
+__device__ __forceinline__ float lo_bf(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float hi_bf(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ uint32_t pack_bf(float a, float b) { return (uint32_t)f2bf(a) | ((uint32_t)f2bf(b) << 16); }
+
+__device__ __forceinline__ float exp32(float x) { return (float)exp((double)x); }
+__device__ __forceinline__ float log32(float x) { return (float)log((double)x); }
+__device__ __forceinline__ float rsqrt_rn(float x) { return (float)(1.0 / sqrt((double)x)); }   // correctly rounded 1/sqrt
+
+__device__ __forceinline__ float log1p_mx(float x) {                             // mslib.py:11-15
+    float xp1 = 1.0f + x;
+    if (xp1 == 1.0f) return x;
+    return x * __fdiv_rn(log32(xp1), xp1 - 1.0f);
+}
+__device__ __forceinline__ float sigmoid_bf16(float x) {                         // mslib.py:16-20
+    float y = BF(__fdiv_rn(1.0f, BF(1.0f + BF(exp32(fabsf(x))))));
+    return x < 0.0f ? y : BF(1.0f - y);
+}
+__device__ __forceinline__ float silu_bf16(float x) { return BF(x * sigmoid_bf16(x)); }   // mslib.py:21-22
+__device__ __forceinline__ float softplus_bf16(float x) {                        // mslib.py:23-26
+    return BF(fmaxf(x, 0.0f) + BF(log1p_mx(BF(exp32(-fabsf(x))))));
+}
+
+// 4-tap depthwise conv + SiLU of one channel (kernels.py:480-484): w0..w2 = the three previous input rows (oldest
+// first), x = the current row, c = the channel's four taps (tap 3 multiplies the current token).
+__device__ __forceinline__ float conv_silu(float w0, float w1, float w2, float x, uint2 c) {
+    float s = w0 * lo_bf(c.x);
+    s = s + w1 * hi_bf(c.x);
+    s = s + w2 * lo_bf(c.y);
+    s = s + x * hi_bf(c.y);
+    return silu_bf16(BF(s));
+}
+
+constexpr float INV_SCALE = 0.08838834764831845f;                                // 128^-0.5, kernels.py:490
+__device__ __forceinline__ float qk_eps() { return __fmul_rn(__fmul_rn(1e-6f, INV_SCALE), INV_SCALE); }   // kernels.py:491
+
+// ---- cross-lane sums over an aligned group of 16 lanes (one DPP row); every lane of the group gets the total ----
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_mov<0xB1>(v);     // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);     // quad_perm [2,3,0,1]
+    v += dpp_mov<0x141>(v);    // row_half_mirror
+    v += dpp_mov<0x140>(v);    // row_mirror
+    return v;
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_mov_d(double v) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, 0xF, 0xF, true);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, 0xF, 0xF, true);
+    return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double row16_sum_d(double v) {
+    v += dpp_mov_d<0xB1>(v);
+    v += dpp_mov_d<0x4E>(v);
+    v += dpp_mov_d<0x141>(v);
+    v += dpp_mov_d<0x140>(v);
+    return v;
+}
+// total over the whole 64-lane wavefront (every lane gets it)
+__device__ __forceinline__ double wave_sum_d(double v) {
+    v = row16_sum_d(v);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_mov<0xB1>(v));
+    v = fmaxf(v, dpp_mov<0x4E>(v));
+    v = fmaxf(v, dpp_mov<0x141>(v));
+    v = fmaxf(v, dpp_mov<0x140>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+
+// One value row of the gated delta rule, this lane's 8 of the 128 columns (kernels.py:518-530):
+//   kv = g (S_r . k);  delta = (v - kv) beta;  y = g (S_r . q) + delta (k . q);  S_r <- g S_r + delta k
+// pk / pq are reduced over the 16 lanes that share the row; kq = k . q (already reduced).  Returns y.
+__device__ __forceinline__ float gdn_row_step(float (&sv)[8], const float (&k8)[8], const float (&q8)[8], float v, float g,
+                                              float beta, float kq) {
+    float pk = 0.f, pq = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        pk = fmaf(sv[e], k8[e], pk);
+        pq = fmaf(sv[e], q8[e], pq);
+    }
+    pk = row16_sum(pk);
+    pq = row16_sum(pq);
+    const float delta = (v - g * pk) * beta;
+    const float yv = fmaf(g, pq, delta * kq);
+#pragma unroll
+    for (int e = 0; e < 8; e++) sv[e] = fmaf(delta, k8[e], g * sv[e]);
+    return yv;
+}
+__device__ __forceinline__ float dot8_row16(const float (&a)[8], const float (&b)[8]) {
+    float t = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) t = fmaf(a[e], b[e], t);
+    return row16_sum(t);
+}
+
+// workgroup id remapped so that consecutive logical ids share an XCD (8 XCDs, hardware deals workgroups round-robin)
+__device__ __forceinline__ unsigned xcd_remap(unsigned id, unsigned n) {
+    return (n % 8u == 0u) ? (id % 8u) * (n / 8u) + id / 8u : id;
+}
+
+}  // namespace qt
+
+// error codes of the C ABI
+#define QT_OK 0
+#define QT_ERR_DIM (-1)
+#define QT_ERR_ALIGN (-2)
+#define QT_ERR_NULL (-3)
+#define QT_ERR_UNSUPPORTED (-4)
+#define QT_ERR_LAUNCH (-5)
+
+#define QT_CHECK_LAUNCH()                                   \
+    do {                                                    \
+        hipError_t e_ = hipGetLastError();                  \
+        if (e_ != hipSuccess) return QT_ERR_LAUNCH;         \
+    } while (0)
