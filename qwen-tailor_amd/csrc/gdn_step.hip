@@ -17,6 +17,8 @@ using namespace qt;
 
 namespace {
 
+typedef float f4 __attribute__((ext_vector_type(4)));   // native vector: nontemporal loads / stores take it
+
 struct RawIn {          // the un-convolved inputs one prologue thread needs for one token
     float w0, w1, w2, x;
     uint2 c;
@@ -63,40 +65,37 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
     const int ch_qk = which * KD + h * DK + (tid & 127);
     const bool has_v = tid < ROWS;
     const int ch_v = 2 * KD + h * DV + row0 + tid;
-    const bool gate_thread = tid == 192;
 
-    // ---- token 0's prologue inputs first, then the state: the prologue runs while the state is in flight
+    // ---- token 0's prologue inputs first, then the state: the prologue runs while the state is in flight.  Every load
+    // below is unconditional (threads without a v channel re-read their q/k channel) so that nothing has to be waited
+    // for before the state loads are issued.
+    const int ch_v_ld = has_v ? ch_v : ch_qk;
     RawIn rq = load_raw(cs_in, proj, cw, 0, ch_qk);
-    RawIn rv;
-    if (has_v) rv = load_raw(cs_in, proj, cw, 0, ch_v);
-    float ga = 0.f, gbv = 0.f, gA = 0.f, gdt = 0.f;
-    if (gate_thread) {
-        ga = bf2f(proj[CD + KD + HV + h]);
-        gbv = bf2f(proj[CD + KD + h]);
-        gA = A_log[h];
-        gdt = dt_bias[h];
-    }
+    RawIn rv = load_raw(cs_in, proj, cw, 0, ch_v_ld);
+    // gates: lane 0 of wave 3 evaluates exp(A_log), lane 1 the softplus, lane 2 the sigmoid (one exp pass for all three)
+    const int gl = lane < 3 ? lane : 0;
+    float gx = bf2f(proj[CD + KD + HV * (gl == 1 ? 1 : 0) + h]);       // lane 1: a;  lanes 0, 2: b
+    const float gA = A_log[h], gdt = dt_bias[h];
+    __builtin_amdgcn_sched_barrier(0);           // keep the small loads ahead of the state loads in issue order
 
-    float4 s[RS][2];
+    f4 s[RS][2];
     {
-        const float4* sin4 = reinterpret_cast<const float4*>(st_in + ((size_t)h * DV + row0) * DK);
+        const f4* sin4 = reinterpret_cast<const f4*>(st_in + ((size_t)h * DV + row0) * DK);
 #pragma unroll
         for (int i = 0; i < RS; i++) {
             const int row = i * 16 + w * 4 + grp;
-            s[i][0] = sin4[row * (DK / 4) + c];
-            s[i][1] = sin4[row * (DK / 4) + 16 + c];
+            s[i][0] = __builtin_nontemporal_load(sin4 + row * (DK / 4) + c);
+            s[i][1] = __builtin_nontemporal_load(sin4 + row * (DK / 4) + 16 + c);
         }
     }
+    __builtin_amdgcn_sched_barrier(0);
 
     const float sc = which == 0 ? BF(INV_SCALE * INV_SCALE) : BF(INV_SCALE);       // kernels.py:492
     for (int j = 0; j < M; j++) {
         if (j > 0) {
             rq = load_raw(cs_in, proj, cw, j, ch_qk);
-            if (has_v) rv = load_raw(cs_in, proj, cw, j, ch_v);
-            if (gate_thread) {
-                ga = bf2f(proj[(size_t)j * PW + CD + KD + HV + h]);
-                gbv = bf2f(proj[(size_t)j * PW + CD + KD + h]);
-            }
+            rv = load_raw(cs_in, proj, cw, j, ch_v_ld);
+            gx = bf2f(proj[(size_t)j * PW + CD + KD + HV * (gl == 1 ? 1 : 0) + h]);
         }
         bf16_t* cso = cs_out + (size_t)j * cs_stride;
         // conv + silu, exact sum of squares over the head's 128 q (waves 0,1) / k (waves 2,3) channels
@@ -110,10 +109,14 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
             store_window(cso, rv, ch_v);
         }
         float g = 0.f, beta = 0.f;
-        if (gate_thread) {                                                       // kernels.py:511-515
-            const float av = BF(ga + gdt);
-            g = exp32(-exp32(gA) * softplus_bf16(av));
-            beta = sigmoid_bf16(gbv);
+        if (w == 3) {                                                            // kernels.py:511-515
+            const float av = BF(gx + gdt);                                       // meaningful on lane 1
+            const float ex = gl == 0 ? gA : (gl == 1 ? -fabsf(av) : fabsf(gx));
+            const float e = exp32(ex);                                           // lane 0: exp(A_log); 1: exp(-|av|); 2: exp(|b|)
+            const float sp = BF(fmaxf(av, 0.0f) + BF(log1p_mx(BF(e))));          // softplus_bf16(av) on lane 1
+            const float yb = BF(__fdiv_rn(1.0f, BF(1.0f + BF(e))));              // sigmoid_bf16(b) on lane 2
+            beta = __shfl(gx < 0.0f ? yb : BF(1.0f - yb), 2, 64);
+            g = exp32(-__shfl(e, 0, 64) * __shfl(sp, 1, 64));
         }
         __syncthreads();
         {
@@ -121,7 +124,7 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
             const float r = rsqrt_rn(ss / (float)DK + qk_eps());
             qk_s[which][tid & 127] = BF(BF(u * r) * sc);                         // kernels.py:507-510
             if (has_v) v_s[tid] = vv;
-            if (gate_thread) {
+            if (tid == 192) {
                 gb_s[0] = g;
                 gb_s[1] = beta;
             }
@@ -139,17 +142,17 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
         const float gg = gb_s[0], bb = gb_s[1];
         const float kq = dot8_row16(k8, q8);
 
-        float4* so4 = reinterpret_cast<float4*>(st_out + (size_t)j * st_stride + ((size_t)h * DV + row0) * DK);
+        f4* so4 = reinterpret_cast<f4*>(st_out + (size_t)j * st_stride + ((size_t)h * DV + row0) * DK);
         bf16_t* yo = y + (size_t)j * KD + h * DV + row0;
 #pragma unroll
         for (int i = 0; i < RS; i++) {
             const int row = i * 16 + w * 4 + grp;
             float sv[8] = {s[i][0].x, s[i][0].y, s[i][0].z, s[i][0].w, s[i][1].x, s[i][1].y, s[i][1].z, s[i][1].w};
             const float yv = gdn_row_step(sv, k8, q8, v_s[row], gg, bb, kq);
-            s[i][0] = make_float4(sv[0], sv[1], sv[2], sv[3]);
-            s[i][1] = make_float4(sv[4], sv[5], sv[6], sv[7]);
-            so4[row * (DK / 4) + c] = s[i][0];
-            so4[row * (DK / 4) + 16 + c] = s[i][1];
+            s[i][0] = f4{sv[0], sv[1], sv[2], sv[3]};
+            s[i][1] = f4{sv[4], sv[5], sv[6], sv[7]};
+            __builtin_nontemporal_store(s[i][0], so4 + row * (DK / 4) + c);
+            __builtin_nontemporal_store(s[i][1], so4 + row * (DK / 4) + 16 + c);
             if (c == 0) yo[row] = f2bf(yv);
         }
     }
