@@ -17,8 +17,8 @@ __global__ __launch_bounds__(256) void gates_kernel(const bf16_t* __restrict__ a
     const long r = i / hv;
     const int h = (int)(i % hv);
     const float av = BF(bf2f(a[r * a_stride + h]) + dt_bias[h]);
-    const float l = -exp32(A_log[h]) * softplus_bf16(av);
-    if (g) g[i] = exp32(l);
+    const float l = log_decay(A_log[h], av);
+    if (g) g[i] = expf(l);
     if (lg) lg[i] = l;
     if (beta) beta[i] = f2bf(sigmoid_bf16(bf2f(b[r * b_stride + h])));
 }
@@ -96,14 +96,12 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(const bf16_t* __restric
         ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
     }
     const float inv = rsqrt_rn((float)row16_sum_d(ss) / 128.f + eps);
-    float o[8];
+    uint32_t o[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-        const float n = gw[c * 8 + j] * (yy[j] * inv);
-        const float sig = __fdiv_rn(zz[j], 1.0f + exp32(-zz[j]));
-        o[j] = sig * n;
+        o[j] = gated_out(zz[j], gw[c * 8 + j] * (yy[j] * inv));
     }
-    uint4 ov = make_uint4(pack_bf(o[0], o[1]), pack_bf(o[2], o[3]), pack_bf(o[4], o[5]), pack_bf(o[6], o[7]));
+    uint4 ov = make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
     reinterpret_cast<uint4*>(out + row * KD + h * DV)[c] = ov;
 }
 

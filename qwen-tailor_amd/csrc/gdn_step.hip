@@ -72,7 +72,7 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
     const int ch_v_ld = has_v ? ch_v : ch_qk;
     RawIn rq = load_raw(cs_in, proj, cw, 0, ch_qk);
     RawIn rv = load_raw(cs_in, proj, cw, 0, ch_v_ld);
-    // gates: lane 0 of wave 3 evaluates exp(A_log), lane 1 the softplus, lane 2 the sigmoid (one exp pass for all three)
+    // gates are evaluated by wave 3: lane 1 the decay gate (reads a), lane 2 beta (reads b)
     const int gl = lane < 3 ? lane : 0;
     float gx = bf2f(proj[CD + KD + HV * (gl == 1 ? 1 : 0) + h]);       // lane 1: a;  lanes 0, 2: b
     const float gA = A_log[h], gdt = dt_bias[h];
@@ -110,13 +110,9 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
         }
         float g = 0.f, beta = 0.f;
         if (w == 3) {                                                            // kernels.py:511-515
-            const float av = BF(gx + gdt);                                       // meaningful on lane 1
-            const float ex = gl == 0 ? gA : (gl == 1 ? -fabsf(av) : fabsf(gx));
-            const float e = exp32(ex);                                           // lane 0: exp(A_log); 1: exp(-|av|); 2: exp(|b|)
-            const float sp = BF(fmaxf(av, 0.0f) + BF(log1p_mx(BF(e))));          // softplus_bf16(av) on lane 1
-            const float yb = BF(__fdiv_rn(1.0f, BF(1.0f + BF(e))));              // sigmoid_bf16(b) on lane 2
-            beta = __shfl(gx < 0.0f ? yb : BF(1.0f - yb), 2, 64);
-            g = exp32(-__shfl(e, 0, 64) * __shfl(sp, 1, 64));
+            // lane 1: decay gate from a; lane 2: beta from b
+            g = __shfl(decay_gate(gA, BF(gx + gdt)), 1, 64);
+            beta = __shfl(sigmoid_bf16(gx), 2, 64);
         }
         __syncthreads();
         {

@@ -36,18 +36,54 @@ __device__ __forceinline__ float exp32(float x) { return (float)exp((double)x); 
 __device__ __forceinline__ float log32(float x) { return (float)log((double)x); }
 __device__ __forceinline__ float rsqrt_rn(float x) { return (float)(1.0 / sqrt((double)x)); }   // correctly rounded 1/sqrt
 
+// The bf16 -> bf16 helpers below must return the bits the contract defines (exp32 / log32 = correctly rounded), but the
+// double-precision libm calls are ~10x the work of the float ones.  A float result that is off by a few ulp rounds to the
+// same bf16 value unless it lies within those few ulp of a bf16 rounding boundary; only then is the slow path taken
+// (about one evaluation in 10^4).  The GPU tests compare all 65536 inputs of each helper with the CPU oracle.
+__device__ __forceinline__ bool near_bf16_tie(float v, uint32_t slack) {
+    const uint32_t lo = __float_as_uint(v) & 0xffffu;
+    return (lo - (0x8000u - slack)) <= 2u * slack;
+}
+__device__ __forceinline__ float bf_exp(float x) {                               // BF(exp32(x))
+    float e = expf(x);                                                           // <= 1 ulp
+    if (__builtin_expect(near_bf16_tie(e, 4) || fabsf(x) > 80.0f, 0)) e = exp32(x);
+    return BF(e);
+}
+__device__ __forceinline__ float bf_rcp(float d) {                               // BF(1 / d), IEEE divide
+    float r = __builtin_amdgcn_rcpf(d);                                          // <= 1 ulp
+    if (__builtin_expect(near_bf16_tie(r, 3) || !(fabsf(d) > 1e-30f && fabsf(d) < 1e30f), 0)) r = __fdiv_rn(1.0f, d);
+    return BF(r);
+}
+
 __device__ __forceinline__ float log1p_mx(float x) {                             // mslib.py:11-15
     float xp1 = 1.0f + x;
     if (xp1 == 1.0f) return x;
     return x * __fdiv_rn(log32(xp1), xp1 - 1.0f);
 }
+__device__ __forceinline__ float bf_log1p_mx(float x) {                          // BF(log1p_mx(x)) for x in [0, 1]
+    const float xp1 = 1.0f + x;
+    if (xp1 == 1.0f) return BF(x);
+    float r = x * __fdiv_rn(logf(xp1), xp1 - 1.0f);
+    if (__builtin_expect(near_bf16_tie(r, 6), 0)) r = log1p_mx(x);
+    return BF(r);
+}
 __device__ __forceinline__ float sigmoid_bf16(float x) {                         // mslib.py:16-20
-    float y = BF(__fdiv_rn(1.0f, BF(1.0f + BF(exp32(fabsf(x))))));
+    const float y = bf_rcp(BF(1.0f + bf_exp(fabsf(x))));
     return x < 0.0f ? y : BF(1.0f - y);
 }
 __device__ __forceinline__ float silu_bf16(float x) { return BF(x * sigmoid_bf16(x)); }   // mslib.py:21-22
 __device__ __forceinline__ float softplus_bf16(float x) {                        // mslib.py:23-26
-    return BF(fmaxf(x, 0.0f) + BF(log1p_mx(BF(exp32(-fabsf(x))))));
+    return BF(fmaxf(x, 0.0f) + bf_log1p_mx(bf_exp(-fabsf(x))));
+}
+// decay gate of one head: g = exp(-exp(A_log) * softplus_bf16(av)) (kernels.py:511-513).  The reference evaluates it with
+// float exp and does not round it; here both exps are float with <= 1 ulp error.
+__device__ __forceinline__ float log_decay(float A_log, float av) { return -expf(A_log) * softplus_bf16(av); }
+__device__ __forceinline__ float decay_gate(float A_log, float av) { return expf(log_decay(A_log, av)); }
+// z * sigmoid(z) * n rounded to bf16 once (kernels.py:134-137): z/(1+exp32(-z)) * n
+__device__ __forceinline__ bf16_t gated_out(float z, float n) {
+    float o = __fdiv_rn(z, 1.0f + expf(-z)) * n;
+    if (__builtin_expect(near_bf16_tie(o, 8) || fabsf(z) > 80.0f, 0)) o = __fdiv_rn(z, 1.0f + exp32(-z)) * n;
+    return f2bf(o);
 }
 
 // 4-tap depthwise conv + SiLU of one channel (kernels.py:480-484): w0..w2 = the three previous input rows (oldest
