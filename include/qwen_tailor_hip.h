@@ -1,0 +1,83 @@
+/* C ABI of libqwen_tailor_hip.so: the GatedDeltaNet + GQA head-dim-256 attention hot path of wang90063/Qwen-tailor
+ * on MI355X (gfx950).
+ *
+ * The reference has no FFI: its boundary is a set of Python functions over MLX arrays that launch Metal kernels
+ * (qwen35/gated_delta.py, kernels.py, batch.py, batch_spec.py, prefill.py, gdn_nax.py).  Each entry point below is what
+ * one of those functions binds to; the citation names the reference function it replaces.
+ *
+ * Conventions: every pointer is a device pointer unless said otherwise; bf16 tensors are passed as raw 16-bit words
+ * (const void*), state is float; tensors are contiguous in the layouts of the reference; index arrays are int32 on the
+ * device; `stream` is a hipStream_t (passed as void* so that this header needs no HIP include).  No entry point
+ * allocates, synchronises or keeps global state; all work is enqueued on `stream`.  Return value: 0 on success, or
+ *   -1 bad dimension, -2 misaligned pointer, -3 null pointer, -4 unsupported shape, -5 launch failure,
+ *   -6 workspace too small.
+ * Rows whose slot index lies outside the pool (or whose position would overflow it) are skipped by the kernels: nothing
+ * outside the caller's buffers is ever read or written.
+ */
+#ifndef QWEN_TAILOR_HIP_H
+#define QWEN_TAILOR_HIP_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* qt_stream_t; /* hipStream_t */
+
+/* batch.deltanet_b (qwen35/batch.py:128-135): one decode token for each of B rows.
+ * proj [B,8224] bf16; conv_pool [n_slots*2,3,6144] bf16 (reads buffer slot*2+(pos&1), writes the other one);
+ * conv_w [6144*4] bf16; A_log, dt_bias [16] f32; ssm_pool [n_slots,16,128,128] f32 (updated in place);
+ * slots, pos [B] int32; y [B,2048] bf16.  rows_per_wg: 0 = choose, else 16/32/64/128 value rows per workgroup. */
+int qt_gdn_decode_step(const void* proj, void* conv_pool, const void* conv_w, const float* A_log, const float* dt_bias,
+                       float* ssm_pool, const int32_t* slots, const int32_t* pos, void* y, int B, int n_slots,
+                       int rows_per_wg, qt_stream_t stream);
+
+/* batch_spec.deltanet_bm (qwen35/batch_spec.py:142-150): M chained tokens for each of B sequences, a state snapshot
+ * after every token.  proj [B*M,8224]; conv_pool [n_entries*2,M,3,6144]; ssm_pool [n_entries,M,16,128,128];
+ * sslots, sels, pars [B] int32 (pool entry, snapshot to start from, conv buffer to read); y [B*M,2048].  1 <= M <= 16. */
+int qt_gdn_verify_step(const void* proj, void* conv_pool, const void* conv_w, const float* A_log, const float* dt_bias,
+                       float* ssm_pool, const int32_t* sslots, const int32_t* sels, const int32_t* pars, void* y, int B,
+                       int M, int n_entries, int rows_per_wg, qt_stream_t stream);
+
+/* kernels.deltanet (qwen35/kernels.py:555-567): one sequence, M tokens from snapshot sel[0] of conv_snap [n_snap,3,6144]
+ * / ssm_snap [n_snap,16,128,128]; writes y [M,2048], cs_out [M,3,6144], st_out [M,16,128,128]. */
+int qt_gdn_deltanet(const void* proj, const void* conv_snap, const void* conv_w, const float* A_log, const float* dt_bias,
+                    const float* ssm_snap, const int32_t* sel, void* y, void* cs_out, float* st_out, int M, int n_snap,
+                    int rows_per_wg, qt_stream_t stream);
+
+/* compute_g and beta = sigmoid(b) (qwen35/gated_delta.py:16-18,158).  a, b: bf16, `rows` rows of hv values with row strides
+ * a_stride / b_stride (elements), so they can point into the projection rows.  Outputs (each may be null): g f32
+ * [rows,hv], log_g f32 [rows,hv] (= log of g before the final exp), beta bf16 [rows,hv]. */
+int qt_gdn_gates(const void* a, const void* b, long a_stride, long b_stride, const float* A_log, const float* dt_bias,
+                 float* g, float* log_g, void* beta, long rows, int hv, qt_stream_t stream);
+
+/* normalize_qk (qwen35/gated_delta.py:21-30) on `rows` rows of dk = 128 bf16 values. */
+int qt_normalize_qk(const void* q, const void* k, void* q_out, void* k_out, long rows, int dk, qt_stream_t stream);
+
+/* prefill.conv_prep (qwen35/prefill.py:228-238): proj [S,8224], conv_state [3,6144] -> q, k, v [S,16,128] bf16. */
+int qt_gdn_conv_prep(const void* proj, const void* conv_state, const void* conv_w, void* q, void* k, void* v, int S,
+                     qt_stream_t stream);
+
+/* batch.gnorm_rows / prefill.gated_norm (qwen35/batch.py:338-343, qwen35/prefill.py:241-244): y [rows,2048] bf16,
+ * z = proj[:,6144:8192] of proj [rows,8224], gw [128] f32 -> out [rows,2048] bf16. */
+int qt_gated_rmsnorm(const void* y, const void* proj, const float* gw, void* out, long rows, float eps, qt_stream_t stream);
+
+/* gated_delta_update's recurrence kernel (qwen35/gated_delta.py:143-174) with g (f32) and beta (bf16) [B,T,Hv] given:
+ * q, k [B,T,Hk,128], v, y [B,T,Hv,Dv] bf16, state [B,Hv,Dv,128] f32.  Dk must be 128 and Dv a multiple of 16, otherwise -4
+ * (the reference raises ValueError, gated_delta.py:164-166). */
+int qt_gdn_recurrent(const void* q, const void* k, const void* v, const float* g, const void* beta, const float* state_in,
+                     float* state_out, void* y, int B, int T, int Hk, int Hv, int Dk, int Dv, qt_stream_t stream);
+
+/* batch.attn_b (qwen35/batch.py:230-237): ragged decode / verify attention, 8 query heads on 2 KV heads, head dim 256.
+ * q [B*M,8,256], k_new / v_new [B*M,2,256], pools Kp / Vp [n_slots,2,Lmax,256] bf16 (rows pos[b]..pos[b]+M-1 are appended),
+ * out [B*M,8,256].  1 <= M <= 4.  CH = pool keys per split-K workgroup (multiple of 16); workspace of at least
+ * qt_gqa_attn_workspace_bytes(B, M, Lmax, CH) bytes, 16-byte aligned, owned by the caller. */
+long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH);
+int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
+                       const int32_t* pos, void* out, void* workspace, long workspace_bytes, int B, int M, int Lmax,
+                       int n_slots, int CH, qt_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -25,6 +25,7 @@ _SIGS = {
     "qt_gdn_conv_prep": [_vp] * 6 + [_i, _vp],
     "qt_gated_rmsnorm": [_vp, _vp, _vp, _vp, _l, _f, _vp],
     "qt_gdn_recurrent": [_vp] * 8 + [_i] * 6 + [_vp],
+    "qt_gqa_attn_decode": [_vp] * 9 + [_l, _i, _i, _i, _i, _i, _vp],
 }
 
 
@@ -38,6 +39,7 @@ def lib():
         for name, args in _SIGS.items():
             fn = getattr(L, name)
             fn.argtypes, fn.restype = args, ctypes.c_int
+        L.qt_gqa_attn_workspace_bytes.argtypes, L.qt_gqa_attn_workspace_bytes.restype = [_i] * 4, ctypes.c_long
         _lib = L
     return _lib
 

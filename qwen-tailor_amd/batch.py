@@ -35,6 +35,48 @@ def deltanet_b(proj, conv_pool, conv_w, A_log, dt_bias, ssm_pool, slots, pos, ro
     return y
 
 
+_WORKSPACE = {}
+
+
+def _workspace(dev, nbytes):
+    """Split-K scratch of the attention kernel: one cached buffer per device, grown on demand (the C ABI never allocates)."""
+    buf = _WORKSPACE.get(dev)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _WORKSPACE[dev] = buf
+    return buf
+
+
+def split_size(Lmax: int) -> int:
+    """keys per split-K workgroup"""
+    return 256 if Lmax <= 4096 else (512 if Lmax <= 16384 else 1024)
+
+
+def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None):
+    """q [R,H,D], k / v [R,KV,D] (normed + roped), pools [S+1,KV,Lmax,D]; R = B*M rows (row b*M+j = position pos[b]+j of slot
+    slots[b]; slots / pos int32 [B]).  Returns o [R,H,D] bf16 and appends k / v at pos[b]+j (in place)
+    (qwen35/batch.py:230-237)."""
+    q = L.dev(q, BF16, "q", (None, 8, 256))
+    R = q.shape[0]
+    if M < 1 or M > 4 or R % M:
+        raise ValueError(f"attn_b: M = {M} (1..4) must divide the number of rows ({R})")
+    B = R // M
+    k, v = L.dev(k, BF16, "k", (R, 2, 256)), L.dev(v, BF16, "v", (R, 2, 256))
+    Kp = L.dev(Kp, BF16, "Kp", (None, 2, None, 256))
+    Vp = L.dev(Vp, BF16, "Vp", tuple(Kp.shape))
+    n_slots, Lmax = Kp.shape[0], Kp.shape[2]
+    slots, pos = L.i32(slots, "slots", B), L.i32(pos, "pos", B)
+    CH = split or split_size(Lmax)
+    nbytes = L.lib().qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)
+    if nbytes < 0:
+        raise ValueError("attn_b: bad split size")
+    ws = _workspace(q.device, nbytes)
+    o = torch.empty((R, 8, 256), dtype=BF16, device=q.device)
+    L.call("qt_gqa_attn_decode", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(Kp), L.ptr(Vp), L.ptr(slots), L.ptr(pos), L.ptr(o), L.ptr(ws),
+           ws.numel(), B, M, Lmax, n_slots, CH, L.stream())
+    return o
+
+
 def gnorm_rows(y, proj, gw, eps=1e-6):
     """Gated RMSNorm of the delta-rule output (qwen35/batch.py:338-343): y [B, 2048] bf16, proj [B, 8224] bf16 (its z slice
     is at 6144:8192), gw float32 [128].  Returns [B, 2048] bf16."""

@@ -1,0 +1,91 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol include/qwen_tailor_hip.h declares, the host layer
+validates its arguments before anything reaches the GPU, and nothing in the product imports the oracle."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "qwen_tailor_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(qt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    import qwen_tailor_amd as qt
+    lib = qt._lib.lib()
+    names = declared_symbols()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/qwen_tailor_hip.h but not exported"
+
+
+def test_every_exported_entry_point_is_declared():
+    import subprocess
+    import qwen_tailor_amd as qt
+    out = subprocess.run(["nm", "-D", "--defined-only", qt._build.SO], capture_output=True, text=True, check=True).stdout
+    exported = sorted(set(re.findall(r"\bT (qt_[a-z0-9_]+)", out)))
+    assert exported == declared_symbols()
+
+
+def test_host_rejects_bad_arguments_without_a_gpu():
+    import qwen_tailor_amd as qt
+    x = torch.zeros((2, 8224), dtype=torch.bfloat16)
+    with pytest.raises(TypeError):                 # CPU tensors never reach the C ABI (no CPU fallback exists)
+        qt.batch.deltanet_b(x, x, x, x, x, x, x, x)
+    with pytest.raises(TypeError):
+        qt.prefill.conv_prep(x, x, x)
+    with pytest.raises(TypeError):
+        qt.batch.attn_b(x, x, x, x, x, x, x)
+
+
+def test_null_and_dimension_errors_from_the_c_abi():
+    import qwen_tailor_amd as qt
+    lib = qt._lib.lib()
+    z = ctypes.c_void_p(0)
+    assert lib.qt_gdn_decode_step(z, z, z, z, z, z, z, z, z, 1, 1, 0, z) == -3
+    assert lib.qt_gqa_attn_workspace_bytes(16, 1, 32768, 1024) == 16 * 2 * 32 * 4 * 258 * 4
+    assert lib.qt_gqa_attn_workspace_bytes(1, 0, 16, 16) == -1
+    assert lib.qt_normalize_qk(ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16), 1, 64, z) == -4
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "qwen-tailor_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"
+
+
+def test_pools_shapes_and_byte_accounting():
+    """Pools / SpecPools layouts and slot_bytes (qwen35/batch.py:405-426, qwen35/batch_spec.py:242-270) on the CPU device."""
+    import qwen_tailor_amd as qt
+    cfg = qt.model.Cfg()
+    assert cfg.conv_dim == 6144 and sum(cfg.is_linear(i) for i in range(cfg.layers)) == 18
+    P = qt.batch.Pools(cfg, 3, 64, device="cpu")
+    assert len(P.ssm) == 18 and len(P.K) == 6
+    assert tuple(P.ssm[0].shape) == (4, 16, 128, 128) and tuple(P.conv[0].shape) == (8, 3, 6144)
+    assert tuple(P.K[0].shape) == (4, 2, 64, 256)
+    assert P.nbytes() == 4 * qt.batch.Pools.slot_bytes(cfg, 64)
+    assert qt.batch.Pools.slot_bytes(cfg, 64, double_conv=False) == 18 * (16 * 128 * 128 * 4 + 3 * 6144 * 2) + 6 * 2 * 2 * 64 * 256 * 2
+    st = {"conv": [torch.randn(1, 3, 6144).bfloat16() for _ in range(18)], "ssm": [torch.randn(1, 16, 128, 128) for _ in range(18)],
+          "kv": [(torch.randn(1, 2, 64, 256).bfloat16(), torch.randn(1, 2, 64, 256).bfloat16()) for _ in range(6)]}
+    P.load(2, st, 37)                                       # tests/batch.py:102-112: load -> read round trip, other slots stay zero
+    back = P.read(2, 37, 64)
+    assert all(torch.equal(a, b) for a, b in zip(back["ssm"], st["ssm"]))
+    assert all(torch.equal(a, b) for a, b in zip(back["conv"], st["conv"]))
+    assert all(torch.equal(a[0][:, :, :37], b[0][:, :, :37]) and torch.equal(a[1][:, :, :37], b[1][:, :, :37])
+               for a, b in zip(back["kv"], st["kv"]))
+    assert all(float(x[0].abs().max()) == 0 and float(x[1].abs().max()) == 0 for x in P.ssm + P.K)
+    assert torch.equal(P.conv[0][2 * 2 + 1], st["conv"][0][0]) and float(P.conv[0][2 * 2].abs().max()) == 0   # parity pos & 1
+    with pytest.raises(AssertionError):
+        P.load(3, st, 1)                                    # the trash slot cannot be loaded (batch.py:434)
+    SP = qt.batch_spec.SpecPools(cfg, 2, 3, 4, 64, device="cpu")
+    assert tuple(SP.ssm[0].shape) == (3, 4, 16, 128, 128) and tuple(SP.conv[0].shape) == (6, 4, 3, 6144)
+    assert qt.batch_spec.SpecPools.entry_bytes(cfg, 4) == 18 * 4 * (16 * 128 * 128 * 4 + 2 * 3 * 6144 * 2)

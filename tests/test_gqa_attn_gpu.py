@@ -1,0 +1,122 @@
+"""GPU parity of the ragged GQA hd256 decode / verify attention against the CPU oracle (float64 softmax attention).
+Tolerance (BASELINE north star): bf16 attention outputs within 1e-2 relative."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gdn_oracle as O
+from tests.util import *  # noqa: F401,F403
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def qt():
+    import qwen_tailor_amd as q
+    q._lib.lib()
+    return q
+
+
+def check_attn(name, got, ref):
+    check_rel(name + " rel-L2", got, ref, 1e-2, rel_l2)
+    check_rel(name + " max", got, ref, 1e-2, rel_max)
+
+
+def run_case(qt, dev, rng, S, Lmax, slots, pos, M, split=None):
+    B = len(slots)
+    Kp = bf(rng.standard_normal((S + 1, 2, Lmax, 256)))
+    Vp = bf(rng.standard_normal((S + 1, 2, Lmax, 256)))
+    q = bf(rng.standard_normal((B * M, 8, 256)))
+    kn = bf(rng.standard_normal((B * M, 2, 256)))
+    vn = bf(rng.standard_normal((B * M, 2, 256)))
+    dK, dV = to_dev(Kp, dev, BF16), to_dev(Vp, dev, BF16)
+    o = qt.batch.attn_b(to_dev(q, dev, BF16), to_dev(kn, dev, BF16), to_dev(vn, dev, BF16), dK, dV, to_dev(slots, dev), to_dev(pos, dev),
+                        M, split=split)
+    oK, oV = Kp.copy(), Vp.copy()
+    ref = O.attn_b(q, kn, vn, oK, oV, slots, pos, M)
+    check_attn(f"o (M={M})", to_np(o), ref)
+    check_equal("K pool (appended rows, everything else untouched)", to_np(dK), oK)
+    check_equal("V pool", to_np(dV), oV)
+    return to_np(o)
+
+
+def test_attn_b_layout_of_reference_test(qt, dev):
+    """reference tests/batch.py:73-100: 6 rows, positions 0..1023, slots scattered in a 7-slot pool"""
+    rng = np.random.default_rng(11)
+    run_case(qt, dev, rng, 6, 1024, np.array([3, 0, 5, 1, 2, 4], np.int32), np.array([0, 1, 31, 32, 300, 1023], np.int32), 1)
+
+
+@pytest.mark.parametrize("M", [2, 3, 4])
+def test_attn_b_verify_rows(qt, dev, M):
+    """reference tests/batch_spec.py:69-101: M query rows per sequence, causal among the new keys"""
+    rng = np.random.default_rng(M)
+    run_case(qt, dev, rng, 6, 1024, np.array([3, 0, 5, 1, 2], np.int32), np.array([0, 1, 30, 300, 1000], np.int32), M)
+
+
+def test_attn_b_split_invariance_and_single_key(qt, dev):
+    rng = np.random.default_rng(5)
+    slots, pos = np.array([1, 0], np.int32), np.array([777, 0], np.int32)
+    outs = []
+    for split in (16, 64, 256, 1024):
+        rng2 = np.random.default_rng(5)
+        outs.append(run_case(qt, dev, rng2, 2, 1024, slots, pos, 1, split=split))
+    for o in outs[1:]:
+        check_rel("split count changes the result only by rounding", o, outs[0], 1e-2, rel_max)
+    # a sequence at position 0 sees exactly one key (its own): o = v for every head of the group
+    rng3 = np.random.default_rng(5)
+    Kp = bf(rng3.standard_normal((3, 2, 1024, 256)))
+    Vp = bf(rng3.standard_normal((3, 2, 1024, 256)))
+    q = bf(rng3.standard_normal((2, 8, 256)))
+    kn = bf(rng3.standard_normal((2, 2, 256)))
+    vn = bf(rng3.standard_normal((2, 2, 256)))
+    check_equal("single key: o == v", outs[0][1], np.repeat(vn[1], 4, axis=0))
+
+
+def test_attn_b_out_of_range_rows_are_skipped(qt, dev):
+    rng = np.random.default_rng(6)
+    Kp = to_dev(bf(rng.standard_normal((3, 2, 64, 256))), dev, BF16)
+    Vp = to_dev(bf(rng.standard_normal((3, 2, 64, 256))), dev, BF16)
+    K0, V0 = Kp.clone(), Vp.clone()
+    q = to_dev(bf(rng.standard_normal((2, 8, 256))), dev, BF16)
+    kn = to_dev(bf(rng.standard_normal((2, 2, 256))), dev, BF16)
+    qt.batch.attn_b(q, kn, kn, Kp, Vp, torch.tensor([5, 1], dtype=torch.int32, device=dev), torch.tensor([3, 64], dtype=torch.int32, device=dev))
+    torch.cuda.synchronize()
+    check_tensors_equal("pools untouched by a bad slot / a full sequence", Kp, K0)
+    check_tensors_equal("pools untouched", Vp, V0)
+    with pytest.raises(ValueError):
+        qt.batch.attn_b(q, kn, kn, Kp, Vp, torch.tensor([0], dtype=torch.int32, device=dev), torch.tensor([0], dtype=torch.int32, device=dev), M=5)
+
+
+def test_attn_b_config3_ragged_long(qt, dev):
+    """BASELINE config 3: B=16, one query each, ragged KV lengths uniform in [512, 32768] (seed 1003)"""
+    rng = np.random.default_rng(1003)
+    B, Lmax = 16, 32768
+    pos = rng.integers(512, 32768, B).astype(np.int32)                          # keys already in the pool (+1 new)
+    pos[0], pos[1] = 32767, 512
+    slots = rng.permutation(B).astype(np.int32)
+    g = torch.Generator().manual_seed(1003)
+    Kp = torch.randn((B + 1, 2, Lmax, 256), generator=g, dtype=torch.float32).bfloat16()
+    Vp = torch.randn((B + 1, 2, Lmax, 256), generator=g, dtype=torch.float32).bfloat16()
+    q = bf(rng.standard_normal((B, 8, 256)))
+    kn = bf(rng.standard_normal((B, 2, 256)))
+    vn = bf(rng.standard_normal((B, 2, 256)))
+    dK, dV = Kp.to(dev), Vp.to(dev)
+    o = to_np(qt.batch.attn_b(to_dev(q, dev, BF16), to_dev(kn, dev, BF16), to_dev(vn, dev, BF16), dK, dV, to_dev(slots, dev), to_dev(pos, dev)))
+    for b in range(B):                                                         # oracle per sequence on views (no 2 GB copies)
+        s_, p = int(slots[b]), int(pos[b])
+        Kb = Kp[s_:s_ + 1, :, :p + 1].float().numpy().copy()
+        Vb = Vp[s_:s_ + 1, :, :p + 1].float().numpy().copy()
+        ref = O.attn_b(q[b:b + 1], kn[b:b + 1], vn[b:b + 1], Kb, Vb, np.array([0]), np.array([p]), 1)
+        check_attn(f"sequence {b} (L={p + 1})", o[b:b + 1], ref)
+        check_equal("appended K row", to_np(dK[s_, :, p]), kn[b])
+        check_equal("appended V row", to_np(dV[s_, :, p]), vn[b])
+    check_tensors_equal("trash slot untouched", dK[B].cpu(), Kp[B])
+
+
+def test_attn_b_config4_verify_mix(qt, dev):
+    """BASELINE config 4 (attention half): B=16 x M=4, KV lengths uniform in [1024, 8192], 4-token causal tail"""
+    rng = np.random.default_rng(1004)
+    B, M, Lmax = 16, 4, 8192 + 8
+    pos = rng.integers(1024, 8192, B).astype(np.int32)
+    slots = rng.permutation(B).astype(np.int32)
+    run_case(qt, dev, rng, B, Lmax, slots, pos, M)
