@@ -39,7 +39,7 @@ __device__ __forceinline__ float rsqrt_rn(float x) { return (float)(1.0 / sqrt((
 // The bf16 -> bf16 helpers below must return the bits the contract defines (exp32 / log32 = correctly rounded), but the
 // double-precision libm calls are ~10x the work of the float ones.  A float result that is off by a few ulp rounds to the
 // same bf16 value unless it lies within those few ulp of a bf16 rounding boundary; only then is the slow path taken
-// (about one evaluation in 10^4).  The GPU tests compare all 65536 inputs of each helper with the CPU oracle.
+// (about one evaluation in 10^4).  The GPU tests compare all 65536 inputs of each helper with a CPU restatement.
 __device__ __forceinline__ bool near_bf16_tie(float v, uint32_t slack) {
     const uint32_t lo = __float_as_uint(v) & 0xffffu;
     return (lo - (0x8000u - slack)) <= 2u * slack;
