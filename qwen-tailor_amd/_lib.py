@@ -26,6 +26,7 @@ _SIGS = {
     "qt_gated_rmsnorm": [_vp, _vp, _vp, _vp, _l, _f, _vp],
     "qt_gdn_recurrent": [_vp] * 8 + [_i] * 6 + [_vp],
     "qt_gqa_attn_decode": [_vp] * 9 + [_l, _i, _i, _i, _i, _i, _vp],
+    "qt_gdn_phase_b": [_vp] * 6 + [_i, _vp],
 }
 
 
@@ -40,6 +41,8 @@ def lib():
             fn = getattr(L, name)
             fn.argtypes, fn.restype = args, ctypes.c_int
         L.qt_gqa_attn_workspace_bytes.argtypes, L.qt_gqa_attn_workspace_bytes.restype = [_i] * 4, ctypes.c_long
+        for name in ("qt_gdn_chunk_ops_bytes", "qt_gdn_chunk_u_bytes", "qt_gdn_chunk_gc_bytes"):
+            getattr(L, name).argtypes, getattr(L, name).restype = [_i], ctypes.c_long
         _lib = L
     return _lib
 

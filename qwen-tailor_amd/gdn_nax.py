@@ -1,0 +1,44 @@
+"""Two-phase chunked gated-delta-rule for prefill: the call surface of qwen35/gdn_nax.py (prep_a, phase_b, gdn_chunked).
+
+Chunk size is 64 (the reference's is 16; the chunked form is an identity for every chunk size).  The three buffers that
+travel from phase A to phase B keep the reference's argument slots (Tbuf, Abuf, gv) but hold this implementation's own
+records: the packed half-precision MFMA operands, the U accumulators, and the per-chunk decay gamma_C."""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+from .kernels import flat_conv_w
+
+BF16 = torch.bfloat16
+HV, DK, DV, CD, PW = 16, 128, 128, 6144, 8224
+CHUNK = 64
+
+# precision flags of the reference (qwen35/gdn_nax.py:363-366) are accepted and ignored: the operands are always fp16
+FLAGS = ("RNE", "SPLIT_P1", "SPLIT_P2", "SPLIT_D", "SPLIT_Y", "SPLIT_DP", "PF")
+DEFAULT_FLAGS = frozenset()
+TG = 64
+
+
+def _alloc_records(S, dev):
+    lib = L.lib()
+    ops = torch.empty(lib.qt_gdn_chunk_ops_bytes(S) // 2, dtype=torch.float16, device=dev)
+    U = torch.empty(lib.qt_gdn_chunk_u_bytes(S) // 4, dtype=torch.float32, device=dev)
+    gC = torch.empty(lib.qt_gdn_chunk_gc_bytes(S) // 4, dtype=torch.float32, device=dev)
+    return ops, U, gC
+
+
+def phase_b(q, k, v, Tb, Am, gv, state, relaxed=True, flags=DEFAULT_FLAGS, tg=None):
+    """The serial state recurrence on the outputs of phase A -> y [S,16,128] bf16, new state [1,16,128,128] f32
+    (qwen35/gdn_nax.py:404-410).  Tb / Am / gv are the records prep_a (or gdn_chunked's phase A) produced."""
+    S = q.shape[0]
+    ops, U, gC = L.dev(Tb, torch.float16, "Tb"), L.dev(Am, torch.float32, "Am"), L.dev(gv, torch.float32, "gv")
+    lib = L.lib()
+    if ops.numel() * 2 < lib.qt_gdn_chunk_ops_bytes(S) or U.numel() * 4 < lib.qt_gdn_chunk_u_bytes(S) or \
+            gC.numel() * 4 < lib.qt_gdn_chunk_gc_bytes(S):
+        raise ValueError("phase_b: the phase A records are too small for this many tokens")
+    state = L.dev(state, torch.float32, "state").reshape(1, HV, DV, DK)
+    y = torch.empty((S, HV, DV), dtype=BF16, device=state.device)
+    out = torch.empty_like(state)
+    L.call("qt_gdn_phase_b", L.ptr(ops), L.ptr(U), L.ptr(gC), L.ptr(state), L.ptr(out), L.ptr(y), S, L.stream())
+    return y, out
