@@ -27,6 +27,7 @@ _SIGS = {
     "qt_gdn_recurrent": [_vp] * 8 + [_i] * 6 + [_vp],
     "qt_gqa_attn_decode": [_vp] * 9 + [_l, _i, _i, _i, _i, _i, _vp],
     "qt_gdn_phase_b": [_vp] * 6 + [_i, _vp],
+    "qt_gdn_phase_a": [_vp] * 8 + [_i, _vp, _vp, _vp, _i, _vp],
 }
 
 

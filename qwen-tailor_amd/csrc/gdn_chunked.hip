@@ -107,6 +107,339 @@ __global__ __launch_bounds__(64) void gdn_phase_b_kernel(const _Float16* __restr
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------------------------
+// Phase A: one workgroup of 256 threads per (chunk, head).
+// ------------------------------------------------------------------------------------------------------------------
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int QS_LD = DK + 8;        // row strides (elements) of the LDS tiles: keep 16-byte alignment, spread the banks
+constexpr int KT_LD = C + 8;
+constexpr int LS_LD = C + 4;
+constexpr int TAB_LO = 118, TAB_N = 14 * 128;      // silu table: bf16 exponent fields 118..131, i.e. 2^-9 <= |x| < 2^5
+
+struct PhaseALds {
+    bf16_t tab[2 * TAB_N];
+    __align__(16) bf16_t Qs[C * QS_LD];
+    __align__(16) bf16_t Ks[C * QS_LD];
+    __align__(16) bf16_t KT[DK * KT_LD];
+    __align__(16) bf16_t VT[DV * KT_LD];
+    __align__(16) float Ls[C * LS_LD];
+    __align__(16) float Ts[C * LS_LD];
+    float Lc[C], beta[C], gam[C], dec[C];
+};
+
+// silu_bf16 of a bf16 value through the table; outside the table's range the closed forms / the direct evaluation
+__device__ __forceinline__ float silu_lookup(const bf16_t* tab, bf16_t xb) {
+    const unsigned e = (xb >> 7) & 0xffu;
+    if (e < (unsigned)TAB_LO) return BF(bf2f(xb) * 0.5f);            // exp(|x|) rounds to 1: sigmoid_bf16 = 0.5 exactly
+    if (__builtin_expect(e > (unsigned)(TAB_LO + 13), 0)) return silu_bf16(bf2f(xb));
+    return bf2f(tab[(xb >> 15) * TAB_N + (xb & 0x7fffu) - TAB_LO * 128]);
+}
+
+__device__ __forceinline__ half8 to_half8(const float (&v)[8]) {
+    half8 h;
+#pragma unroll
+    for (int j = 0; j < 8; j++) h[j] = (_Float16)v[j];
+    return h;
+}
+__device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]) {
+    f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
+    f[4] = lo_bf(w.z); f[5] = hi_bf(w.z); f[6] = lo_bf(w.w); f[7] = hi_bf(w.w);
+}
+__device__ __forceinline__ void unpack4(uint2 w, float* f) {
+    f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
+}
+
+// proj [S,8224], cs [3,6144], cw [6144*4] -> q, k, v [S,16,128] (optional) and the phase B records.
+// FROM_QKV: q, k, v are inputs (already convolved and normalized, gdn_nax.gdn_chunked) and the conv is skipped.
+template <bool FROM_QKV>
+__global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs,
+                                                          const bf16_t* __restrict__ cw, const float* __restrict__ A_log,
+                                                          const float* __restrict__ dt_bias, bf16_t* __restrict__ qo,
+                                                          bf16_t* __restrict__ ko, bf16_t* __restrict__ vo,
+                                                          _Float16* __restrict__ ops, float* __restrict__ U,
+                                                          float* __restrict__ gC, int S) {
+    __shared__ PhaseALds L;
+    const int c = blockIdx.x / HV, h = blockIdx.x % HV, t0 = c * C;
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const size_t rec = (size_t)c * HV + h;
+    _Float16* op = ops + rec * OP_HALVES;
+
+    // ---- silu table, zero the blocks of T above the diagonal
+    for (int i = tid; i < 2 * TAB_N; i += 256) {
+        const int sgn = i / TAB_N, em = i % TAB_N;
+        const bf16_t xb = (bf16_t)((sgn << 15) | (TAB_LO * 128 + em));
+        L.tab[i] = f2bf(silu_bf16(bf2f(xb)));
+    }
+    for (int i = tid; i < C * LS_LD; i += 256) L.Ts[i] = 0.f;
+
+    // ---- gates of the chunk's tokens (gdn_nax.py:80-104): wave 0, one token per lane
+    if (w == 0) {
+        const int t = t0 + lane;
+        float lg = 0.f, be = 0.f;
+        if (t < S) {
+            lg = log_decay(A_log[h], BF(bf2f(proj[(size_t)t * PW + CD + KD + HV + h]) + dt_bias[h]));
+            be = sigmoid_bf16(bf2f(proj[(size_t)t * PW + CD + KD + h]));
+        }
+        float lc = lg;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const float o = __shfl_up(lc, d, 64);
+            if (lane >= d) lc += o;
+        }
+        const float tot = __shfl(lc, 63, 64);
+        L.Lc[lane] = lc;
+        L.beta[lane] = be;
+        L.gam[lane] = expf(lc);
+        L.dec[lane] = expf(tot - lc);
+        if (lane == 63) gC[rec] = expf(lc);
+    }
+    __syncthreads();
+
+    // ---- conv + silu + q/k norm (kernels.py:476-510): a 16-lane group owns one token, a lane 8 channels of q, k and v
+    {
+        const int gi = tid >> 4, cc = tid & 15;
+        const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
+        for (int rr = 0; rr < 4; rr++) {
+            const int tl = rr * 16 + gi, t = t0 + tl;
+            float u[3][8];
+            if (FROM_QKV) {
+                if (t < S) {
+                    const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
+                    unpack8(*reinterpret_cast<const uint4*>(qo + o), u[0]);
+                    unpack8(*reinterpret_cast<const uint4*>(ko + o), u[1]);
+                    unpack8(*reinterpret_cast<const uint4*>(vo + o), u[2]);
+                } else {
+#pragma unroll
+                    for (int part = 0; part < 3; part++)
+#pragma unroll
+                        for (int e = 0; e < 8; e++) u[part][e] = 0.f;
+                }
+            } else if (t < S) {
+#pragma unroll
+                for (int part = 0; part < 3; part++) {
+                    const int ch0 = part * KD + h * DK + cc * 8;
+                    float x[4][8];
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+                        const int tt = t - 3 + d;
+                        const bf16_t* src = tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0;
+                        unpack8(*reinterpret_cast<const uint4*>(src), x[d]);
+                    }
+#pragma unroll
+                    for (int e2 = 0; e2 < 8; e2 += 2) {
+                        const uint4 ww = *reinterpret_cast<const uint4*>(cw + (size_t)(ch0 + e2) * 4);
+                        const uint2 w0 = make_uint2(ww.x, ww.y), w1 = make_uint2(ww.z, ww.w);
+#pragma unroll
+                        for (int e = 0; e < 2; e++) {
+                            const uint2 wc = e ? w1 : w0;
+                            float sacc = x[0][e2 + e] * lo_bf(wc.x);
+                            sacc = sacc + x[1][e2 + e] * hi_bf(wc.x);
+                            sacc = sacc + x[2][e2 + e] * lo_bf(wc.y);
+                            sacc = sacc + x[3][e2 + e] * hi_bf(wc.y);
+                            u[part][e2 + e] = silu_lookup(L.tab, f2bf(sacc));
+                        }
+                    }
+                }
+                double sq = 0.0, sk = 0.0;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    sq += (double)u[0][e] * u[0][e];
+                    sk += (double)u[1][e] * u[1][e];
+                }
+                const float qr = rsqrt_rn((float)row16_sum_d(sq) / (float)DK + qk_eps());
+                const float kr = rsqrt_rn((float)row16_sum_d(sk) / (float)DK + qk_eps());
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    u[0][e] = BF(BF(u[0][e] * qr) * scq);
+                    u[1][e] = BF(BF(u[1][e] * kr) * sck);
+                }
+            } else {
+#pragma unroll
+                for (int part = 0; part < 3; part++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) u[part][e] = 0.f;             // rows past the end are zero (gdn_nax.py:172-174)
+            }
+            uint4 pk[3];
+#pragma unroll
+            for (int part = 0; part < 3; part++)
+                pk[part] = make_uint4(pack_bf(u[part][0], u[part][1]), pack_bf(u[part][2], u[part][3]),
+                                      pack_bf(u[part][4], u[part][5]), pack_bf(u[part][6], u[part][7]));
+            *reinterpret_cast<uint4*>(&L.Qs[tl * QS_LD + cc * 8]) = pk[0];
+            *reinterpret_cast<uint4*>(&L.Ks[tl * QS_LD + cc * 8]) = pk[1];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                L.KT[(cc * 8 + e) * KT_LD + tl] = f2bf(u[1][e]);
+                L.VT[(cc * 8 + e) * KT_LD + tl] = f2bf(u[2][e]);
+            }
+            if (!FROM_QKV && qo && t < S) {
+                const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
+                *reinterpret_cast<uint4*>(qo + o) = pk[0];
+                *reinterpret_cast<uint4*>(ko + o) = pk[1];
+                *reinterpret_cast<uint4*>(vo + o) = pk[2];
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- K K^T (lower tiles) -> L, and (Q K^T)^T -> Am, on bf16 MFMA.  Wave w: row of tiles ti = 3 - w of K K^T and the
+    // Am tiles of ct = w.
+    {
+        const int ti = 3 - w;
+        for (int tj = 0; tj <= ti; tj++) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kb = 0; kb < 4; kb++) {
+                const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * ti + n) * QS_LD + 32 * kb + 8 * g]));
+                const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+            }
+            const int j = 16 * tj + n;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int i = 16 * ti + 4 * g + r;
+                L.Ls[i * LS_LD + j] = i > j ? L.beta[i] * expf(L.Lc[i] - L.Lc[j]) * acc[r] : 0.f;
+            }
+        }
+        const int ct = w, co = 16 * ct + n;                         // Am: rows c_out = 16 ct + n, k = c_in (permuted)
+        for (int kb2 = 0; kb2 < 2; kb2++) {
+            f32x4 part[2];
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+                const int tj = 2 * kb2 + hf;
+                part[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (tj <= ct) {
+#pragma unroll
+                    for (int kb = 0; kb < 4; kb++) {
+                        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]));
+                        const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 8 * g]));
+                        part[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, part[hf], 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int ci = 16 * tj + 4 * g + r;
+                        part[hf][r] = ci <= co ? expf(L.Lc[co] - L.Lc[ci]) * part[hf][r] : 0.f;
+                    }
+                }
+            }
+            *reinterpret_cast<half8*>(op + OP_A + (ct * 2 + kb2) * 512 + lane * 8) = pack_half8(part[0], part[1]);
+        }
+    }
+    __syncthreads();
+
+    // ---- T = (I + L)^-1 by blocks of 16 (exact fp32: forward substitution on the diagonal blocks, fp32 MFMA below them)
+    f32x4 TR[4];                                   // TR[d] = block (w + d, w) of T, accumulator layout
+    {
+        float x[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float a = (i == n) ? 1.f : 0.f;
+            const float* lr = &L.Ls[(16 * w + i) * LS_LD + 16 * w];
+#pragma unroll
+            for (int m = 0; m < i; m++) a -= lr[m] * x[m];
+            x[i] = a;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float v = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) v = (i == 4 * g + r) ? x[i] : v;
+            TR[0][r] = v;
+            L.Ts[(16 * w + 4 * g + r) * LS_LD + 16 * w + n] = v;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int d = 1; d < 4; d++) {
+        if (w + d < 4) {
+            const int I = w + d;
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int e = 0; e < d; e++) {
+                const f32x4 a4 = *reinterpret_cast<const f32x4*>(&L.Ls[(16 * I + n) * LS_LD + 16 * (w + e) + 4 * g]);
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[kk], TR[e][kk], acc, 0, 0, 0);
+            }
+            f32x4 res = {0.f, 0.f, 0.f, 0.f};
+            const f32x4 d4 = *reinterpret_cast<const f32x4*>(&L.Ts[(16 * I + n) * LS_LD + 16 * I + 4 * g]);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) res = __builtin_amdgcn_mfma_f32_16x16x4f32(d4[kk], acc[kk], res, 0, 0, 0);
+            TR[d] = -res;
+#pragma unroll
+            for (int r = 0; r < 4; r++) L.Ts[(16 * I + 4 * g + r) * LS_LD + 16 * w + n] = TR[d][r];
+        }
+    }
+    __syncthreads();
+
+    // ---- Wn^T = -(gamma K)^T Tb^T and U = Tb V on fp16 MFMA; wave w owns the chunk rows of tile ct = w
+    {
+        const int ct = w, nkb = ct < 2 ? 1 : 2;                     // Tb is lower triangular: columns past the row tile are zero
+        half8 tb[2];
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; kb2++) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int cp = 32 * kb2 + 8 * g + j;
+                v[j] = L.Ts[(16 * ct + n) * LS_LD + cp] * L.beta[cp];
+            }
+            tb[kb2] = to_half8(v);
+        }
+        for (int kb = 0; kb < 4; kb++) {
+            f32x4 acc[2];
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+                const int mt = 2 * kb + hf;
+                acc[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kb2 = 0; kb2 < 2; kb2++) {
+                    if (kb2 >= nkb) continue;
+                    float kf[8];
+                    unpack8(*reinterpret_cast<const uint4*>(&L.KT[(16 * mt + n) * KT_LD + 32 * kb2 + 8 * g]), kf);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) kf[j] *= -L.gam[32 * kb2 + 8 * g + j];
+                    acc[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(to_half8(kf), tb[kb2], acc[hf], 0, 0, 0);
+                }
+            }
+            *reinterpret_cast<half8*>(op + OP_W + (ct * 4 + kb) * 512 + lane * 8) = pack_half8(acc[0], acc[1]);
+        }
+        float* up = U + rec * U_FLOATS;
+        for (int sl = 0; sl < 8; sl++) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kb2 = 0; kb2 < 2; kb2++) {
+                if (kb2 >= nkb) continue;
+                float vf[8];
+                unpack8(*reinterpret_cast<const uint4*>(&L.VT[(16 * sl + n) * KT_LD + 32 * kb2 + 8 * g]), vf);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tb[kb2], to_half8(vf), acc, 0, 0, 0);
+            }
+            *reinterpret_cast<f32x4*>(up + ((sl * NCT + ct) * 64 + lane) * 4) = acc;
+        }
+        // Qg = gamma * Q (rows of tile ct) and Kd = (dec * K)^T (rows dk of tiles 2w, 2w+1), k index permuted
+        const float gm = L.gam[16 * ct + n];
+        for (int kb = 0; kb < 4; kb++) {
+            float qf[8];
+            unpack4(*reinterpret_cast<const uint2*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 4 * g]), qf);
+            unpack4(*reinterpret_cast<const uint2*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 16 + 4 * g]), qf + 4);
+#pragma unroll
+            for (int j = 0; j < 8; j++) qf[j] *= gm;
+            *reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8) = to_half8(qf);
+        }
+        for (int mm = 0; mm < 2; mm++) {
+            const int mt = 2 * w + mm;
+            for (int kb2 = 0; kb2 < 2; kb2++) {
+                float kf[8];
+                unpack4(*reinterpret_cast<const uint2*>(&L.KT[(16 * mt + n) * KT_LD + 32 * kb2 + 4 * g]), kf);
+                unpack4(*reinterpret_cast<const uint2*>(&L.KT[(16 * mt + n) * KT_LD + 32 * kb2 + 16 + 4 * g]), kf + 4);
+#pragma unroll
+                for (int j = 0; j < 8; j++) kf[j] *= L.dec[32 * kb2 + 16 * (j >> 2) + 4 * g + (j & 3)];
+                *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = to_half8(kf);
+            }
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -125,6 +458,26 @@ int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, const float
     const int NC = (S + C - 1) / C;
     hipLaunchKernelGGL(gdn_phase_b_kernel, dim3(HV * 8), dim3(64), 0, stream, (const _Float16*)ops, U, gC, state_in, state_out,
                        (bf16_t*)y, S, NC);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_gdn_phase_a(const void* proj, const void* conv_state, const void* conv_w, const float* A_log, const float* dt_bias,
+                   void* q, void* k, void* v, int from_qkv, void* ops, float* U, float* gC, int S, hipStream_t stream) {
+    if (!proj || !A_log || !dt_bias || !ops || !U || !gC) return QT_ERR_NULL;
+    if (!from_qkv && (!conv_state || !conv_w)) return QT_ERR_NULL;
+    if ((q || k || v || from_qkv) && !(q && k && v)) return QT_ERR_NULL;
+    if (S < 0) return QT_ERR_DIM;
+    if (S == 0) return QT_OK;
+    for (const void* p : {proj, conv_state, conv_w, (const void*)ops, (const void*)U, (const void*)q, (const void*)k, (const void*)v})
+        if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
+    const int NC = (S + C - 1) / C;
+    if (from_qkv)
+        hipLaunchKernelGGL(gdn_phase_a_kernel<true>, dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (const bf16_t*)conv_state,
+                           (const bf16_t*)conv_w, A_log, dt_bias, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, (_Float16*)ops, U, gC, S);
+    else
+        hipLaunchKernelGGL(gdn_phase_a_kernel<false>, dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (const bf16_t*)conv_state,
+                           (const bf16_t*)conv_w, A_log, dt_bias, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, (_Float16*)ops, U, gC, S);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

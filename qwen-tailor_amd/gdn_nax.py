@@ -28,6 +28,37 @@ def _alloc_records(S, dev):
     return ops, U, gC
 
 
+def _phase_a(proj, conv_state, conv_w, A_log, dt_bias, qkv=None, want_qkv=True):
+    proj = L.dev(proj, BF16, "proj", (None, PW))
+    S = proj.shape[0]
+    dev = proj.device
+    A, dtb = L.f32(A_log, "A_log", (HV,)), L.f32(dt_bias, "dt_bias", (HV,))
+    ops, U, gC = _alloc_records(S, dev)
+    if qkv is not None:
+        q, k, v = (L.dev(t, BF16, name, (S, HV, DK)) for t, name in zip(qkv, "qkv"))
+        cs = w = None
+    else:
+        cs = L.dev(conv_state, BF16, "conv_state", (3, CD))
+        w = flat_conv_w(conv_w)
+        q, k, v = (torch.empty((S, HV, DK), dtype=BF16, device=dev) for _ in range(3)) if want_qkv else (None, None, None)
+    L.call("qt_gdn_phase_a", L.ptr(proj), L.ptr(cs), L.ptr(w), L.ptr(A), L.ptr(dtb), L.ptr(q), L.ptr(k), L.ptr(v),
+           1 if qkv is not None else 0, L.ptr(ops), L.ptr(U), L.ptr(gC), S, L.stream())
+    return q, k, v, ops, U, gC
+
+
+def prep_a(proj, conv_state, conv_w, A_log, dt_bias, relaxed=True):
+    """conv+silu+qk-norm and phase A in one kernel (qwen35/gdn_nax.py:394-401).
+    proj [S,8224], conv_state [3,6144], conv_w [6144,4,1] -> q, k, v [S,16,128] bf16 and the three phase-B records."""
+    return _phase_a(proj, conv_state, conv_w, A_log, dt_bias)
+
+
+def gdn_chunked(q, k, v, proj, A_log, dt_bias, state, relaxed=True, flags=DEFAULT_FLAGS, tg=None):
+    """q,k,v [S,16,128] bf16 (q/k already normalized + scaled), proj [S,8224] bf16 (b at 8192:8208, a at 8208:8224),
+    state [1,16,128,128] fp32.  Returns y [S,16,128] bf16, new_state [1,16,128,128] fp32  (qwen35/gdn_nax.py:413-426)."""
+    _, _, _, ops, U, gC = _phase_a(proj, None, None, A_log, dt_bias, qkv=(q, k, v))
+    return phase_b(q, k, v, ops, U, gC, state)
+
+
 def phase_b(q, k, v, Tb, Am, gv, state, relaxed=True, flags=DEFAULT_FLAGS, tg=None):
     """The serial state recurrence on the outputs of phase A -> y [S,16,128] bf16, new state [1,16,128,128] f32
     (qwen35/gdn_nax.py:404-410).  Tb / Am / gv are the records prep_a (or gdn_chunked's phase A) produced."""

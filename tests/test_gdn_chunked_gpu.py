@@ -41,3 +41,75 @@ def test_phase_b_on_reference_records(qt, dev, T):
     check_rel("final state rel-L2", to_np(s1), os_, 2e-3, rel_l2)
     check_rel("final state max", to_np(s1), os_, 2e-3, rel_max)
     check_rel("y rel-L2", to_np(y), oy[0], 2e-3, rel_l2)
+
+
+def proj_inputs(seed, T, scale=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    cw, A_log, dtb, gw = layer_params(seed)
+    proj = rand_bf(gen, (T, PW), scale)
+    cs = rand_bf(gen, (3, CD))
+    S0 = (torch.randn((16, 128, 128), generator=gen) * 0.02).numpy()
+    return proj, cs, cw, A_log, dtb, gw, S0
+
+
+@pytest.mark.parametrize("T", [5, 64, 100])
+def test_phase_a_records_vs_float64(qt, dev, T):
+    """phase A's packed operands against the float64 chunk matrices (the fp16 operands carry 11 significant bits)"""
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(60 + T, T)
+    q, k, v, ops, U, gC = qt.gdn_nax.prep_a(to_dev(proj, dev, BF16), to_dev(cs, dev, BF16), to_dev(cw, dev, BF16), to_dev(A_log, dev),
+                                             to_dev(dtb, dev))
+    oq, ok, ov = O.conv_prep(proj, cs, cw)
+    check_equal("q", to_np(q), oq)                                            # bit-identical to conv_prep (tests/gdn_fuse.py:29-45)
+    check_equal("k", to_np(k), ok)
+    check_equal("v", to_np(v), ov)
+    lg = O.log_decay(proj[:, 8208:8224], A_log, dtb)
+    _, beta = O.gates(proj[:, 8208:8224], proj[:, 8192:8208], A_log, dtb)
+    raw, rops, rU, rgC = P.chunk_records(oq, ok, ov, lg, beta)
+    NC = (T + 63) // 64
+    gops = to_np(ops).reshape(NC, 16, 28672).astype(np.float64)
+    rops = rops.astype(np.float64)
+    names = (("Wn", 0, 8192), ("Qg", 8192, 16384), ("Kd", 16384, 24576), ("Am", 24576, 28672))
+    for name, lo, hi in names:
+        for c in range(NC):
+            for h in range(16):
+                ref = rops[c, h, lo:hi]
+                tol = 3e-3 * np.abs(ref).max() + 1.2e-7                    # + two fp16 subnormal steps (fast-decaying heads)
+                d = np.abs(gops[c, h, lo:hi] - ref).max()
+                if d > tol:
+                    raise AssertionError(f"{name} chunk {c} head {h}: max abs diff {d:.3e} (scale {np.abs(ref).max():.3e})")
+    check_rel("U", to_np(U).reshape(rU.shape), rU, 3e-3, rel_max)
+    check_rel("gamma_C", to_np(gC).reshape(rgC.shape), rgC, 1e-5, rel_max)
+
+
+@pytest.mark.parametrize("T", [5, 16, 37, 64, 65, 300])
+def test_chunked_prefill_vs_sequential_oracle(qt, dev, T):
+    """prep_a + phase_b + gated norm against the sequential restatement of the layer core (partial chunks as tests/gdn_fuse.py:29)"""
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(80 + T, T)
+    dproj = to_dev(proj, dev, BF16)
+    q, k, v, ops, U, gC = qt.gdn_nax.prep_a(dproj, to_dev(cs, dev, BF16), to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev))
+    y, s1 = qt.gdn_nax.phase_b(q, k, v, ops, U, gC, to_dev(S0[None], dev))
+    out = qt.prefill.gated_norm(y, dproj, to_dev(gw, dev))
+    oo, oy, otail, os_ = O.prefill_gdn(proj, cs, cw, A_log, dtb, S0, gw)
+    check_rel("final state rel-L2", to_np(s1)[0], os_, 2e-3, rel_l2)
+    check_rel("final state max", to_np(s1)[0], os_, 2e-3, rel_max)
+    check_rel("y rel-L2", to_np(y).reshape(T, 2048), oy, 2e-3, rel_l2)
+    check_rel("gated output rel-L2", to_np(out), oo, 2e-3, rel_l2)
+    # gdn_chunked (q, k, v given) is the same computation
+    y2, s2 = qt.gdn_nax.gdn_chunked(q, k, v, dproj, to_dev(A_log, dev), to_dev(dtb, dev), to_dev(S0[None], dev))
+    check_tensors_equal("gdn_chunked y", y2, y)
+    check_tensors_equal("gdn_chunked state", s2, s1)
+
+
+@pytest.mark.parametrize("T", [512, 2048])
+def test_config2_chunked_prefill(qt, dev, T):
+    """BASELINE config 2: B=1, chunk 64, nonzero initial state ~N(0,0.02) (prefix-cache resume), conv first, gated norm last"""
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(1002, T)
+    dproj = to_dev(proj, dev, BF16)
+    q, k, v, ops, U, gC = qt.gdn_nax.prep_a(dproj, to_dev(cs, dev, BF16), to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev))
+    y, s1 = qt.gdn_nax.phase_b(q, k, v, ops, U, gC, to_dev(S0[None], dev))
+    out = qt.prefill.gated_norm(y, dproj, to_dev(gw, dev))
+    oo, oy, otail, os_ = O.prefill_gdn(proj, cs, cw, A_log, dtb, S0, gw)
+    e1 = check_rel("final state rel-L2", to_np(s1)[0], os_, 2e-3, rel_l2)
+    e2 = check_rel("y rel-L2", to_np(y).reshape(T, 2048), oy, 2e-3, rel_l2)
+    e3 = check_rel("gated output rel-L2", to_np(out), oo, 2e-3, rel_l2)
+    print(f"T={T}: state {e1:.2e}, y {e2:.2e}, out {e3:.2e}")
