@@ -43,13 +43,56 @@ __device__ __forceinline__ half8 pack_half8(const f32x4& a, const f32x4& b) {
 }
 
 // Phase B: serial over the chunks.  grid = 128 wavefronts (head, dv slice); ops / U / gC are phase A's records.
-__global__ __launch_bounds__(64) void gdn_phase_b_kernel(const _Float16* __restrict__ ops, const float* __restrict__ U,
+constexpr int PF_AHEAD = 8;                     // chunks the L2 prefetch wavefront runs ahead of the MFMA wavefront
+
+__global__ __launch_bounds__(128) void gdn_phase_b_kernel(const _Float16* __restrict__ ops, const float* __restrict__ U,
                                                          const float* __restrict__ gC, const float* __restrict__ st_in,
                                                          float* __restrict__ st_out, bf16_t* __restrict__ y, int S, int NC) {
     // heads that share an XCD's L2 keep their 8 slices there: workgroup id = xcd + 8 k, head = xcd + 8 (k / 8), slice = k % 8
     const int xcd = blockIdx.x & 7, kq = blockIdx.x >> 3;
     const int h = xcd + 8 * (kq >> 3), sl = kq & 7;
-    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+
+    // Wavefront 0 runs the serial MFMA chain and touches global memory with loads only: on gfx9-family targets loads and
+    // stores share one in-order counter only as long as a single kind is in flight, so a store in the loop would force
+    // every wait down to zero outstanding loads and expose the full memory latency at every chunk.
+    // Wavefront 1 is its helper: it writes the finished output rows, which wavefront 0 hands over through two buffers in
+    // LDS, and it pulls the records of the coming chunks into this XCD's L2 (one dword per 128-byte line), PF_AHEAD chunks
+    // in front.  The hand-over is one bare s_barrier per chunk (no fence: only LDS is exchanged, and s_waitcnt lgkmcnt(0)
+    // orders it): after barrier c the helper reads buffer c & 1, and wavefront 0 next writes that buffer after barrier c+1.
+    __shared__ __align__(16) bf16_t y_s[2][C * 16];                           // one chunk of this slice's outputs, row major
+    if (threadIdx.x >= 64) {
+        unsigned sink = 0;
+        for (int c = 0; c < NC; c++) {
+            // touch the record of chunk c + PF_AHEAD; the values are only folded into `sink` after the hand-over below,
+            // so these loads never delay the barrier
+            unsigned pfv[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            const int pf = c + PF_AHEAD;
+            if (PF_AHEAD > 0 && pf < NC) {
+                const size_t rec = (size_t)pf * HV + h;
+                const unsigned* o32 = reinterpret_cast<const unsigned*>(ops + rec * OP_HALVES) + lane * 32;
+#pragma unroll
+                for (int i = 0; i < OP_HALVES * 2 / 8192; i++) pfv[i] = o32[i * 2048];
+                const unsigned* u32 = reinterpret_cast<const unsigned*>(U + rec * U_FLOATS + (size_t)sl * NCT * 256);
+                pfv[7] = u32[(lane & 31) * 32];
+            }
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            const uint4* src = reinterpret_cast<const uint4*>(&y_s[c & 1][lane * 16]);
+            const uint4 lo = src[0], hi = src[1];
+            const int t = c * C + lane;
+            if (t < S) {
+                uint4* dst = reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV + sl * 16);
+                dst[0] = lo;
+                dst[1] = hi;
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                  // the LDS reads are done before the next barrier
+#pragma unroll
+            for (int i = 0; i < 8; i++) sink ^= pfv[i];
+        }
+        if (sink == 0x9e3779b9u && S < 0) st_out[0] = 0.f;                      // keeps the prefetch loads alive; never true
+        return;
+    }
 
     f32x4 ST[8];
     {
@@ -57,48 +100,102 @@ __global__ __launch_bounds__(64) void gdn_phase_b_kernel(const _Float16* __restr
 #pragma unroll
         for (int mt = 0; mt < 8; mt++) ST[mt] = *reinterpret_cast<const f32x4*>(sp + mt * 16 + 4 * g);
     }
+    // Operand FIFO, one chunk deep: tile i of chunk c+1 is loaded into the registers of tile i of chunk c right after the
+    // MFMA that consumed it, so a whole chunk step of MFMA work covers the latency of every load.
+    half8 Wt[16], Qt[16], Kt[16], At[8];
+    f32x4 Ut[NCT];
+    float gc;
+    {
+        const half8* op = reinterpret_cast<const half8*>(ops + (size_t)h * OP_HALVES) + lane;
+        const f32x4* up = reinterpret_cast<const f32x4*>(U + (size_t)h * U_FLOATS + (size_t)sl * NCT * 256) + lane;
+        // same issue order as inside the loop
+#pragma unroll
+        for (int ct = 0; ct < NCT; ct++) Ut[ct] = up[ct * 64];
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) Wt[ct * 4 + kb] = op[(OP_W / 8) + (ct * 4 + kb) * 64];
+        gc = gC[h];
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; kb2++)
+#pragma unroll
+            for (int mt = 0; mt < 8; mt++) Kt[mt * 2 + kb2] = op[(OP_K / 8) + (mt * 2 + kb2) * 64];
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) Qt[ct * 4 + kb] = op[(OP_Q / 8) + (ct * 4 + kb) * 64];
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; kb2++)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) At[ct * 2 + kb2] = op[(OP_A / 8) + (ct * 2 + kb2) * 64];
+    }
+    __builtin_amdgcn_sched_barrier(0);
     for (int c = 0; c < NC; c++) {
-        const size_t rec = (size_t)c * HV + h;
-        const half8* op = reinterpret_cast<const half8*>(ops + rec * OP_HALVES) + lane;
-        const f32x4* up = reinterpret_cast<const f32x4*>(U + rec * U_FLOATS + (size_t)sl * NCT * 256) + lane;
-        const float gc = gC[rec];
+        const int cn = c + 1 < NC ? c + 1 : c;                                  // the last step re-reads its own record
+        const size_t recn = (size_t)cn * HV + h;
+        const half8* op = reinterpret_cast<const half8*>(ops + recn * OP_HALVES) + lane;
+        const f32x4* up = reinterpret_cast<const f32x4*>(U + recn * U_FLOATS + (size_t)sl * NCT * 256) + lane;
 
         half8 Sb[4];
 #pragma unroll
         for (int kb = 0; kb < 4; kb++) Sb[kb] = pack_half8(ST[2 * kb], ST[2 * kb + 1]);
 
+        // Every MFMA is followed by the load that refills its operand registers for the next chunk, and the scheduler is
+        // pinned to this order: loads then complete in the order in which the next chunk consumes them, so the waits stay
+        // partial (a reordered load would force a wait for all 60).  Independent accumulators alternate (ct / mt inner).
         f32x4 D[NCT], Y[NCT];
 #pragma unroll
         for (int ct = 0; ct < NCT; ct++) {
-            D[ct] = up[ct * 64];
+            D[ct] = Ut[ct];
+            Ut[ct] = up[ct * 64];
             Y[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int kb = 0; kb < 4; kb++) {
-                D[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[(OP_W / 8) + (ct * 4 + kb) * 64], Sb[kb], D[ct], 0, 0, 0);
-                Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[(OP_Q / 8) + (ct * 4 + kb) * 64], Sb[kb], Y[ct], 0, 0, 0);
-            }
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) {
+                D[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Wt[ct * 4 + kb], Sb[kb], D[ct], 0, 0, 0);
+                Wt[ct * 4 + kb] = op[(OP_W / 8) + (ct * 4 + kb) * 64];
+            }
         half8 Db[2];
         Db[0] = pack_half8(D[0], D[1]);
         Db[1] = pack_half8(D[2], D[3]);
 #pragma unroll
-        for (int mt = 0; mt < 8; mt++) {
-            ST[mt] *= gc;
+        for (int mt = 0; mt < 8; mt++) ST[mt] *= gc;
+        gc = gC[recn];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int kb2 = 0; kb2 < 2; kb2++)
-                ST[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[(OP_K / 8) + (mt * 2 + kb2) * 64], Db[kb2], ST[mt], 0, 0, 0);
-        }
+        for (int kb2 = 0; kb2 < 2; kb2++)
 #pragma unroll
-        for (int ct = 0; ct < NCT; ct++) {
-#pragma unroll
-            for (int kb2 = 0; kb2 < 2; kb2++)
-                Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[(OP_A / 8) + (ct * 2 + kb2) * 64], Db[kb2], Y[ct], 0, 0, 0);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int t = c * C + ct * 16 + 4 * g + r;
-                if (t < S) y[((size_t)t * HV + h) * DV + sl * 16 + n] = f2bf(Y[ct][r]);
+            for (int mt = 0; mt < 8; mt++) {
+                ST[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Kt[mt * 2 + kb2], Db[kb2], ST[mt], 0, 0, 0);
+                Kt[mt * 2 + kb2] = op[(OP_K / 8) + (mt * 2 + kb2) * 64];
             }
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) {
+                Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Qt[ct * 4 + kb], Sb[kb], Y[ct], 0, 0, 0);
+                Qt[ct * 4 + kb] = op[(OP_Q / 8) + (ct * 4 + kb) * 64];
+            }
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; kb2++)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) {
+                Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(At[ct * 2 + kb2], Db[kb2], Y[ct], 0, 0, 0);
+                At[ct * 2 + kb2] = op[(OP_A / 8) + (ct * 2 + kb2) * 64];
+            }
+        // hand the chunk's outputs to the helper wavefront
+        {
+            bf16_t* ys = y_s[c & 1];
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) ys[(ct * 16 + 4 * g + r) * 16 + n] = f2bf(Y[ct][r]);
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                      // the LDS writes have landed
+        __builtin_amdgcn_s_barrier();
     }
     {
         float* sp = st_out + ((size_t)h * DV + sl * 16 + n) * DK;
@@ -456,7 +553,7 @@ int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, const float
     for (const void* p : {ops, (const void*)U, (const void*)state_in, (const void*)state_out})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     const int NC = (S + C - 1) / C;
-    hipLaunchKernelGGL(gdn_phase_b_kernel, dim3(HV * 8), dim3(64), 0, stream, (const _Float16*)ops, U, gC, state_in, state_out,
+    hipLaunchKernelGGL(gdn_phase_b_kernel, dim3(HV * 8), dim3(128), 0, stream, (const _Float16*)ops, U, gC, state_in, state_out,
                        (bf16_t*)y, S, NC);
     QT_CHECK_LAUNCH();
     return QT_OK;
