@@ -77,6 +77,28 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
                        const int32_t* pos, void* out, void* workspace, long workspace_bytes, int B, int M, int Lmax,
                        int n_slots, int CH, qt_stream_t stream);
 
+/* Chunked (chunk = 64) GatedDeltaNet prefill, two phases (qwen35/gdn_nax.py:394-426: prep_a / gdn_chunked's phase A, phase_b).
+ * Phase A is parallel over (chunk, head): conv + SiLU + q/k norm (or, with from_qkv != 0, q / k / v [S,16,128] bf16 given),
+ * gates, K K^T / Q K^T on bf16 MFMA, the 64 x 64 unit-lower-triangular inverse in fp32, and the state-independent MFMA
+ * operands of phase B.  It fills three caller-owned buffers of qt_gdn_chunk_{ops,u,gc}_bytes(S) bytes: `ops` (half-precision
+ * operand tiles), `U` and `gC` (f32).  q, k, v may be null (not written) when from_qkv == 0.
+ * Phase B is serial over the chunks: state_in / state_out [16,128,128] f32, y [S,16,128] bf16. */
+long qt_gdn_chunk_ops_bytes(int S);
+long qt_gdn_chunk_u_bytes(int S);
+long qt_gdn_chunk_gc_bytes(int S);
+int qt_gdn_phase_a(const void* proj, const void* conv_state, const void* conv_w, const float* A_log, const float* dt_bias,
+                   void* q, void* k, void* v, int from_qkv, void* ops, float* U, float* gC, int S, qt_stream_t stream);
+int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, const float* state_in, float* state_out, void* y, int S,
+                   qt_stream_t stream);
+
+/* Causal prefill attention: the mx.fast.scaled_dot_product_attention(..., mask="causal") call of the full-attention layers
+ * (qwen35/model.py:160-167, qwen35/prefill.py:468).  q, out [8][S][256] bf16 with head stride q_head_stride (elements);
+ * K, V [2][>=L][256] bf16 with head stride kv_head_stride; query i sits at position q_pos0 + i and sees keys 0..q_pos0+i.
+ * workspace: qt_gqa_prefill_workspace_bytes(L) bytes (a transposed copy of V), 16-byte aligned. */
+long qt_gqa_prefill_workspace_bytes(int L);
+int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out, void* workspace, long workspace_bytes, int S,
+                          int L, int q_pos0, long q_head_stride, long kv_head_stride, qt_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

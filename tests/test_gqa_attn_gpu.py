@@ -120,3 +120,34 @@ def test_attn_b_config4_verify_mix(qt, dev):
     pos = rng.integers(1024, 8192, B).astype(np.int32)
     slots = rng.permutation(B).astype(np.int32)
     run_case(qt, dev, rng, B, Lmax, slots, pos, M)
+
+
+# ------------------------------------------------------------------------------------- causal prefill attention
+@pytest.mark.parametrize("S,L", [(1, 1), (5, 5), (64, 64), (100, 100), (37, 200), (300, 300), (128, 1000)])
+def test_prefill_causal_vs_oracle(qt, dev, S, L):
+    """softmax(Q K^T / 16 + causal) V, GQA 8/2, D=256 (model.py:160-167); with L > S the queries are the last S positions"""
+    rng = np.random.default_rng(S * 1000 + L)
+    q = bf(rng.standard_normal((8, S, 256)))
+    K = bf(rng.standard_normal((2, L + 7, 256)))
+    V = bf(rng.standard_normal((2, L + 7, 256)))
+    dK, dV = to_dev(K, dev, BF16)[None], to_dev(V, dev, BF16)[None]
+    o = qt.attention.scaled_dot_product_attention(to_dev(q, dev, BF16)[None], dK[:, :, :L], dV[:, :, :L], scale=256 ** -0.5, mask="causal")
+    ref = O.sdpa_causal(q, K[:, :L], V[:, :L])
+    check_attn(f"S={S} L={L}", to_np(o)[0], ref)
+
+
+def test_prefill_causal_2048(qt, dev):
+    rng = np.random.default_rng(2048)
+    S = 2048
+    q = bf(rng.standard_normal((8, S, 256)))
+    K = bf(rng.standard_normal((2, S, 256)))
+    V = bf(rng.standard_normal((2, S, 256)))
+    o = to_np(qt.attention.scaled_dot_product_attention(to_dev(q, dev, BF16)[None], to_dev(K, dev, BF16)[None], to_dev(V, dev, BF16)[None],
+                                                        scale=256 ** -0.5, mask="causal"))[0]
+    ref = O.sdpa_causal(q, K, V)
+    check_attn("S=2048", o, ref)
+    # the first row sees one key: o = v
+    check_equal("row 0 == v[0]", o[:, 0], np.repeat(V[:, 0], 4, axis=0))
+    with pytest.raises(ValueError):
+        qt.attention.scaled_dot_product_attention(to_dev(q, dev, BF16)[None], to_dev(K, dev, BF16)[None], to_dev(V, dev, BF16)[None],
+                                                  scale=256 ** -0.5, mask=None)
