@@ -98,6 +98,113 @@ def time_decode(torch, qt, st, B, n_layers, steps, warmup, use_graph=True):
     return wall, e0.elapsed_time(e1) * 1e-3
 
 
+def time_graph(torch, fn, reps=200, inner=10):
+    """average device time (s) of fn(), measured with events around replays of a HIP graph holding `inner` calls"""
+    fn()
+    torch.cuda.synchronize()
+    st = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        with torch.cuda.graph(g, stream=st):
+            for _ in range(inner):
+                fn()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        g.replay()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n = max(1, reps // inner)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(n):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / (n * inner)
+
+
+MFMA_PEAK_TFLOPS = 2500.0
+GDN_FLOP_PER_TOKEN = 2621440.0        # 16 heads x (4 C^2 dk + 4 C^2 dv + 6 C dk dv) / C at C = 64, dk = dv = 128
+
+
+def bench_prefill(torch, qt, dev, T, seed=1002):
+    """BASELINE config 2: conv + chunked GDN (chunk 64) + gated RMSNorm over T tokens from a nonzero state"""
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    proj = torch.randn((T, PW), generator=g).to(bf).to(dev)
+    cs = torch.randn((1, 3, CD), generator=g).to(bf).to(dev)
+    cw = (torch.randn((CD, 4), generator=g) * 0.5).to(bf).to(dev)
+    A = (torch.rand(HV, generator=g) * 2.7).to(dev)
+    dtb = (torch.randn(HV, generator=g) * 0.1).to(dev)
+    gw = torch.ones(DV, device=dev)
+    S0 = (torch.randn((1, HV, DV, DK), generator=g) * 0.02).to(dev)
+    q, k, v, ops, U, gC = qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb, want_qkv=False)
+    y, _ = qt.gdn_nax.phase_b(proj, None, None, ops, U, gC, S0)
+    t_all = time_graph(torch, lambda: qt.prefill.gdn_core(proj, cs, S0, cw, A, dtb, gw), reps=60, inner=3)
+    t_a = time_graph(torch, lambda: qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb, want_qkv=False), reps=60, inner=3)
+    t_b = time_graph(torch, lambda: qt.gdn_nax.phase_b(proj, None, None, ops, U, gC, S0), reps=60, inner=3)
+    t_n = time_graph(torch, lambda: qt.prefill.gated_norm(y, proj, gw), reps=60, inner=3)
+    flop = GDN_FLOP_PER_TOKEN * T
+    hbm = T * PW * 2 + T * 2048 * 2 + 2 * HV * DV * DK * 4          # compulsory: projection rows in, gated output out, state in + out
+    return {"T": T, "tok_per_s": T / t_all, "us": t_all * 1e6, "phase_a_us": t_a * 1e6, "phase_b_us": t_b * 1e6,
+            "gated_norm_us": t_n * 1e6, "mfma_tflops": flop / t_all / 1e12, "mfma_frac": flop / t_all / 1e12 / MFMA_PEAK_TFLOPS,
+            "compulsory_hbm_GBps": hbm / t_all / 1e9}
+
+
+def bench_verify_gdn(torch, qt, dev, B=16, M=4, seed=1004):
+    """BASELINE config 4, GDN half: B sequences x M draft tokens, a state snapshot after every token"""
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    pools = [((torch.randn((B + 1, M, HV, DV, DK), generator=g) * 0.02).to(dev), torch.randn(((B + 1) * 2, M, 3, CD), generator=g).to(bf).to(dev))
+             for _ in range(N_LAYERS)]
+    proj = torch.randn((B * M, PW), generator=g).to(bf).to(dev)
+    cw = (torch.randn((CD, 4), generator=g) * 0.5).to(bf).to(dev)
+    A = (torch.rand(HV, generator=g) * 2.7).to(dev)
+    dtb = (torch.randn(HV, generator=g) * 0.1).to(dev)
+    ss = torch.randperm(B, generator=g).to(torch.int32).to(dev)
+    sels = torch.randint(0, M, (B,), generator=g).to(torch.int32).to(dev)
+    pars = torch.zeros(B, dtype=torch.int32, device=dev)
+    it = [0]
+
+    def step():
+        ssm, conv = pools[it[0] % N_LAYERS]
+        it[0] += 1
+        qt.batch_spec.deltanet_bm(proj, conv, cw, A, dtb, ssm, ss, sels, pars, M)
+    t = time_graph(torch, step, reps=N_LAYERS * 20, inner=N_LAYERS)
+    nbytes = B * ((1 + M) * HV * DV * DK * 4 + M * PW * 2 + 3 * CD * 2 + M * 3 * CD * 2 + M * 2048 * 2)
+    return {"B": B, "M": M, "us": t * 1e6, "bytes": nbytes, "GBps": nbytes / t / 1e9, "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
+
+
+def bench_attn(torch, qt, dev, B, M, lo, hi, seed):
+    """BASELINE configs 3 / 4 (attention half): ragged KV lengths uniform in [lo, hi], M query rows per sequence"""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    Lmax = hi + 8
+    pos = torch.from_numpy(rng.integers(lo, hi, B).astype(np.int32)).to(dev)
+    slots = torch.from_numpy(rng.permutation(B).astype(np.int32)).to(dev)
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    Kp = torch.randn((B + 1, 2, Lmax, 256), generator=g).to(bf).to(dev)
+    Vp = torch.randn((B + 1, 2, Lmax, 256), generator=g).to(bf).to(dev)
+    q = torch.randn((B * M, 8, 256), generator=g).to(bf).to(dev)
+    kn = torch.randn((B * M, 2, 256), generator=g).to(bf).to(dev)
+    vn = torch.randn((B * M, 2, 256), generator=g).to(bf).to(dev)
+    t = time_graph(torch, lambda: qt.batch.attn_b(q, kn, vn, Kp, Vp, slots, pos, M), reps=100, inner=5)
+    nbytes = int(pos.sum().item()) * 2 * 2 * 256 * 2                  # K and V rows of both KV heads, read once
+    return {"B": B, "M": M, "sum_L": int(pos.sum().item()), "us": t * 1e6, "bytes": nbytes, "GBps": nbytes / t / 1e9,
+            "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
+
+
+def bench_attn_prefill(torch, qt, dev, S=2048, seed=7):
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    q = torch.randn((1, 8, S, 256), generator=g).to(bf).to(dev)
+    K = torch.randn((1, 2, S, 256), generator=g).to(bf).to(dev)
+    V = torch.randn((1, 2, S, 256), generator=g).to(bf).to(dev)
+    t = time_graph(torch, lambda: qt.attention.scaled_dot_product_attention(q, K, V, scale=256 ** -0.5, mask="causal"), reps=40, inner=2)
+    flop = 4.0 * S * S * 256 * 8 / 2
+    return {"S": S, "us": t * 1e6, "tflops": flop / t / 1e12, "mfma_frac": flop / t / 1e12 / MFMA_PEAK_TFLOPS}
+
+
 def cpu_baseline(B, budget_s=12.0):
     """The C restatement of the decode step (float accumulation) timed on this host's cores: a reported baseline only."""
     import numpy as np
@@ -126,6 +233,50 @@ def cpu_baseline(B, budget_s=12.0):
                       f"float accumulation, OpenMP over (row, head), {el:.1f} s"}
 
 
+def profile_leg(torch, qt, dev, args):
+    """Runs one leg eagerly a few times so that rocprofv3 (--kernel-trace --stats, or --pmc) sees a short, clean trace."""
+    leg, n = args.only, max(1, min(args.steps, 72))
+    if leg == "decode":
+        st = build_decode_state(torch, dev, args.batch, N_LAYERS)
+        for i in range(n):
+            l = i % N_LAYERS
+            qt.batch.deltanet_b(st["proj"][l & 3], st["conv"][l], st["cw"][l], st["A_log"][l], st["dtb"][l], st["ssm"][l], st["slots"],
+                                st["pos"][(i // N_LAYERS) & 1])
+    elif leg == "copy":
+        # plain copy of known size: the scale factor for the FETCH_SIZE / WRITE_SIZE counters (64 MiB read + 64 MiB written)
+        src = [torch.randn(16 * 1024 * 1024, device=dev) for _ in range(N_LAYERS)]
+        dst = [torch.empty_like(src[0]) for _ in range(2)]
+        for i in range(n):
+            dst[i & 1].copy_(src[i % N_LAYERS])
+    elif leg == "prefill":
+        for _ in range(3):
+            bench_prefill_once(torch, qt, dev, 2048)
+    elif leg == "verify":
+        bench_verify_gdn(torch, qt, dev)
+    elif leg == "attn_decode":
+        bench_attn(torch, qt, dev, 16, 1, 512, 32768, 1003)
+    elif leg == "attn_verify":
+        bench_attn(torch, qt, dev, 16, 4, 1024, 8192, 1004)
+    elif leg == "attn_prefill":
+        bench_attn_prefill(torch, qt, dev)
+    else:
+        raise SystemExit(f"unknown leg {leg}")
+    torch.cuda.synchronize()
+    print(json.dumps({"profiled": leg, "launches": n}))
+
+
+def bench_prefill_once(torch, qt, dev, T, seed=1002):
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    proj = torch.randn((T, PW), generator=g).to(bf).to(dev)
+    cs = torch.randn((1, 3, CD), generator=g).to(bf).to(dev)
+    cw = (torch.randn((CD, 4), generator=g) * 0.5).to(bf).to(dev)
+    A, dtb = (torch.rand(HV, generator=g) * 2.7).to(dev), (torch.randn(HV, generator=g) * 0.1).to(dev)
+    S0 = (torch.randn((1, HV, DV, DK), generator=g) * 0.02).to(dev)
+    for _ in range(5):
+        qt.prefill.gdn_core(proj, cs, S0, cw, A, dtb, torch.ones(DV, device=dev))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,6 +286,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every step eagerly instead of replaying HIP graphs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the B sweep and the single-pool run")
+    ap.add_argument("--only", default="", help="profile helper: run only one leg a few times and exit "
+                                               "(decode | copy | prefill | verify | attn_decode | attn_verify | attn_prefill)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every work item of the path is an independent (slot, head) pair; "
@@ -147,6 +300,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B = args.batch
+
+    if args.only:
+        return profile_leg(torch, qt, dev, args)
 
     st = build_decode_state(torch, dev, B, N_LAYERS)
     wall, dev_s = time_decode(torch, qt, st, B, N_LAYERS, args.steps, args.warmup, use_graph=not args.no_graph)
@@ -169,6 +325,13 @@ def main():
             extras[f"B{b}"] = {"steps_per_s": args.steps / wb, "us_per_step": db / args.steps * 1e6,
                                "GBps": decode_bytes(b) / (db / args.steps) / 1e9}
             del stb
+        torch.cuda.empty_cache()
+        extras["gdn_prefill"] = [bench_prefill(torch, qt, dev, T) for T in (512, 2048, 8192)]
+        extras["gdn_verify"] = bench_verify_gdn(torch, qt, dev)
+        extras["attn_decode_config3"] = bench_attn(torch, qt, dev, 16, 1, 512, 32768, 1003)
+        torch.cuda.empty_cache()
+        extras["attn_verify_config4"] = bench_attn(torch, qt, dev, 16, 4, 1024, 8192, 1004)
+        extras["attn_prefill_causal"] = bench_attn_prefill(torch, qt, dev)
 
     out = {
         "metric": "GDN decode steps/s @B=64 (% HBM peak); GDN prefill tok/s @2048 (% MFMA)",
@@ -183,6 +346,13 @@ def main():
                      "avg_launch_us": launch_s * 1e6},
         "extras": extras,
     }
+    if "gdn_prefill" in extras:
+        p2k = extras["gdn_prefill"][1]
+        out["secondary"] = {"metric": "GDN prefill tok/s @2048 (% MFMA)", "value": p2k["tok_per_s"], "unit": "tok/s",
+                            "config": {"workload": "configs[2]: conv + chunked GDN (chunk 64) + gated RMSNorm, B=1, T=2048, 16 heads, "
+                                                   "nonzero initial state"},
+                            "roofline": {"bound": "mfma", "achieved": p2k["mfma_tflops"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                         "frac": p2k["mfma_frac"], "traffic": None}}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B)
     print(json.dumps(out))
