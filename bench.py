@@ -137,10 +137,10 @@ def bench_prefill(torch, qt, dev, T, seed=1002):
     dtb = (torch.randn(HV, generator=g) * 0.1).to(dev)
     gw = torch.ones(DV, device=dev)
     S0 = (torch.randn((1, HV, DV, DK), generator=g) * 0.02).to(dev)
-    q, k, v, ops, U, gC = qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb, want_qkv=False)
+    q, k, v, ops, U, gC = qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb)
     y, _ = qt.gdn_nax.phase_b(proj, None, None, ops, U, gC, S0)
     t_all = time_graph(torch, lambda: qt.prefill.gdn_core(proj, cs, S0, cw, A, dtb, gw), reps=60, inner=3)
-    t_a = time_graph(torch, lambda: qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb, want_qkv=False), reps=60, inner=3)
+    t_a = time_graph(torch, lambda: qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb), reps=60, inner=3)
     t_b = time_graph(torch, lambda: qt.gdn_nax.phase_b(proj, None, None, ops, U, gC, S0), reps=60, inner=3)
     t_n = time_graph(torch, lambda: qt.prefill.gated_norm(y, proj, gw), reps=60, inner=3)
     flop = GDN_FLOP_PER_TOKEN * T

@@ -54,9 +54,13 @@ int qt_gdn_gates(const void* a, const void* b, long a_stride, long b_stride, con
 /* normalize_qk (qwen35/gated_delta.py:21-30) on `rows` rows of dk = 128 bf16 values. */
 int qt_normalize_qk(const void* q, const void* k, void* q_out, void* k_out, long rows, int dk, qt_stream_t stream);
 
-/* prefill.conv_prep (qwen35/prefill.py:228-238): proj [S,8224], conv_state [3,6144] -> q, k, v [S,16,128] bf16. */
-int qt_gdn_conv_prep(const void* proj, const void* conv_state, const void* conv_w, void* q, void* k, void* v, int S,
-                     qt_stream_t stream);
+/* prefill.conv_prep (qwen35/prefill.py:228-238): proj [S,8224], conv_state [3,6144] -> q, k, v [S,16,128] bf16.
+ * silu_table: the qt_silu_table_bytes() byte table written once by qt_silu_table_build (the bf16 -> bf16 map of
+ * mslib.py:21-22 on 2^-9 <= |x| < 2^5), owned by the caller; null = every workgroup computes its own copy. */
+int qt_silu_table_bytes(void);
+int qt_silu_table_build(void* table, qt_stream_t stream);
+int qt_gdn_conv_prep(const void* proj, const void* conv_state, const void* conv_w, const void* silu_table, void* q, void* k,
+                     void* v, int S, qt_stream_t stream);
 
 /* batch.gnorm_rows / prefill.gated_norm (qwen35/batch.py:338-343, qwen35/prefill.py:241-244): y [rows,2048] bf16,
  * z = proj[:,6144:8192] of proj [rows,8224], gw [128] f32 -> out [rows,2048] bf16. */
@@ -78,16 +82,16 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
                        int n_slots, int CH, qt_stream_t stream);
 
 /* Chunked (chunk = 64) GatedDeltaNet prefill, two phases (qwen35/gdn_nax.py:394-426: prep_a / gdn_chunked's phase A, phase_b).
- * Phase A is parallel over (chunk, head): conv + SiLU + q/k norm (or, with from_qkv != 0, q / k / v [S,16,128] bf16 given),
- * gates, K K^T / Q K^T on bf16 MFMA, the 64 x 64 unit-lower-triangular inverse in fp32, and the state-independent MFMA
- * operands of phase B.  It fills three caller-owned buffers of qt_gdn_chunk_{ops,u,gc}_bytes(S) bytes: `ops` (half-precision
- * operand tiles), `U` and `gC` (f32).  q, k, v may be null (not written) when from_qkv == 0.
+ * Phase A is parallel over (chunk, head): it takes q, k, v [S,16,128] bf16 (qt_gdn_conv_prep's outputs) and the gate inputs in
+ * proj [S,8224], and computes the gates, K K^T / Q K^T on bf16 MFMA, the 64 x 64 unit-lower-triangular inverse in fp32 and the
+ * state-independent MFMA operands of phase B.  It fills three caller-owned buffers of qt_gdn_chunk_{ops,u,gc}_bytes(S) bytes:
+ * `ops` (half-precision operand tiles), `U` and `gC` (f32).
  * Phase B is serial over the chunks: state_in / state_out [16,128,128] f32, y [S,16,128] bf16. */
 long qt_gdn_chunk_ops_bytes(int S);
 long qt_gdn_chunk_u_bytes(int S);
 long qt_gdn_chunk_gc_bytes(int S);
-int qt_gdn_phase_a(const void* proj, const void* conv_state, const void* conv_w, const float* A_log, const float* dt_bias,
-                   void* q, void* k, void* v, int from_qkv, void* ops, float* U, float* gC, int S, qt_stream_t stream);
+int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v, const float* A_log, const float* dt_bias,
+                   void* ops, float* U, float* gC, int S, qt_stream_t stream);
 int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, const float* state_in, float* state_out, void* y, int S,
                    qt_stream_t stream);
 

@@ -22,13 +22,14 @@ _SIGS = {
     "qt_gdn_deltanet": [_vp] * 10 + [_i, _i, _i, _vp],
     "qt_gdn_gates": [_vp, _vp, _l, _l, _vp, _vp, _vp, _vp, _vp, _l, _i, _vp],
     "qt_normalize_qk": [_vp, _vp, _vp, _vp, _l, _i, _vp],
-    "qt_gdn_conv_prep": [_vp] * 6 + [_i, _vp],
+    "qt_gdn_conv_prep": [_vp] * 7 + [_i, _vp],
+    "qt_silu_table_build": [_vp, _vp],
     "qt_gated_rmsnorm": [_vp, _vp, _vp, _vp, _l, _f, _vp],
     "qt_gdn_recurrent": [_vp] * 8 + [_i] * 6 + [_vp],
     "qt_gqa_attn_decode": [_vp] * 9 + [_l, _i, _i, _i, _i, _i, _vp],
     "qt_gdn_phase_b": [_vp] * 6 + [_i, _vp],
     "qt_gqa_prefill_causal": [_vp] * 5 + [_l, _i, _i, _i, _l, _l, _vp],
-    "qt_gdn_phase_a": [_vp] * 8 + [_i, _vp, _vp, _vp, _i, _vp],
+    "qt_gdn_phase_a": [_vp] * 9 + [_i, _vp],
 }
 
 
@@ -61,6 +62,19 @@ def call(name, *args):
     rc = getattr(lib(), name)(*args)
     if rc != 0:
         raise RuntimeError(f"{name} failed: {ERRORS.get(rc, rc)}")
+
+
+_SILU_TABLES = {}
+
+
+def silu_table(dev):
+    """The 7 KiB silu_bf16 table of `dev` (built once per device by the library, owned here: the C ABI keeps no state)."""
+    t = _SILU_TABLES.get(dev)
+    if t is None:
+        t = torch.empty(lib().qt_silu_table_bytes() // 2, dtype=torch.bfloat16, device=dev)
+        call("qt_silu_table_build", ptr(t), stream())
+        _SILU_TABLES[dev] = t
+    return t
 
 
 def stream():

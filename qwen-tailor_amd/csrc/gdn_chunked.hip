@@ -213,10 +213,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int QS_LD = DK + 8;        // row strides (elements) of the LDS tiles: keep 16-byte alignment, spread the banks
 constexpr int KT_LD = C + 8;
 constexpr int LS_LD = C + 4;
-constexpr int TAB_LO = 118, TAB_N = 14 * 128;      // silu table: bf16 exponent fields 118..131, i.e. 2^-9 <= |x| < 2^5
 
 struct PhaseALds {
-    bf16_t tab[2 * TAB_N];
     __align__(16) bf16_t Qs[C * QS_LD];
     __align__(16) bf16_t Ks[C * QS_LD];
     __align__(16) bf16_t KT[DK * KT_LD];
@@ -226,35 +224,20 @@ struct PhaseALds {
     float Lc[C], beta[C], gam[C], dec[C];
 };
 
-// silu_bf16 of a bf16 value through the table; outside the table's range the closed forms / the direct evaluation
-__device__ __forceinline__ float silu_lookup(const bf16_t* tab, bf16_t xb) {
-    const unsigned e = (xb >> 7) & 0xffu;
-    if (e < (unsigned)TAB_LO) return BF(bf2f(xb) * 0.5f);            // exp(|x|) rounds to 1: sigmoid_bf16 = 0.5 exactly
-    if (__builtin_expect(e > (unsigned)(TAB_LO + 13), 0)) return silu_bf16(bf2f(xb));
-    return bf2f(tab[(xb >> 15) * TAB_N + (xb & 0x7fffu) - TAB_LO * 128]);
-}
-
 __device__ __forceinline__ half8 to_half8(const float (&v)[8]) {
     half8 h;
 #pragma unroll
     for (int j = 0; j < 8; j++) h[j] = (_Float16)v[j];
     return h;
 }
-__device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]) {
-    f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
-    f[4] = lo_bf(w.z); f[5] = hi_bf(w.z); f[6] = lo_bf(w.w); f[7] = hi_bf(w.w);
-}
 __device__ __forceinline__ void unpack4(uint2 w, float* f) {
     f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
 }
 
-// proj [S,8224], cs [3,6144], cw [6144*4] -> q, k, v [S,16,128] (optional) and the phase B records.
-// FROM_QKV: q, k, v are inputs (already convolved and normalized, gdn_nax.gdn_chunked) and the conv is skipped.
-template <bool FROM_QKV>
-__global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs,
-                                                          const bf16_t* __restrict__ cw, const float* __restrict__ A_log,
-                                                          const float* __restrict__ dt_bias, bf16_t* __restrict__ qo,
-                                                          bf16_t* __restrict__ ko, bf16_t* __restrict__ vo,
+// q, k, v [S,16,128] bf16 (convolved, normalized: conv_prep's outputs), proj [S,8224] (gate inputs a, b) -> phase B records
+__global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ qi,
+                                                          const bf16_t* __restrict__ ki, const bf16_t* __restrict__ vi,
+                                                          const float* __restrict__ A_log, const float* __restrict__ dt_bias,
                                                           _Float16* __restrict__ ops, float* __restrict__ U,
                                                           float* __restrict__ gC, int S) {
     __shared__ PhaseALds L;
@@ -263,13 +246,22 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
     const size_t rec = (size_t)c * HV + h;
     _Float16* op = ops + rec * OP_HALVES;
 
-    // ---- silu table, zero the blocks of T above the diagonal
-    for (int i = tid; i < 2 * TAB_N; i += 256) {
-        const int sgn = i / TAB_N, em = i % TAB_N;
-        const bf16_t xb = (bf16_t)((sgn << 15) | (TAB_LO * 128 + em));
-        L.tab[i] = f2bf(silu_bf16(bf2f(xb)));
+    // ---- the chunk's q, k, v rows: every load is issued before anything else (a 16-lane group owns a token per round,
+    // a lane 8 consecutive columns); rows past the end are zero (gdn_nax.py:172-174)
+    uint4 raw[4][3];
+    {
+        const int gi = tid >> 4, cc = tid & 15;
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            const int t = t0 + rr * 16 + gi;
+            const size_t o = ((size_t)min(t, S - 1) * HV + h) * DK + cc * 8;
+            raw[rr][0] = *reinterpret_cast<const uint4*>(qi + o);
+            raw[rr][1] = *reinterpret_cast<const uint4*>(ki + o);
+            raw[rr][2] = *reinterpret_cast<const uint4*>(vi + o);
+            if (t >= S) raw[rr][0] = raw[rr][1] = raw[rr][2] = make_uint4(0, 0, 0, 0);
+        }
     }
-    for (int i = tid; i < C * LS_LD; i += 256) L.Ts[i] = 0.f;
+    for (int i = tid; i < C * LS_LD; i += 256) L.Ts[i] = 0.f;                   // blocks of T above the diagonal stay zero
 
     // ---- gates of the chunk's tokens (gdn_nax.py:80-104): wave 0, one token per lane
     if (w == 0) {
@@ -292,89 +284,21 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
         L.dec[lane] = expf(tot - lc);
         if (lane == 63) gC[rec] = expf(lc);
     }
-    __syncthreads();
-
-    // ---- conv + silu + q/k norm (kernels.py:476-510): a 16-lane group owns one token, a lane 8 channels of q, k and v
     {
         const int gi = tid >> 4, cc = tid & 15;
-        const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
+#pragma unroll
         for (int rr = 0; rr < 4; rr++) {
-            const int tl = rr * 16 + gi, t = t0 + tl;
-            float u[3][8];
-            if (FROM_QKV) {
-                if (t < S) {
-                    const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
-                    unpack8(*reinterpret_cast<const uint4*>(qo + o), u[0]);
-                    unpack8(*reinterpret_cast<const uint4*>(ko + o), u[1]);
-                    unpack8(*reinterpret_cast<const uint4*>(vo + o), u[2]);
-                } else {
+            const int tl = rr * 16 + gi;
+            *reinterpret_cast<uint4*>(&L.Qs[tl * QS_LD + cc * 8]) = raw[rr][0];
+            *reinterpret_cast<uint4*>(&L.Ks[tl * QS_LD + cc * 8]) = raw[rr][1];
+            const uint32_t kw[4] = {raw[rr][1].x, raw[rr][1].y, raw[rr][1].z, raw[rr][1].w};
+            const uint32_t vw[4] = {raw[rr][2].x, raw[rr][2].y, raw[rr][2].z, raw[rr][2].w};
 #pragma unroll
-                    for (int part = 0; part < 3; part++)
-#pragma unroll
-                        for (int e = 0; e < 8; e++) u[part][e] = 0.f;
-                }
-            } else if (t < S) {
-#pragma unroll
-                for (int part = 0; part < 3; part++) {
-                    const int ch0 = part * KD + h * DK + cc * 8;
-                    float x[4][8];
-#pragma unroll
-                    for (int d = 0; d < 4; d++) {
-                        const int tt = t - 3 + d;
-                        const bf16_t* src = tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0;
-                        unpack8(*reinterpret_cast<const uint4*>(src), x[d]);
-                    }
-#pragma unroll
-                    for (int e2 = 0; e2 < 8; e2 += 2) {
-                        const uint4 ww = *reinterpret_cast<const uint4*>(cw + (size_t)(ch0 + e2) * 4);
-                        const uint2 w0 = make_uint2(ww.x, ww.y), w1 = make_uint2(ww.z, ww.w);
-#pragma unroll
-                        for (int e = 0; e < 2; e++) {
-                            const uint2 wc = e ? w1 : w0;
-                            float sacc = x[0][e2 + e] * lo_bf(wc.x);
-                            sacc = sacc + x[1][e2 + e] * hi_bf(wc.x);
-                            sacc = sacc + x[2][e2 + e] * lo_bf(wc.y);
-                            sacc = sacc + x[3][e2 + e] * hi_bf(wc.y);
-                            u[part][e2 + e] = silu_lookup(L.tab, f2bf(sacc));
-                        }
-                    }
-                }
-                double sq = 0.0, sk = 0.0;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    sq += (double)u[0][e] * u[0][e];
-                    sk += (double)u[1][e] * u[1][e];
-                }
-                const float qr = rsqrt_rn((float)row16_sum_d(sq) / (float)DK + qk_eps());
-                const float kr = rsqrt_rn((float)row16_sum_d(sk) / (float)DK + qk_eps());
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    u[0][e] = BF(BF(u[0][e] * qr) * scq);
-                    u[1][e] = BF(BF(u[1][e] * kr) * sck);
-                }
-            } else {
-#pragma unroll
-                for (int part = 0; part < 3; part++)
-#pragma unroll
-                    for (int e = 0; e < 8; e++) u[part][e] = 0.f;             // rows past the end are zero (gdn_nax.py:172-174)
-            }
-            uint4 pk[3];
-#pragma unroll
-            for (int part = 0; part < 3; part++)
-                pk[part] = make_uint4(pack_bf(u[part][0], u[part][1]), pack_bf(u[part][2], u[part][3]),
-                                      pack_bf(u[part][4], u[part][5]), pack_bf(u[part][6], u[part][7]));
-            *reinterpret_cast<uint4*>(&L.Qs[tl * QS_LD + cc * 8]) = pk[0];
-            *reinterpret_cast<uint4*>(&L.Ks[tl * QS_LD + cc * 8]) = pk[1];
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                L.KT[(cc * 8 + e) * KT_LD + tl] = f2bf(u[1][e]);
-                L.VT[(cc * 8 + e) * KT_LD + tl] = f2bf(u[2][e]);
-            }
-            if (!FROM_QKV && qo && t < S) {
-                const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
-                *reinterpret_cast<uint4*>(qo + o) = pk[0];
-                *reinterpret_cast<uint4*>(ko + o) = pk[1];
-                *reinterpret_cast<uint4*>(vo + o) = pk[2];
+            for (int e = 0; e < 4; e++) {
+                L.KT[(cc * 8 + 2 * e) * KT_LD + tl] = (bf16_t)(kw[e] & 0xffffu);
+                L.KT[(cc * 8 + 2 * e + 1) * KT_LD + tl] = (bf16_t)(kw[e] >> 16);
+                L.VT[(cc * 8 + 2 * e) * KT_LD + tl] = (bf16_t)(vw[e] & 0xffffu);
+                L.VT[(cc * 8 + 2 * e + 1) * KT_LD + tl] = (bf16_t)(vw[e] >> 16);
             }
         }
     }
@@ -559,22 +483,16 @@ int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, const float
     return QT_OK;
 }
 
-int qt_gdn_phase_a(const void* proj, const void* conv_state, const void* conv_w, const float* A_log, const float* dt_bias,
-                   void* q, void* k, void* v, int from_qkv, void* ops, float* U, float* gC, int S, hipStream_t stream) {
-    if (!proj || !A_log || !dt_bias || !ops || !U || !gC) return QT_ERR_NULL;
-    if (!from_qkv && (!conv_state || !conv_w)) return QT_ERR_NULL;
-    if ((q || k || v || from_qkv) && !(q && k && v)) return QT_ERR_NULL;
+int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v, const float* A_log, const float* dt_bias,
+                   void* ops, float* U, float* gC, int S, hipStream_t stream) {
+    if (!proj || !q || !k || !v || !A_log || !dt_bias || !ops || !U || !gC) return QT_ERR_NULL;
     if (S < 0) return QT_ERR_DIM;
     if (S == 0) return QT_OK;
-    for (const void* p : {proj, conv_state, conv_w, (const void*)ops, (const void*)U, (const void*)q, (const void*)k, (const void*)v})
+    for (const void* p : {proj, q, k, v, (const void*)ops, (const void*)U})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     const int NC = (S + C - 1) / C;
-    if (from_qkv)
-        hipLaunchKernelGGL(gdn_phase_a_kernel<true>, dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (const bf16_t*)conv_state,
-                           (const bf16_t*)conv_w, A_log, dt_bias, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, (_Float16*)ops, U, gC, S);
-    else
-        hipLaunchKernelGGL(gdn_phase_a_kernel<false>, dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (const bf16_t*)conv_state,
-                           (const bf16_t*)conv_w, A_log, dt_bias, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, (_Float16*)ops, U, gC, S);
+    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (const bf16_t*)q,
+                       (const bf16_t*)k, (const bf16_t*)v, A_log, dt_bias, (_Float16*)ops, U, gC, S);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

@@ -40,37 +40,78 @@ __global__ __launch_bounds__(256) void normalize_qk_kernel(const bf16_t* __restr
     reinterpret_cast<uint32_t*>(ko + row * DK)[lane] = pack_bf(BF(BF(k0 * kr) * sck), BF(BF(k1 * kr) * sck));
 }
 
-// conv_prep (qwen35/prefill.py:96-134, 228-238): one workgroup of 128 threads per (token, head); thread i owns channel i
-// of the head's q, k and v.  proj [S,8224], cs [3,6144] -> q, k, v [S,16,128].
-__global__ __launch_bounds__(128) void conv_prep_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs,
-                                                        const bf16_t* __restrict__ cw, bf16_t* __restrict__ q,
-                                                        bf16_t* __restrict__ k, bf16_t* __restrict__ v, int S) {
-    __shared__ double red[2][2];
-    const int t = blockIdx.x / HV, h = blockIdx.x % HV, i = threadIdx.x, w = i >> 6;
-    float u[3];
+// conv_prep (qwen35/prefill.py:96-134, 228-238): proj [S,8224], cs [3,6144] -> q, k, v [S,16,128].
+// A workgroup of 256 threads handles 32 consecutive tokens of one head: a 16-lane group owns one token per round (two
+// rounds), a lane 8 consecutive channels of q, of k and of v; all row loads of both rounds are issued before the first
+// conv, SiLU comes from the LDS table, the sum of squares is reduced over the 16 lanes of the group.
+constexpr int CP_TOK = 32;
+__global__ __launch_bounds__(256) void conv_prep_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs,
+                                                        const bf16_t* __restrict__ cw, const bf16_t* __restrict__ silu_tab,
+                                                        bf16_t* __restrict__ q, bf16_t* __restrict__ k, bf16_t* __restrict__ v,
+                                                        int S) {
+    __shared__ __align__(16) bf16_t tab[SILU_TAB_SIZE];
+    const int tb = blockIdx.x / HV, h = blockIdx.x % HV, tid = threadIdx.x, gi = tid >> 4, cc = tid & 15;
+    uint4 raw[2][3][4], wt[3][4];
 #pragma unroll
     for (int part = 0; part < 3; part++) {
-        const int ch = part * KD + h * DK + i;
-        float x[4];
+        const int ch0 = part * KD + h * DK + cc * 8;
 #pragma unroll
-        for (int d = 0; d < 4; d++) {
-            const int tt = t - 3 + d;
-            x[d] = tt < 0 ? bf2f(cs[(tt + 3) * CD + ch]) : bf2f(proj[(size_t)tt * PW + ch]);
+        for (int e = 0; e < 4; e++) wt[part][e] = *reinterpret_cast<const uint4*>(cw + (size_t)(ch0 + 2 * e) * 4);
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const int t = min(tb * CP_TOK + r * 16 + gi, S - 1);               // rows past the end are computed and dropped
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const int tt = t - 3 + d;
+                raw[r][part][d] = *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0);
+            }
         }
-        u[part] = conv_silu(x[0], x[1], x[2], x[3], *reinterpret_cast<const uint2*>(cw + (size_t)ch * 4));
     }
-    const double sq = wave_sum_d((double)u[0] * u[0]), sk = wave_sum_d((double)u[1] * u[1]);
-    if ((i & 63) == 0) {
-        red[0][w] = sq;
-        red[1][w] = sk;
-    }
+    silu_table_fill(tab, silu_tab, tid, 256);
     __syncthreads();
-    const float qr = rsqrt_rn((float)(red[0][0] + red[0][1]) / (float)DK + qk_eps());
-    const float kr = rsqrt_rn((float)(red[1][0] + red[1][1]) / (float)DK + qk_eps());
-    const size_t o = ((size_t)t * HV + h) * DK + i;
-    q[o] = f2bf(BF(BF(u[0] * qr) * BF(INV_SCALE * INV_SCALE)));
-    k[o] = f2bf(BF(BF(u[1] * kr) * BF(INV_SCALE)));
-    v[o] = f2bf(u[2]);
+    const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const int t = tb * CP_TOK + r * 16 + gi;
+        float u[3][8];
+#pragma unroll
+        for (int part = 0; part < 3; part++) {
+            float x[4][8];
+#pragma unroll
+            for (int d = 0; d < 4; d++) unpack8(raw[r][part][d], x[d]);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint4 ww = wt[part][e >> 1];
+                const uint2 wc = (e & 1) ? make_uint2(ww.z, ww.w) : make_uint2(ww.x, ww.y);
+                u[part][e] = conv_silu_tab(tab, x[0][e], x[1][e], x[2][e], x[3][e], wc);
+            }
+        }
+        double sq = 0.0, sk = 0.0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            sq += (double)u[0][e] * u[0][e];
+            sk += (double)u[1][e] * u[1][e];
+        }
+        const float qr = rsqrt_rn((float)row16_sum_d(sq) / (float)DK + qk_eps());
+        const float kr = rsqrt_rn((float)row16_sum_d(sk) / (float)DK + qk_eps());
+        if (t < S) {
+            const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
+            uint4 pq, pk, pv;
+            pq.x = pack_bf(BF(BF(u[0][0] * qr) * scq), BF(BF(u[0][1] * qr) * scq)); pq.y = pack_bf(BF(BF(u[0][2] * qr) * scq), BF(BF(u[0][3] * qr) * scq));
+            pq.z = pack_bf(BF(BF(u[0][4] * qr) * scq), BF(BF(u[0][5] * qr) * scq)); pq.w = pack_bf(BF(BF(u[0][6] * qr) * scq), BF(BF(u[0][7] * qr) * scq));
+            pk.x = pack_bf(BF(BF(u[1][0] * kr) * sck), BF(BF(u[1][1] * kr) * sck)); pk.y = pack_bf(BF(BF(u[1][2] * kr) * sck), BF(BF(u[1][3] * kr) * sck));
+            pk.z = pack_bf(BF(BF(u[1][4] * kr) * sck), BF(BF(u[1][5] * kr) * sck)); pk.w = pack_bf(BF(BF(u[1][6] * kr) * sck), BF(BF(u[1][7] * kr) * sck));
+            pv.x = pack_bf(u[2][0], u[2][1]); pv.y = pack_bf(u[2][2], u[2][3]); pv.z = pack_bf(u[2][4], u[2][5]); pv.w = pack_bf(u[2][6], u[2][7]);
+            *reinterpret_cast<uint4*>(q + o) = pq;
+            *reinterpret_cast<uint4*>(k + o) = pk;
+            *reinterpret_cast<uint4*>(v + o) = pv;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void silu_table_kernel(bf16_t* __restrict__ tab) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < SILU_TAB_SIZE) tab[i] = silu_table_entry(i);
 }
 
 // gated RMSNorm (qwen35/batch.py:304-343, qwen35/prefill.py:137-157): 16 lanes per (row, head), 8 elements per lane.
@@ -179,14 +220,26 @@ int qt_normalize_qk(const void* q, const void* k, void* q_out, void* k_out, long
     return QT_OK;
 }
 
-int qt_gdn_conv_prep(const void* proj, const void* conv_state, const void* conv_w, void* q, void* k, void* v, int S,
-                     hipStream_t stream) {
+int qt_silu_table_bytes(void) { return SILU_TAB_SIZE * 2; }
+
+int qt_silu_table_build(void* table, hipStream_t stream) {
+    if (!table) return QT_ERR_NULL;
+    if (!al(table, 16)) return QT_ERR_ALIGN;
+    hipLaunchKernelGGL(silu_table_kernel, dim3((SILU_TAB_SIZE + 255) / 256), dim3(256), 0, stream, (bf16_t*)table);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_gdn_conv_prep(const void* proj, const void* conv_state, const void* conv_w, const void* silu_table, void* q, void* k,
+                     void* v, int S, hipStream_t stream) {
     if (!proj || !conv_state || !conv_w || !q || !k || !v) return QT_ERR_NULL;
     if (S < 0) return QT_ERR_DIM;
     if (S == 0) return QT_OK;
-    if (!al(conv_w, 8)) return QT_ERR_ALIGN;
-    hipLaunchKernelGGL(conv_prep_kernel, dim3((unsigned)S * HV), dim3(128), 0, stream, (const bf16_t*)proj,
-                       (const bf16_t*)conv_state, (const bf16_t*)conv_w, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, S);
+    for (const void* p : {proj, conv_state, conv_w, silu_table, (const void*)q, (const void*)k, (const void*)v})
+        if (!al(p, 16)) return QT_ERR_ALIGN;
+    hipLaunchKernelGGL(conv_prep_kernel, dim3((unsigned)((S + CP_TOK - 1) / CP_TOK) * HV), dim3(256), 0, stream, (const bf16_t*)proj,
+                       (const bf16_t*)conv_state, (const bf16_t*)conv_w, (const bf16_t*)silu_table, (bf16_t*)q, (bf16_t*)k,
+                       (bf16_t*)v, S);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

@@ -19,11 +19,8 @@ typedef uint16_t bf16_t;   // raw bf16 bits
 
 __device__ __forceinline__ float bf2f(bf16_t b) { return __uint_as_float((uint32_t)b << 16); }
 
-__device__ __forceinline__ bf16_t f2bf(float f) {   // round to nearest even; NaN stays NaN
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+__device__ __forceinline__ bf16_t f2bf(float f) {   // round to nearest even (v_cvt_pk_bf16_f32 on gfx950)
+    return __builtin_bit_cast(bf16_t, static_cast<__bf16>(f));
 }
 
 __device__ __forceinline__ float BF(float f) { return bf2f(f2bf(f)); }          // `#define BF(v)`, mslib.py:8-10
@@ -94,6 +91,42 @@ __device__ __forceinline__ float conv_silu(float w0, float w1, float w2, float x
     s = s + w2 * lo_bf(c.y);
     s = s + x * hi_bf(c.y);
     return silu_bf16(BF(s));
+}
+
+// silu_bf16 is a bf16 -> bf16 map, so kernels that evaluate it many times per thread read it from a table in LDS:
+// 2 signs x 14 exponents (bf16 exponent fields 118..131, 2^-9 <= |x| < 2^5) x 128 mantissas = 3584 entries (7 KiB).
+// Below the range exp(|x|) rounds to 1 and sigmoid_bf16 is exactly 0.5; above it the direct evaluation is used.
+constexpr int SILU_TAB_LO = 118, SILU_TAB_N = 14 * 128, SILU_TAB_SIZE = 2 * SILU_TAB_N;
+__device__ __forceinline__ bf16_t silu_table_entry(int i) {
+    const bf16_t xb = (bf16_t)(((i / SILU_TAB_N) << 15) | (SILU_TAB_LO * 128 + i % SILU_TAB_N));
+    return f2bf(silu_bf16(bf2f(xb)));
+}
+// fills `tab` (LDS) from a prebuilt copy in global memory, or computes it when there is none
+__device__ __forceinline__ void silu_table_fill(bf16_t* tab, const bf16_t* __restrict__ prebuilt, int tid, int nthreads) {
+    if (prebuilt) {
+        for (int i = tid; i < SILU_TAB_SIZE / 8; i += nthreads)
+            reinterpret_cast<uint4*>(tab)[i] = reinterpret_cast<const uint4*>(prebuilt)[i];
+    } else {
+        for (int i = tid; i < SILU_TAB_SIZE; i += nthreads) tab[i] = silu_table_entry(i);
+    }
+}
+__device__ __forceinline__ float silu_lookup(const bf16_t* tab, bf16_t xb) {
+    const unsigned idx = (xb & 0x7fffu) - SILU_TAB_LO * 128;                    // wraps for small |x|
+    if (idx < (unsigned)SILU_TAB_N) return bf2f(tab[(xb >> 15) * SILU_TAB_N + idx]);
+    if ((xb & 0x7fffu) < SILU_TAB_LO * 128) return BF(bf2f(xb) * 0.5f);
+    return silu_bf16(bf2f(xb));
+}
+// conv4 + silu through the table: taps in c (4 bf16), inputs oldest first
+__device__ __forceinline__ float conv_silu_tab(const bf16_t* tab, float w0, float w1, float w2, float x, uint2 c) {
+    float s = w0 * lo_bf(c.x);
+    s = s + w1 * hi_bf(c.x);
+    s = s + w2 * lo_bf(c.y);
+    s = s + x * hi_bf(c.y);
+    return silu_lookup(tab, f2bf(s));
+}
+__device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]) {
+    f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
+    f[4] = lo_bf(w.z); f[5] = hi_bf(w.z); f[6] = lo_bf(w.w); f[7] = hi_bf(w.w);
 }
 
 constexpr float INV_SCALE = 0.08838834764831845f;                                // 128^-0.5, kernels.py:490

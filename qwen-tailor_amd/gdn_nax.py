@@ -29,25 +29,23 @@ def _alloc_records(S, dev):
 
 
 def _phase_a(proj, conv_state, conv_w, A_log, dt_bias, qkv=None, want_qkv=True):
+    """conv_prep (unless q, k, v are given) followed by the phase A kernel.  Returns (q, k, v, ops, U, gC)."""
+    from . import prefill
     proj = L.dev(proj, BF16, "proj", (None, PW))
     S = proj.shape[0]
-    dev = proj.device
     A, dtb = L.f32(A_log, "A_log", (HV,)), L.f32(dt_bias, "dt_bias", (HV,))
-    ops, U, gC = _alloc_records(S, dev)
     if qkv is not None:
         q, k, v = (L.dev(t, BF16, name, (S, HV, DK)) for t, name in zip(qkv, "qkv"))
-        cs = w = None
     else:
-        cs = L.dev(conv_state, BF16, "conv_state", (3, CD))
-        w = flat_conv_w(conv_w)
-        q, k, v = (torch.empty((S, HV, DK), dtype=BF16, device=dev) for _ in range(3)) if want_qkv else (None, None, None)
-    L.call("qt_gdn_phase_a", L.ptr(proj), L.ptr(cs), L.ptr(w), L.ptr(A), L.ptr(dtb), L.ptr(q), L.ptr(k), L.ptr(v),
-           1 if qkv is not None else 0, L.ptr(ops), L.ptr(U), L.ptr(gC), S, L.stream())
+        q, k, v = prefill.conv_prep(proj, conv_state, conv_w)
+    ops, U, gC = _alloc_records(S, proj.device)
+    L.call("qt_gdn_phase_a", L.ptr(proj), L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(A), L.ptr(dtb), L.ptr(ops), L.ptr(U), L.ptr(gC), S,
+           L.stream())
     return q, k, v, ops, U, gC
 
 
 def prep_a(proj, conv_state, conv_w, A_log, dt_bias, relaxed=True):
-    """conv+silu+qk-norm and phase A in one kernel (qwen35/gdn_nax.py:394-401).
+    """conv+silu+qk-norm and phase A (qwen35/gdn_nax.py:394-401; here two launches: the conv kernel, then phase A).
     proj [S,8224], conv_state [3,6144], conv_w [6144,4,1] -> q, k, v [S,16,128] bf16 and the three phase-B records."""
     return _phase_a(proj, conv_state, conv_w, A_log, dt_bias)
 

@@ -27,7 +27,7 @@ def gdn_core(proj, conv_state, ssm_state, conv_w, A_log, dt_bias, gnorm, want_qk
     S = proj.shape[0]
     cs = conv_state.reshape(3, CD)
     if GDN_IMPL == "nax":
-        q, k, v, ops, U, gC = gdn_nax._phase_a(proj, cs, conv_w, A_log, dt_bias, want_qkv=want_qkv)
+        q, k, v, ops, U, gC = gdn_nax._phase_a(proj, cs, conv_w, A_log, dt_bias)
         out, new_ssm = gdn_nax.phase_b(proj, None, None, ops, U, gC, ssm_state)
     else:
         q, k, v = conv_prep(proj, cs, conv_w)
@@ -45,7 +45,8 @@ def conv_prep(proj, conv_state, conv_w):
     cs = L.dev(conv_state, BF16, "conv_state", (3, CD))
     w = flat_conv_w(conv_w)
     q, k, v = (torch.empty((S, HV, DK), dtype=BF16, device=proj.device) for _ in range(3))
-    L.call("qt_gdn_conv_prep", L.ptr(proj), L.ptr(cs), L.ptr(w), L.ptr(q), L.ptr(k), L.ptr(v), S, L.stream())
+    L.call("qt_gdn_conv_prep", L.ptr(proj), L.ptr(cs), L.ptr(w), L.ptr(L.silu_table(proj.device)), L.ptr(q), L.ptr(k), L.ptr(v), S,
+           L.stream())
     return q, k, v
 
 
