@@ -211,16 +211,26 @@ __global__ __launch_bounds__(128) void gdn_phase_b_kernel(const _Float16* __rest
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int QS_LD = DK + 8;        // row strides (elements) of the LDS tiles: keep 16-byte alignment, spread the banks
-constexpr int KT_LD = C + 8;
+constexpr int KT_LD = C;             // K^T / V^T rows are unpadded; their 16-byte chunks are XOR-swizzled by (row >> 3) & 7
 constexpr int LS_LD = C + 4;
 
-struct PhaseALds {
-    __align__(16) bf16_t Qs[C * QS_LD];
-    __align__(16) bf16_t Ks[C * QS_LD];
+// element (row d, token t) of the transposed tiles: chunk (t >> 3) ^ ((d >> 3) & 7), so that the 2-byte transposing writes of
+// a wavefront (16 lanes = 16 values of d >> 3, same t) spread over the banks while a 16-byte read stays one chunk
+__device__ __forceinline__ int kt_at(int d, int t) { return d * KT_LD + ((((t >> 3) ^ (d >> 3)) & 7) << 3) + (t & 7); }
+
+struct PhaseALds {                       // 68 KiB: two workgroups per CU
+    union {
+        struct {                         // first half of the kernel: the chunk's q, k rows
+            __align__(16) bf16_t Qs[C * QS_LD];
+            __align__(16) bf16_t Ks[C * QS_LD];
+        };
+        struct {                         // second half: L = strict_lower(beta G K K^T) and T = (I + L)^-1
+            __align__(16) float Ls[C * LS_LD];
+            __align__(16) float Ts[C * LS_LD];
+        };
+    };
     __align__(16) bf16_t KT[DK * KT_LD];
     __align__(16) bf16_t VT[DV * KT_LD];
-    __align__(16) float Ls[C * LS_LD];
-    __align__(16) float Ts[C * LS_LD];
     float Lc[C], beta[C], gam[C], dec[C];
 };
 
@@ -261,7 +271,6 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
             if (t >= S) raw[rr][0] = raw[rr][1] = raw[rr][2] = make_uint4(0, 0, 0, 0);
         }
     }
-    for (int i = tid; i < C * LS_LD; i += 256) L.Ts[i] = 0.f;                   // blocks of T above the diagonal stay zero
 
     // ---- gates of the chunk's tokens (gdn_nax.py:80-104): wave 0, one token per lane
     if (w == 0) {
@@ -295,32 +304,37 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
             const uint32_t vw[4] = {raw[rr][2].x, raw[rr][2].y, raw[rr][2].z, raw[rr][2].w};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                L.KT[(cc * 8 + 2 * e) * KT_LD + tl] = (bf16_t)(kw[e] & 0xffffu);
-                L.KT[(cc * 8 + 2 * e + 1) * KT_LD + tl] = (bf16_t)(kw[e] >> 16);
-                L.VT[(cc * 8 + 2 * e) * KT_LD + tl] = (bf16_t)(vw[e] & 0xffffu);
-                L.VT[(cc * 8 + 2 * e + 1) * KT_LD + tl] = (bf16_t)(vw[e] >> 16);
+                L.KT[kt_at(cc * 8 + 2 * e, tl)] = (bf16_t)(kw[e] & 0xffffu);
+                L.KT[kt_at(cc * 8 + 2 * e + 1, tl)] = (bf16_t)(kw[e] >> 16);
+                L.VT[kt_at(cc * 8 + 2 * e, tl)] = (bf16_t)(vw[e] & 0xffffu);
+                L.VT[kt_at(cc * 8 + 2 * e + 1, tl)] = (bf16_t)(vw[e] >> 16);
             }
         }
     }
     __syncthreads();
 
     // ---- K K^T (lower tiles) -> L, and (Q K^T)^T -> Am, on bf16 MFMA.  Wave w: row of tiles ti = 3 - w of K K^T and the
-    // Am tiles of ct = w.
+    // Am / Qg tiles of ct = w.  L stays in registers until every wave is done with Qs / Ks, whose LDS it then takes over.
+    f32x4 Lreg[4];
     {
         const int ti = 3 - w;
-        for (int tj = 0; tj <= ti; tj++) {
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kb = 0; kb < 4; kb++) {
-                const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * ti + n) * QS_LD + 32 * kb + 8 * g]));
-                const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]));
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
-            }
-            const int j = 16 * tj + n;
+        for (int tj = 0; tj < 4; tj++) {
+            Lreg[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (tj <= ti) {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int i = 16 * ti + 4 * g + r;
-                L.Ls[i * LS_LD + j] = i > j ? L.beta[i] * expf(L.Lc[i] - L.Lc[j]) * acc[r] : 0.f;
+                for (int kb = 0; kb < 4; kb++) {
+                    const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * ti + n) * QS_LD + 32 * kb + 8 * g]));
+                    const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]));
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+                }
+                const int j = 16 * tj + n;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int i = 16 * ti + 4 * g + r;
+                    Lreg[tj][r] = i > j ? L.beta[i] * expf(L.Lc[i] - L.Lc[j]) * acc[r] : 0.f;
+                }
             }
         }
         const int ct = w, co = 16 * ct + n;                         // Am: rows c_out = 16 ct + n, k = c_in (permuted)
@@ -346,6 +360,27 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
             }
             *reinterpret_cast<half8*>(op + OP_A + (ct * 2 + kb2) * 512 + lane * 8) = pack_half8(part[0], part[1]);
         }
+        // Qg = gamma * Q (rows of tile ct), k index permuted
+        const float gm = L.gam[16 * ct + n];
+        for (int kb = 0; kb < 4; kb++) {
+            float qf[8];
+            unpack4(*reinterpret_cast<const uint2*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 4 * g]), qf);
+            unpack4(*reinterpret_cast<const uint2*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 16 + 4 * g]), qf + 4);
+#pragma unroll
+            for (int j = 0; j < 8; j++) qf[j] *= gm;
+            *reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8) = to_half8(qf);
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < C * LS_LD; i += 256) L.Ts[i] = 0.f;                   // blocks of T above the diagonal stay zero
+    {
+        const int ti = 3 - w;
+#pragma unroll
+        for (int tj = 0; tj < 4; tj++)
+            if (tj <= ti) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) L.Ls[(16 * ti + 4 * g + r) * LS_LD + 16 * tj + n] = Lreg[tj][r];
+            }
     }
     __syncthreads();
 
@@ -417,7 +452,7 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
                 for (int kb2 = 0; kb2 < 2; kb2++) {
                     if (kb2 >= nkb) continue;
                     float kf[8];
-                    unpack8(*reinterpret_cast<const uint4*>(&L.KT[(16 * mt + n) * KT_LD + 32 * kb2 + 8 * g]), kf);
+                    unpack8(*reinterpret_cast<const uint4*>(&L.KT[kt_at(16 * mt + n, 32 * kb2 + 8 * g)]), kf);
 #pragma unroll
                     for (int j = 0; j < 8; j++) kf[j] *= -L.gam[32 * kb2 + 8 * g + j];
                     acc[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(to_half8(kf), tb[kb2], acc[hf], 0, 0, 0);
@@ -432,27 +467,18 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
             for (int kb2 = 0; kb2 < 2; kb2++) {
                 if (kb2 >= nkb) continue;
                 float vf[8];
-                unpack8(*reinterpret_cast<const uint4*>(&L.VT[(16 * sl + n) * KT_LD + 32 * kb2 + 8 * g]), vf);
+                unpack8(*reinterpret_cast<const uint4*>(&L.VT[kt_at(16 * sl + n, 32 * kb2 + 8 * g)]), vf);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tb[kb2], to_half8(vf), acc, 0, 0, 0);
             }
             *reinterpret_cast<f32x4*>(up + ((sl * NCT + ct) * 64 + lane) * 4) = acc;
         }
-        // Qg = gamma * Q (rows of tile ct) and Kd = (dec * K)^T (rows dk of tiles 2w, 2w+1), k index permuted
-        const float gm = L.gam[16 * ct + n];
-        for (int kb = 0; kb < 4; kb++) {
-            float qf[8];
-            unpack4(*reinterpret_cast<const uint2*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 4 * g]), qf);
-            unpack4(*reinterpret_cast<const uint2*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 16 + 4 * g]), qf + 4);
-#pragma unroll
-            for (int j = 0; j < 8; j++) qf[j] *= gm;
-            *reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8) = to_half8(qf);
-        }
+        // Kd = (dec * K)^T (rows dk of tiles 2w, 2w+1), k index permuted
         for (int mm = 0; mm < 2; mm++) {
             const int mt = 2 * w + mm;
             for (int kb2 = 0; kb2 < 2; kb2++) {
                 float kf[8];
-                unpack4(*reinterpret_cast<const uint2*>(&L.KT[(16 * mt + n) * KT_LD + 32 * kb2 + 4 * g]), kf);
-                unpack4(*reinterpret_cast<const uint2*>(&L.KT[(16 * mt + n) * KT_LD + 32 * kb2 + 16 + 4 * g]), kf + 4);
+                unpack4(*reinterpret_cast<const uint2*>(&L.KT[kt_at(16 * mt + n, 32 * kb2 + 4 * g)]), kf);
+                unpack4(*reinterpret_cast<const uint2*>(&L.KT[kt_at(16 * mt + n, 32 * kb2 + 16 + 4 * g)]), kf + 4);
 #pragma unroll
                 for (int j = 0; j < 8; j++) kf[j] *= L.dec[32 * kb2 + 16 * (j >> 2) + 4 * g + (j & 3)];
                 *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = to_half8(kf);
