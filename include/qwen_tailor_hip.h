@@ -86,14 +86,21 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
  * proj [S,8224], and computes the gates, K K^T / Q K^T on bf16 MFMA, the 64 x 64 unit-lower-triangular inverse in fp32 and the
  * state-independent MFMA operands of phase B.  It fills three caller-owned buffers of qt_gdn_chunk_{ops,u,gc}_bytes(S) bytes:
  * `ops` (half-precision operand tiles), `U` and `gC` (f32).
- * Phase B is serial over the chunks: state_in / state_out [16,128,128] f32, y [S,16,128] bf16. */
+ * Phase B: state_in / state_out [16,128,128] f32, y [S,16,128] bf16.  It runs as a serial kernel over the chunks (the state
+ * chain, which leaves the per-chunk B operands in `snap`, qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned)
+ * and a kernel parallel over (chunk, head) that computes the outputs from `snap`.
+ * qt_gdn_phase_b_norm is the same with prefill.gated_norm (qwen35/prefill.py:241-244) fused into the output kernel: it
+ * writes out [S,2048] bf16 = gated RMSNorm of y with z = proj[:,6144:8192] and weight gw [128] f32 instead of y. */
 long qt_gdn_chunk_ops_bytes(int S);
 long qt_gdn_chunk_u_bytes(int S);
 long qt_gdn_chunk_gc_bytes(int S);
+long qt_gdn_chunk_snap_bytes(int S);
 int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v, const float* A_log, const float* dt_bias,
                    void* ops, float* U, float* gC, int S, qt_stream_t stream);
-int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, const float* state_in, float* state_out, void* y, int S,
-                   qt_stream_t stream);
+int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
+                   void* y, int S, qt_stream_t stream);
+int qt_gdn_phase_b_norm(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
+                        const void* proj, const float* gw, float eps, void* out, int S, qt_stream_t stream);
 
 /* Causal prefill attention: the mx.fast.scaled_dot_product_attention(..., mask="causal") call of the full-attention layers
  * (qwen35/model.py:160-167, qwen35/prefill.py:468).  q, out [8][S][256] bf16 with head stride q_head_stride (elements);

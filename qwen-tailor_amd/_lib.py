@@ -27,7 +27,8 @@ _SIGS = {
     "qt_gated_rmsnorm": [_vp, _vp, _vp, _vp, _l, _f, _vp],
     "qt_gdn_recurrent": [_vp] * 8 + [_i] * 6 + [_vp],
     "qt_gqa_attn_decode": [_vp] * 9 + [_l, _i, _i, _i, _i, _i, _vp],
-    "qt_gdn_phase_b": [_vp] * 6 + [_i, _vp],
+    "qt_gdn_phase_b": [_vp] * 7 + [_i, _vp],
+    "qt_gdn_phase_b_norm": [_vp] * 8 + [_f, _vp, _i, _vp],
     "qt_gqa_prefill_causal": [_vp] * 5 + [_l, _i, _i, _i, _l, _l, _vp],
     "qt_gdn_phase_a": [_vp] * 9 + [_i, _vp],
 }
@@ -44,7 +45,8 @@ def lib():
             fn = getattr(L, name)
             fn.argtypes, fn.restype = args, ctypes.c_int
         L.qt_gqa_attn_workspace_bytes.argtypes, L.qt_gqa_attn_workspace_bytes.restype = [_i] * 4, ctypes.c_long
-        for name in ("qt_gdn_chunk_ops_bytes", "qt_gdn_chunk_u_bytes", "qt_gdn_chunk_gc_bytes", "qt_gqa_prefill_workspace_bytes"):
+        for name in ("qt_gdn_chunk_ops_bytes", "qt_gdn_chunk_u_bytes", "qt_gdn_chunk_gc_bytes", "qt_gdn_chunk_snap_bytes",
+                     "qt_gqa_prefill_workspace_bytes"):
             getattr(L, name).argtypes, getattr(L, name).restype = [_i], ctypes.c_long
         _lib = L
     return _lib

@@ -42,168 +42,247 @@ __device__ __forceinline__ half8 pack_half8(const f32x4& a, const f32x4& b) {
     return h;
 }
 
-// Phase B: serial over the chunks.  grid = 128 wavefronts (head, dv slice); ops / U / gC are phase A's records.
-constexpr int PF_AHEAD = 8;                     // chunks the L2 prefetch wavefront runs ahead of the MFMA wavefront
+// Phase B runs in two kernels.
+//
+// The chain kernel is the serial part: S_{c+1}^T = gamma_c S_c^T + Kd_c D_c with D_c = U_c + Wn_c S_c^T.  It does not
+// compute outputs; it leaves, per (chunk, head, slice), the two half-precision B operands that the outputs need
+// (S_c^T and D_c, 6 KiB) in `snap`.  The output kernel then computes Y_c = Qg_c S_c^T + Am_c D_c for all chunks in parallel.
+// Splitting the outputs off halves the bytes the serial kernel has to pull per step (W and Kd: 32 of the 56 KiB).
+//
+// Chain kernel: one workgroup of 5 wavefronts per (head, 16-wide dv slice).  MFMA wavefront w owns rows 16w..16w+15 of D
+// (the chunk's tokens) and rows 32w..32w+31 of S^T (dk): per chunk it pulls only its 8 operand tiles (8 KiB) and keeps
+// PB_DEP chunks of them in flight in registers, so the latency of a load is covered by PB_DEP chain steps.  Two exchanges
+// through LDS per step make up for the split: every wavefront publishes its block of S^T as the fp16 B operand and reads
+// all four (barrier E1), and publishes its rows of D and reads both k-blocks (barrier E2).  The fifth wavefront copies
+// exactly these two LDS areas to `snap`: the MFMA wavefronts issue loads only, which keeps their vmcnt waits partial
+// (a store in flight next to loads forces every wait to zero on this target).
+constexpr int PB_DEP = 4;                        // chunks of operands in flight per MFMA wavefront
+constexpr int SNAP_S = 4 * 512;                  // halves: S^T as B operand, [kb 4][lane 64][8]
+constexpr int SNAP_D = 2 * 512;                  // halves: D as B operand, [kb2 2][lane 64][8]
+constexpr int SNAP_HALVES = SNAP_S + SNAP_D;     // 6 KiB per (chunk, head, slice)
+constexpr int KORD[4] = {0, 2, 1, 3};            // order in which a step consumes its Kd tiles (two independent accumulators)
 
-__global__ __launch_bounds__(128) void gdn_phase_b_kernel(const _Float16* __restrict__ ops, const float* __restrict__ U,
-                                                         const float* __restrict__ gC, const float* __restrict__ st_in,
-                                                         float* __restrict__ st_out, bf16_t* __restrict__ y, int S, int NC) {
+__global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, const float* U, const float* gC, const float* st_in,
+                                                        float* st_out, _Float16* snap, int NC) {
     // heads that share an XCD's L2 keep their 8 slices there: workgroup id = xcd + 8 k, head = xcd + 8 (k / 8), slice = k % 8
     const int xcd = blockIdx.x & 7, kq = blockIdx.x >> 3;
     const int h = xcd + 8 * (kq >> 3), sl = kq & 7;
-    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    __shared__ __align__(16) _Float16 sb_x[SNAP_S];
+    __shared__ __align__(16) _Float16 db_x[SNAP_D];
+    const half8* sbx = reinterpret_cast<const half8*>(sb_x) + lane;
+    const half8* dbx = reinterpret_cast<const half8*>(db_x) + lane;
 
-    // Wavefront 0 runs the serial MFMA chain and touches global memory with loads only: on gfx9-family targets loads and
-    // stores share one in-order counter only as long as a single kind is in flight, so a store in the loop would force
-    // every wait down to zero outstanding loads and expose the full memory latency at every chunk.
-    // Wavefront 1 is its helper: it writes the finished output rows, which wavefront 0 hands over through two buffers in
-    // LDS, and it pulls the records of the coming chunks into this XCD's L2 (one dword per 128-byte line), PF_AHEAD chunks
-    // in front.  The hand-over is one bare s_barrier per chunk (no fence: only LDS is exchanged, and s_waitcnt lgkmcnt(0)
-    // orders it): after barrier c the helper reads buffer c & 1, and wavefront 0 next writes that buffer after barrier c+1.
-    __shared__ __align__(16) bf16_t y_s[2][C * 16];                           // one chunk of this slice's outputs, row major
-    if (threadIdx.x >= 64) {
-        unsigned sink = 0;
+    if (w == 4) {
+        half8* dst = reinterpret_cast<half8*>(snap + ((size_t)h * 8 + sl) * SNAP_HALVES) + lane;
+        const size_t cst = (size_t)HV * 8 * SNAP_HALVES / 8;                    // half8 per chunk
         for (int c = 0; c < NC; c++) {
-            // touch the record of chunk c + PF_AHEAD; the values are only folded into `sink` after the hand-over below,
-            // so these loads never delay the barrier
-            unsigned pfv[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            const int pf = c + PF_AHEAD;
-            if (PF_AHEAD > 0 && pf < NC) {
-                const size_t rec = (size_t)pf * HV + h;
-                const unsigned* o32 = reinterpret_cast<const unsigned*>(ops + rec * OP_HALVES) + lane * 32;
-#pragma unroll
-                for (int i = 0; i < OP_HALVES * 2 / 8192; i++) pfv[i] = o32[i * 2048];
-                const unsigned* u32 = reinterpret_cast<const unsigned*>(U + rec * U_FLOATS + (size_t)sl * NCT * 256);
-                pfv[7] = u32[(lane & 31) * 32];
-            }
-            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_s_barrier();                                       // E1: sb_x holds S_c^T
             asm volatile("" ::: "memory");
-            const uint4* src = reinterpret_cast<const uint4*>(&y_s[c & 1][lane * 16]);
-            const uint4 lo = src[0], hi = src[1];
-            const int t = c * C + lane;
-            if (t < S) {
-                uint4* dst = reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV + sl * 16);
-                dst[0] = lo;
-                dst[1] = hi;
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                  // the LDS reads are done before the next barrier
-#pragma unroll
-            for (int i = 0; i < 8; i++) sink ^= pfv[i];
+            const half8 a0 = sbx[0], a1 = sbx[64], a2 = sbx[128], a3 = sbx[192];
+            dst[0] = a0;
+            dst[64] = a1;
+            dst[128] = a2;
+            dst[192] = a3;
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();                                       // E2: db_x holds D_c
+            asm volatile("" ::: "memory");
+            const half8 d0 = dbx[0], d1 = dbx[64];
+            dst[256] = d0;
+            dst[320] = d1;
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            dst += cst;
         }
-        if (sink == 0x9e3779b9u && S < 0) st_out[0] = 0.f;                      // keeps the prefetch loads alive; never true
         return;
     }
 
-    f32x4 ST[8];
+    f32x4 ST[2];
     {
-        const float* sp = st_in + ((size_t)h * DV + sl * 16 + n) * DK;          // S[h][dv][dk], dk contiguous
-#pragma unroll
-        for (int mt = 0; mt < 8; mt++) ST[mt] = *reinterpret_cast<const f32x4*>(sp + mt * 16 + 4 * g);
+        const float* sp = st_in + ((size_t)h * DV + sl * 16 + n) * DK + w * 32 + 4 * g;   // S[h][dv][dk], dk contiguous
+        ST[0] = *reinterpret_cast<const f32x4*>(sp);
+        ST[1] = *reinterpret_cast<const f32x4*>(sp + 16);
     }
-    // Operand FIFO, one chunk deep: tile i of chunk c+1 is loaded into the registers of tile i of chunk c right after the
-    // MFMA that consumed it, so a whole chunk step of MFMA work covers the latency of every load.
-    half8 Wt[16], Qt[16], Kt[16], At[8];
-    f32x4 Ut[NCT];
-    float gc;
-    {
-        const half8* op = reinterpret_cast<const half8*>(ops + (size_t)h * OP_HALVES) + lane;
-        const f32x4* up = reinterpret_cast<const f32x4*>(U + (size_t)h * U_FLOATS + (size_t)sl * NCT * 256) + lane;
-        // same issue order as inside the loop
+    const half8* opb = reinterpret_cast<const half8*>(ops + (size_t)h * OP_HALVES) + lane;
+    const f32x4* upb = reinterpret_cast<const f32x4*>(U + (size_t)h * U_FLOATS + (size_t)(sl * NCT + w) * 256) + lane;
+    const size_t ost = (size_t)HV * OP_HALVES / 8, ust = (size_t)HV * U_FLOATS / 4;
+    const int wq = (OP_W / 8) + w * 4 * 64, kq0 = (OP_K / 8) + w * 4 * 64;       // W[ct = w][kb], Kd[mt = 2w + i][kb2]
+
+    half8 Wt[PB_DEP][4], Kt[PB_DEP][4];
+    f32x4 Ut[PB_DEP];
+    float gct[PB_DEP];                       // the chunk's decay rides in the FIFO as one more (lane-uniform) vector load
 #pragma unroll
-        for (int ct = 0; ct < NCT; ct++) Ut[ct] = up[ct * 64];
+    for (int j = 0; j < PB_DEP; j++) {                                          // same issue order as inside the steps
+        const int cc = min(j, NC - 1);
 #pragma unroll
-        for (int kb = 0; kb < 4; kb++)
+        for (int i = 0; i < 4; i++) Wt[j][i] = opb[cc * ost + wq + i * 64];
+        Ut[j] = upb[cc * ust];
 #pragma unroll
-            for (int ct = 0; ct < NCT; ct++) Wt[ct * 4 + kb] = op[(OP_W / 8) + (ct * 4 + kb) * 64];
-        gc = gC[h];
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; kb2++)
-#pragma unroll
-            for (int mt = 0; mt < 8; mt++) Kt[mt * 2 + kb2] = op[(OP_K / 8) + (mt * 2 + kb2) * 64];
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++)
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++) Qt[ct * 4 + kb] = op[(OP_Q / 8) + (ct * 4 + kb) * 64];
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; kb2++)
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++) At[ct * 2 + kb2] = op[(OP_A / 8) + (ct * 2 + kb2) * 64];
+        for (int i = 0; i < 4; i++) Kt[j][KORD[i]] = opb[cc * ost + kq0 + KORD[i] * 64];
+        gct[j] = gC[(size_t)cc * HV + h];
     }
     __builtin_amdgcn_sched_barrier(0);
-    for (int c = 0; c < NC; c++) {
-        const int cn = c + 1 < NC ? c + 1 : c;                                  // the last step re-reads its own record
-        const size_t recn = (size_t)cn * HV + h;
-        const half8* op = reinterpret_cast<const half8*>(ops + recn * OP_HALVES) + lane;
-        const f32x4* up = reinterpret_cast<const f32x4*>(U + recn * U_FLOATS + (size_t)sl * NCT * 256) + lane;
+    asm volatile("" ::: "memory");
 
+    // One chain step on FIFO entry j (a compile-time index: the steps are unrolled PB_DEP at a time).  Every MFMA is
+    // followed by the load that refills its operand for chunk c + PB_DEP and the scheduler is pinned to this order, so
+    // loads complete in the order of their use and the waits name exact counts.
+    auto step = [&](auto J, int c) {
+        constexpr int j = decltype(J)::value;
+        const int cn = min(c + PB_DEP, NC - 1);
+        const half8* on = opb + cn * ost;
+        reinterpret_cast<half8*>(sb_x)[w * 64 + lane] = pack_half8(ST[0], ST[1]);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                                           // E1
+        asm volatile("" ::: "memory");
         half8 Sb[4];
 #pragma unroll
-        for (int kb = 0; kb < 4; kb++) Sb[kb] = pack_half8(ST[2 * kb], ST[2 * kb + 1]);
-
-        // Every MFMA is followed by the load that refills its operand registers for the next chunk, and the scheduler is
-        // pinned to this order: loads then complete in the order in which the next chunk consumes them, so the waits stay
-        // partial (a reordered load would force a wait for all 60).  Independent accumulators alternate (ct / mt inner).
-        f32x4 D[NCT], Y[NCT];
-#pragma unroll
-        for (int ct = 0; ct < NCT; ct++) {
-            D[ct] = Ut[ct];
-            Ut[ct] = up[ct * 64];
-            Y[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+        for (int kb = 0; kb < 4; kb++) Sb[kb] = sbx[kb * 64];
+        // U joins after the MFMAs: as an accumulator input it would tie its FIFO register to the MFMA's destination
+        f32x4 D0 = f32x4{0.f, 0.f, 0.f, 0.f}, D1 = f32x4{0.f, 0.f, 0.f, 0.f};
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++)
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++) {
-                D[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Wt[ct * 4 + kb], Sb[kb], D[ct], 0, 0, 0);
-                Wt[ct * 4 + kb] = op[(OP_W / 8) + (ct * 4 + kb) * 64];
-            }
-        half8 Db[2];
-        Db[0] = pack_half8(D[0], D[1]);
-        Db[1] = pack_half8(D[2], D[3]);
-#pragma unroll
-        for (int mt = 0; mt < 8; mt++) ST[mt] *= gc;
-        gc = gC[recn];
+        D0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Wt[j][0], Sb[0], D0, 0, 0, 0);
+        Wt[j][0] = on[wq];
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; kb2++)
-#pragma unroll
-            for (int mt = 0; mt < 8; mt++) {
-                ST[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Kt[mt * 2 + kb2], Db[kb2], ST[mt], 0, 0, 0);
-                Kt[mt * 2 + kb2] = op[(OP_K / 8) + (mt * 2 + kb2) * 64];
-            }
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++)
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++) {
-                Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Qt[ct * 4 + kb], Sb[kb], Y[ct], 0, 0, 0);
-                Qt[ct * 4 + kb] = op[(OP_Q / 8) + (ct * 4 + kb) * 64];
-            }
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; kb2++)
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++) {
-                Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(At[ct * 2 + kb2], Db[kb2], Y[ct], 0, 0, 0);
-                At[ct * 2 + kb2] = op[(OP_A / 8) + (ct * 2 + kb2) * 64];
-            }
-        // hand the chunk's outputs to the helper wavefront
-        {
-            bf16_t* ys = y_s[c & 1];
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) ys[(ct * 16 + 4 * g + r) * 16 + n] = f2bf(Y[ct][r]);
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                      // the LDS writes have landed
-        __builtin_amdgcn_s_barrier();
+        D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Wt[j][1], Sb[1], D1, 0, 0, 0);
+        Wt[j][1] = on[wq + 64];
+        __builtin_amdgcn_sched_barrier(0);
+        D0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Wt[j][2], Sb[2], D0, 0, 0, 0);
+        Wt[j][2] = on[wq + 128];
+        __builtin_amdgcn_sched_barrier(0);
+        D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Wt[j][3], Sb[3], D1, 0, 0, 0);
+        Wt[j][3] = on[wq + 192];
+        __builtin_amdgcn_sched_barrier(0);
+        const f32x4 D = (D0 + D1) + Ut[j];
+        Ut[j] = upb[cn * ust];
+        __builtin_amdgcn_sched_barrier(0);
+        half4 dh;
+        dh[0] = (_Float16)D[0]; dh[1] = (_Float16)D[1]; dh[2] = (_Float16)D[2]; dh[3] = (_Float16)D[3];
+        // B-operand layout of D: k-block w / 2, halves 4 (w & 1) .. + 3 of the lane's eight
+        reinterpret_cast<half4*>(db_x)[((w >> 1) * 64 + lane) * 2 + (w & 1)] = dh;
+        ST[0] *= gct[j];
+        ST[1] *= gct[j];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                                           // E2
+        asm volatile("" ::: "memory");
+        const half8 Db0 = dbx[0], Db1 = dbx[64];
+        __builtin_amdgcn_sched_barrier(0);
+        ST[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Kt[j][0], Db0, ST[0], 0, 0, 0);
+        Kt[j][0] = on[kq0];
+        __builtin_amdgcn_sched_barrier(0);
+        ST[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Kt[j][2], Db0, ST[1], 0, 0, 0);
+        Kt[j][2] = on[kq0 + 128];
+        __builtin_amdgcn_sched_barrier(0);
+        ST[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Kt[j][1], Db1, ST[0], 0, 0, 0);
+        Kt[j][1] = on[kq0 + 64];
+        __builtin_amdgcn_sched_barrier(0);
+        ST[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Kt[j][3], Db1, ST[1], 0, 0, 0);
+        Kt[j][3] = on[kq0 + 192];
+        gct[j] = gC[(size_t)cn * HV + h];
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int c = 0;
+    for (; c + PB_DEP <= NC; c += PB_DEP) {
+        step(std::integral_constant<int, 0>{}, c);
+        step(std::integral_constant<int, 1>{}, c + 1);
+        step(std::integral_constant<int, 2>{}, c + 2);
+        step(std::integral_constant<int, 3>{}, c + 3);
     }
+    if (c < NC) step(std::integral_constant<int, 0>{}, c);
+    if (c + 1 < NC) step(std::integral_constant<int, 1>{}, c + 1);
+    if (c + 2 < NC) step(std::integral_constant<int, 2>{}, c + 2);
     {
-        float* sp = st_out + ((size_t)h * DV + sl * 16 + n) * DK;
-#pragma unroll
-        for (int mt = 0; mt < 8; mt++) *reinterpret_cast<f32x4*>(sp + mt * 16 + 4 * g) = ST[mt];
+        float* sp = st_out + ((size_t)h * DV + sl * 16 + n) * DK + w * 32 + 4 * g;
+        *reinterpret_cast<f32x4*>(sp) = ST[0];
+        *reinterpret_cast<f32x4*>(sp + 16) = ST[1];
     }
 }
+static_assert(PB_DEP == 4, "the chain loop is unrolled by hand for four FIFO entries");
 
+// Output kernel: Y_c = Qg_c S_c^T + Am_c D_c for one (chunk, head) per workgroup of 4 wavefronts; wavefront w covers the dv
+// slices 2w and 2w+1.  The 64 x 128 tile goes through LDS as bf16 and leaves either as y [S,16,128] or, with NORM, straight
+// through the gated RMSNorm (same arithmetic as the stand-alone kernel: 16 lanes per row, 8 columns each; batch.py:338-343).
+constexpr int YS_LD = DV + 8;
+template <bool NORM>
+__global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restrict__ ops, const _Float16* __restrict__ snap,
+                                                         bf16_t* __restrict__ y, const bf16_t* __restrict__ proj,
+                                                         const float* __restrict__ gw, float eps, int S) {
+    const int rec = blockIdx.x, c = rec / HV, h = rec % HV;
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    __shared__ __align__(16) bf16_t ys[C * YS_LD];
+    const half8* op = reinterpret_cast<const half8*>(ops + (size_t)rec * OP_HALVES) + lane;
+    const half8* sp = reinterpret_cast<const half8*>(snap + ((size_t)rec * 8 + 2 * w) * SNAP_HALVES) + lane;
+    half8 Sb[2][4], Db[2][2], Qt[16], At[8];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++) Sb[s][kb] = sp[s * (SNAP_HALVES / 8) + kb * 64];
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; kb2++) Db[s][kb2] = sp[s * (SNAP_HALVES / 8) + (SNAP_S / 8) + kb2 * 64];
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) Qt[i] = op[(OP_Q / 8) + i * 64];
+#pragma unroll
+    for (int i = 0; i < 8; i++) At[i] = op[(OP_A / 8) + i * 64];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        f32x4 Y[NCT];
+#pragma unroll
+        for (int ct = 0; ct < NCT; ct++) Y[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Qt[ct * 4 + kb], Sb[s][kb], Y[ct], 0, 0, 0);
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; kb2++)
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(At[ct * 2 + kb2], Db[s][kb2], Y[ct], 0, 0, 0);
+#pragma unroll
+        for (int ct = 0; ct < NCT; ct++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) ys[(ct * 16 + 4 * g + r) * YS_LD + (2 * w + s) * 16 + n] = f2bf(Y[ct][r]);
+    }
+    __syncthreads();
+    if (!NORM) {
+        const int row = threadIdx.x >> 2, q4 = threadIdx.x & 3;
+        const int t = c * C + row;
+        if (t < S) {
+            const uint4* src = reinterpret_cast<const uint4*>(&ys[row * YS_LD + q4 * 32]);
+            uint4* dst = reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV + q4 * 32);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[i] = src[i];
+        }
+    } else {
+        const int cc = threadIdx.x & 15;
+        float gwv[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) gwv[j] = gw[cc * 8 + j];
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int row = it * 16 + (threadIdx.x >> 4);
+            const int t = c * C + row;
+            if (t >= S) continue;                                               // whole 16-lane groups leave together
+            const uint4 yv = *reinterpret_cast<const uint4*>(&ys[row * YS_LD + cc * 8]);
+            const uint4 zv = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
+            const uint32_t yw[4] = {yv.x, yv.y, yv.z, yv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
+            float yy[8], zz[8];
+            double ss = 0.0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                yy[2 * j] = lo_bf(yw[j]);
+                yy[2 * j + 1] = hi_bf(yw[j]);
+                zz[2 * j] = lo_bf(zw[j]);
+                zz[2 * j + 1] = hi_bf(zw[j]);
+                ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
+            }
+            const float inv = rsqrt_rn((float)row16_sum_d(ss) / 128.f + eps);
+            uint32_t o[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv));
+            reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV)[cc] =
+                make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
+        }
+    }
+}
 
 // ------------------------------------------------------------------------------------------------------------------
 // Phase A: one workgroup of 256 threads per (chunk, head).
@@ -496,17 +575,43 @@ long qt_gdn_chunk_ops_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C)
 long qt_gdn_chunk_u_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * U_FLOATS * 4; }
 long qt_gdn_chunk_gc_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * 4; }
 
-int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, const float* state_in, float* state_out, void* y, int S,
-                   hipStream_t stream) {
-    if (!ops || !U || !gC || !state_in || !state_out || !y) return QT_ERR_NULL;
+static int phase_b_launch(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
+                          void* y, const void* proj, const float* gw, float eps, bool norm, int S, hipStream_t stream) {
+    if (!ops || !U || !gC || !snap || !state_in || !state_out || !y) return QT_ERR_NULL;
+    if (norm && (!proj || !gw)) return QT_ERR_NULL;
     if (S < 0) return QT_ERR_DIM;
-    for (const void* p : {ops, (const void*)U, (const void*)state_in, (const void*)state_out})
+    for (const void* p : {ops, (const void*)U, (const void*)snap, (const void*)state_in, (const void*)state_out, (const void*)y, proj})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     const int NC = (S + C - 1) / C;
-    hipLaunchKernelGGL(gdn_phase_b_kernel, dim3(HV * 8), dim3(128), 0, stream, (const _Float16*)ops, U, gC, state_in, state_out,
-                       (bf16_t*)y, S, NC);
+    if (NC == 0) {
+        if (state_out != state_in &&
+            hipMemcpyAsync(state_out, state_in, sizeof(float) * HV * DV * DK, hipMemcpyDeviceToDevice, stream) != hipSuccess)
+            return QT_ERR_LAUNCH;
+        return QT_OK;
+    }
+    hipLaunchKernelGGL(gdn_chain_kernel, dim3(HV * 8), dim3(320), 0, stream, (const _Float16*)ops, U, gC, state_in, state_out,
+                       (_Float16*)snap, NC);
+    QT_CHECK_LAUNCH();
+    if (norm)
+        hipLaunchKernelGGL(gdn_output_kernel<true>, dim3(NC * HV), dim3(256), 0, stream, (const _Float16*)ops,
+                           (const _Float16*)snap, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S);
+    else
+        hipLaunchKernelGGL(gdn_output_kernel<false>, dim3(NC * HV), dim3(256), 0, stream, (const _Float16*)ops,
+                           (const _Float16*)snap, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S);
     QT_CHECK_LAUNCH();
     return QT_OK;
+}
+
+long qt_gdn_chunk_snap_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * 8 * SNAP_HALVES * 2; }
+
+int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out, void* y,
+                   int S, hipStream_t stream) {
+    return phase_b_launch(ops, U, gC, snap, state_in, state_out, y, nullptr, nullptr, 0.f, false, S, stream);
+}
+
+int qt_gdn_phase_b_norm(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
+                        const void* proj, const float* gw, float eps, void* out, int S, hipStream_t stream) {
+    return phase_b_launch(ops, U, gC, snap, state_in, state_out, out, proj, gw, eps, true, S, stream);
 }
 
 int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v, const float* A_log, const float* dt_bias,

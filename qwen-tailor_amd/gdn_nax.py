@@ -57,17 +57,35 @@ def gdn_chunked(q, k, v, proj, A_log, dt_bias, state, relaxed=True, flags=DEFAUL
     return phase_b(q, k, v, ops, U, gC, state)
 
 
-def phase_b(q, k, v, Tb, Am, gv, state, relaxed=True, flags=DEFAULT_FLAGS, tg=None):
-    """The serial state recurrence on the outputs of phase A -> y [S,16,128] bf16, new state [1,16,128,128] f32
-    (qwen35/gdn_nax.py:404-410).  Tb / Am / gv are the records prep_a (or gdn_chunked's phase A) produced."""
-    S = q.shape[0]
+def _phase_b_args(S, Tb, Am, gv, state):
     ops, U, gC = L.dev(Tb, torch.float16, "Tb"), L.dev(Am, torch.float32, "Am"), L.dev(gv, torch.float32, "gv")
     lib = L.lib()
     if ops.numel() * 2 < lib.qt_gdn_chunk_ops_bytes(S) or U.numel() * 4 < lib.qt_gdn_chunk_u_bytes(S) or \
             gC.numel() * 4 < lib.qt_gdn_chunk_gc_bytes(S):
         raise ValueError("phase_b: the phase A records are too small for this many tokens")
     state = L.dev(state, torch.float32, "state").reshape(1, HV, DV, DK)
+    snap = torch.empty(max(lib.qt_gdn_chunk_snap_bytes(S) // 2, 8), dtype=torch.float16, device=state.device)
+    return ops, U, gC, snap, state, torch.empty_like(state)
+
+
+def phase_b(q, k, v, Tb, Am, gv, state, relaxed=True, flags=DEFAULT_FLAGS, tg=None):
+    """The serial state recurrence on the outputs of phase A -> y [S,16,128] bf16, new state [1,16,128,128] f32
+    (qwen35/gdn_nax.py:404-410).  Tb / Am / gv are the records prep_a (or gdn_chunked's phase A) produced."""
+    S = q.shape[0]
+    ops, U, gC, snap, state, out = _phase_b_args(S, Tb, Am, gv, state)
     y = torch.empty((S, HV, DV), dtype=BF16, device=state.device)
-    out = torch.empty_like(state)
-    L.call("qt_gdn_phase_b", L.ptr(ops), L.ptr(U), L.ptr(gC), L.ptr(state), L.ptr(out), L.ptr(y), S, L.stream())
+    L.call("qt_gdn_phase_b", L.ptr(ops), L.ptr(U), L.ptr(gC), L.ptr(snap), L.ptr(state), L.ptr(out), L.ptr(y), S, L.stream())
     return y, out
+
+
+def phase_b_norm(proj, Tb, Am, gv, state, gw, eps=1e-6):
+    """phase_b followed by prefill.gated_norm (qwen35/prefill.py:241-244) in one pass: the outputs never leave the chip
+    un-normalised.  proj [S,8224] bf16 supplies z; gw [128].  -> out [S,2048] bf16, new state [1,16,128,128] f32."""
+    proj = L.dev(proj, BF16, "proj", (None, PW))
+    S = proj.shape[0]
+    ops, U, gC, snap, state, new_state = _phase_b_args(S, Tb, Am, gv, state)
+    gw = L.f32(gw, "gw", (DV,))
+    out = torch.empty((S, HV * DV), dtype=BF16, device=state.device)
+    L.call("qt_gdn_phase_b_norm", L.ptr(ops), L.ptr(U), L.ptr(gC), L.ptr(snap), L.ptr(state), L.ptr(new_state), L.ptr(proj),
+           L.ptr(gw), float(eps), L.ptr(out), S, L.stream())
+    return out, new_state

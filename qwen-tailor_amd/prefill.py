@@ -28,14 +28,15 @@ def gdn_core(proj, conv_state, ssm_state, conv_w, A_log, dt_bias, gnorm, want_qk
     cs = conv_state.reshape(3, CD)
     if GDN_IMPL == "nax":
         q, k, v, ops, U, gC = gdn_nax._phase_a(proj, cs, conv_w, A_log, dt_bias)
-        out, new_ssm = gdn_nax.phase_b(proj, None, None, ops, U, gC, ssm_state)
+        normed, new_ssm = gdn_nax.phase_b_norm(proj, ops, U, gC, ssm_state, gnorm)
     else:
         q, k, v = conv_prep(proj, cs, conv_w)
         out, new_ssm = gated_delta.gated_delta_update(q[None], k[None], v[None], proj[:, 8208:][None], proj[:, 8192:8208][None],
                                                       A_log, dt_bias, ssm_state.reshape(1, HV, DV, DK))
+        normed = gated_norm(out.reshape(S, HV * DV), proj, gnorm)
     tail = proj[:, :CD]
     new_conv = (tail[S - 3:] if S >= 3 else torch.cat([cs, tail], dim=0)[-3:])[None].contiguous()   # prefill.py:262-263
-    return gated_norm(out.reshape(S, HV * DV), proj, gnorm), new_conv, new_ssm.reshape(1, HV, DV, DK)
+    return normed, new_conv, new_ssm.reshape(1, HV, DV, DK)
 
 
 def conv_prep(proj, conv_state, conv_w):
