@@ -183,14 +183,23 @@ def bench_attn(torch, qt, dev, B, M, lo, hi, seed):
     slots = torch.from_numpy(rng.permutation(B).astype(np.int32)).to(dev)
     g = torch.Generator().manual_seed(seed)
     bf = torch.bfloat16
-    Kp = torch.randn((B + 1, 2, Lmax, 256), generator=g).to(bf).to(dev)
-    Vp = torch.randn((B + 1, 2, Lmax, 256), generator=g).to(bf).to(dev)
+    nbytes = int(pos.sum().item()) * 2 * 2 * 256 * 2                  # K and V rows of both KV heads, read once
+    # a step's K / V must come from HBM, not from the 256 MB last-level cache: rotate over enough pools (layers) to exceed it
+    n_pools = max(2, min(16, -(-1100000000 // nbytes)))
+    Kp0 = torch.randn((B + 1, 2, Lmax, 256), generator=g).to(bf).to(dev)
+    Vp0 = torch.randn((B + 1, 2, Lmax, 256), generator=g).to(bf).to(dev)
+    pools = [(Kp0, Vp0)] + [(Kp0.clone(), Vp0.clone()) for _ in range(n_pools - 1)]
     q = torch.randn((B * M, 8, 256), generator=g).to(bf).to(dev)
     kn = torch.randn((B * M, 2, 256), generator=g).to(bf).to(dev)
     vn = torch.randn((B * M, 2, 256), generator=g).to(bf).to(dev)
-    t = time_graph(torch, lambda: qt.batch.attn_b(q, kn, vn, Kp, Vp, slots, pos, M), reps=100, inner=5)
-    nbytes = int(pos.sum().item()) * 2 * 2 * 256 * 2                  # K and V rows of both KV heads, read once
-    return {"B": B, "M": M, "sum_L": int(pos.sum().item()), "us": t * 1e6, "bytes": nbytes, "GBps": nbytes / t / 1e9,
+    it = [0]
+
+    def step():
+        Kp, Vp = pools[it[0] % n_pools]
+        it[0] += 1
+        qt.batch.attn_b(q, kn, vn, Kp, Vp, slots, pos, M)
+    t = time_graph(torch, step, reps=n_pools * 12, inner=n_pools)
+    return {"B": B, "M": M, "pools": n_pools, "sum_L": int(pos.sum().item()), "us": t * 1e6, "bytes": nbytes, "GBps": nbytes / t / 1e9,
             "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
 
 

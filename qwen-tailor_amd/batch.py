@@ -47,9 +47,11 @@ def _workspace(dev, nbytes):
     return buf
 
 
-def split_size(Lmax: int) -> int:
-    """keys per split-K workgroup"""
-    return 256 if Lmax <= 4096 else (512 if Lmax <= 16384 else 1024)
+def split_size(Lmax: int, B: int = 16) -> int:
+    """keys per split-K workgroup: aims at roughly 768 workgroups for full pools (about half of that in a ragged batch),
+    a few per CU, each long enough that a wavefront streams several tiles per partial result it writes"""
+    ch = (2 * B * Lmax // 768 + 64) // 128 * 128
+    return max(256, min(1024, ch))
 
 
 def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None):
@@ -66,7 +68,7 @@ def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None):
     Vp = L.dev(Vp, BF16, "Vp", tuple(Kp.shape))
     n_slots, Lmax = Kp.shape[0], Kp.shape[2]
     slots, pos = L.i32(slots, "slots", B), L.i32(pos, "pos", B)
-    CH = split or split_size(Lmax)
+    CH = split or split_size(Lmax, B)
     nbytes = L.lib().qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)
     if nbytes < 0:
         raise ValueError("attn_b: bad split size")

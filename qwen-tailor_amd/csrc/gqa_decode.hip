@@ -6,7 +6,13 @@
 // Split-K: workgroup (b, kv head, split s) streams the pool keys [s*CH, min((s+1)*CH, pos[b])) ONCE for all 4*M query
 // rows that share the KV head, so K and V are read from HBM exactly once per step.
 //   scores : S^T[16 keys x 16 rows] = K_tile[16 x 256] . Q^T[256 x 16] on bf16 MFMA (16x16x32), K straight from HBM
-//   P . V  : on the vector ALU, lane l owns output columns 4l .. 4l+3 of every row; probabilities are broadcast through LDS
+//   P . V  : O[16 rows x 256] += P[16 x 16 keys] . V[16 keys x 256] on bf16 MFMA (16x16x16): the transposed scores in
+//            their accumulator layout ARE the A operand; the V tile is parked row-major in LDS and read back through the
+//            transposing LDS load (ds_read_b64_tr_b16), which delivers the B operand (4 consecutive keys of one column).
+//            P is split into two bf16 terms (p = hi + lo, error 2^-17), so the product keeps fp32-like accuracy.
+// Each wavefront walks its tiles with a one-tile-deep register FIFO: the registers of a K (V) fragment are refilled with
+// the next tile's fragment right after the MFMA (LDS store) that consumed them, so a tile's loads fly during the previous
+// tile's arithmetic.  The loop issues loads only, in the order of their use, which keeps every vmcnt wait partial.
 // Each wavefront keeps its own online-softmax state (m, l, O); the 4 wavefronts of a workgroup are merged through LDS and
 // the workgroup writes one unnormalised partial (m, l, O) per row; a second kernel merges the splits (batch.py:203-221).
 #include "qt_common.h"
@@ -16,37 +22,27 @@ using namespace qt;
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GQA = AH / AKV;          // 4 query heads per KV head
 constexpr float SCALE = 0.0625f;       // 256^-0.5, batch.py:177
 constexpr float NEG = -3.0e38f;
+constexpr int VL_LD = AD + 16;         // row stride (elements) of the V tile in LDS: 544 bytes spread the 16 rows over the banks
 
-__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// One tile of up to 16 keys for one wavefront.  kt / vt point at the first key's row (256 bf16, row stride `stride`
-// elements); keys [0, nvalid) exist; `causal0` >= 0 marks new keys: key i is visible to query token j only if i <= j.
-template <int M>
-__device__ __forceinline__ void tile_step(const bf16_t* __restrict__ kt, const bf16_t* __restrict__ vt, size_t stride, int nvalid,
-                                          bool causal, const bf16x8 (&bq)[8], float& m_run, float& l_run, float (&o)[4 * M][4],
-                                          float* p_lds, float* c_lds, int lane) {
+// Online-softmax update of one tile of 16 keys from its transposed scores: lane (row n, group g) holds keys 4g .. 4g+3.
+// Leaves the probabilities of those keys in p (fp32) and writes the row's rescale factor to c_lds[row].
+__device__ __forceinline__ void softmax_tile(const f32x4& acc, int nvalid, bool causal, float& m_run, float& l_run, float (&p)[4],
+                                             float* c_lds, int lane) {
     const int n = lane & 15, g = lane >> 4;
-    // ---- scores, transposed: lane (row n, group g) gets keys 4g .. 4g+3
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    {
-        const int key = n < nvalid ? n : 0;                      // rows past the end re-read key 0 and are masked below
-        const uint4* kr = reinterpret_cast<const uint4*>(kt + (size_t)key * stride);
-        uint4 a[8];
-#pragma unroll
-        for (int kb = 0; kb < 8; kb++) a[kb] = kr[kb * 4 + g];
-#pragma unroll
-        for (int kb = 0; kb < 8; kb++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[kb]), bq[kb], acc, 0, 0, 0);
-    }
     const int jq = n / GQA;                                      // query token of this row (rows >= 4*M are padding)
     float s[4], mx = NEG;
 #pragma unroll
@@ -63,61 +59,62 @@ __device__ __forceinline__ void tile_step(const bf16_t* __restrict__ kt, const b
     float ps = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const float p = s[i] > 0.5f * NEG ? __expf(s[i] - m_new) : 0.f;
-        ps += p;
-        p_lds[(4 * g + i) * 16 + n] = p;
+        p[i] = s[i] > 0.5f * NEG ? __expf(s[i] - m_new) : 0.f;
+        ps += p[i];
     }
     l_run = l_run * corr + ps;                                   // this lane's share; summed over g at the end
     m_run = m_new;
     if (g == 0) c_lds[n] = corr;
-    wave_lds_sync();
-    // ---- O += P V, lane owns columns 4*lane .. 4*lane+3
+}
+
+// O (16 rows x 256, accumulator layout: block j, lane (column 16 j + n, group g), rows 4g .. 4g+3) = c * O + P . V for the
+// V tile in v_lds ([16 keys][VL_LD]).  p: this lane's probabilities (row n, keys 4g .. 4g+3).
+__device__ __forceinline__ void pv_tile(f32x4 (&O)[16], const float (&p)[4], const bf16_t* v_lds, const float* c_lds, int lane) {
+    const int n = lane & 15, g = lane >> 4;
+    s16x4 ph, pl;
 #pragma unroll
-    for (int r = 0; r < 4 * M; r += 4) {
-        const f32x4 c4 = *reinterpret_cast<const f32x4*>(c_lds + r);
-#pragma unroll
-        for (int rr = 0; rr < 4; rr++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) o[r + rr][e] *= c4[rr];
+    for (int i = 0; i < 4; i++) {
+        const bf16_t h = f2bf(p[i]);
+        ph[i] = (short)h;
+        pl[i] = (short)f2bf(p[i] - bf2f(h));
     }
-#pragma unroll 4
-    for (int key = 0; key < 16; key++) {
-        if (key < nvalid) {
-            const uint2 vv = reinterpret_cast<const uint2*>(vt + (size_t)key * stride)[lane];
-            const float v4[4] = {lo_bf(vv.x), hi_bf(vv.x), lo_bf(vv.y), hi_bf(vv.y)};
+    const f32x4 c4 = *reinterpret_cast<const f32x4*>(c_lds + 4 * g);
+    // transposing load: within a group of 16 lanes, lane 4q + i receives element i of the 8-byte chunks addressed by lanes
+    // q, q+4, q+8, q+12.  Lane j' = n of group g points at key 4g + n/4, columns 4 (n%4) .. + 3 of the block: lane n then
+    // receives keys 4g .. 4g+3 of column n, the B operand.
+    const bf16_t* vrow = v_lds + (4 * g + (n >> 2)) * VL_LD + 4 * (n & 3);
 #pragma unroll
-            for (int r = 0; r < 4 * M; r += 4) {
-                const f32x4 p4 = *reinterpret_cast<const f32x4*>(p_lds + key * 16 + r);
-#pragma unroll
-                for (int rr = 0; rr < 4; rr++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) o[r + rr][e] = fmaf(p4[rr], v4[e], o[r + rr][e]);
-            }
-        }
+    for (int j = 0; j < 16; j++) {
+        const s16x4 B = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(vrow + 16 * j)));
+        O[j] *= c4;
+        O[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ph, B, O[j], 0, 0, 0);
+        O[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pl, B, O[j], 0, 0, 0);
     }
-    wave_lds_sync();
 }
 
 // partial results of one workgroup: part_o [(b*KV + kvh)*nsplit + s][4*M rows][256] f32 (unnormalised),
 // part_ml [...][4*M][2] = (running max, running sum)
 template <int M>
-__global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_new,
+__global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_new,
                                                            const bf16_t* __restrict__ v_new, bf16_t* Kp, bf16_t* Vp,
                                                            const int* __restrict__ slots, const int* __restrict__ pos,
                                                            float* __restrict__ part_o, float* __restrict__ part_ml, int Lmax,
                                                            int CH, int nsplit, int n_slots) {
     constexpr int R = 4 * M;
-    __shared__ __align__(16) float p_s[4][16 * 16];
+    __shared__ __align__(16) bf16_t v_s[4][16 * VL_LD];          // one V tile per wavefront; reused for the merged O below
     __shared__ __align__(16) float c_s[4][16];
     __shared__ float m_s[4][16], l_s[4][16];
-    __shared__ __align__(16) float o_s[R][AD];
+    static_assert(sizeof(bf16_t) * 4 * 16 * VL_LD >= sizeof(float) * 16 * AD, "the merged O tile must fit into the V tiles");
+    float (*o_s)[AD] = reinterpret_cast<float (*)[AD]>(&v_s[0][0]);
 
     const int s = blockIdx.x % nsplit, bk = blockIdx.x / nsplit, kvh = bk % AKV, b = bk / AKV;
     const int slot = slots[b], p0 = pos[b];
     if ((unsigned)slot >= (unsigned)n_slots || p0 < 0 || p0 + M > Lmax) return;
     const int lo = s * CH, hi = min(lo + CH, p0);
     if (s > 0 && lo >= p0) return;                               // nothing to do for this split (split 0 always runs)
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int hw = lane >> 5, cl = lane & 31;
 
     // Q^T as the MFMA B operand: lane (row n, group g) holds q[row n][32 kb + 8 g .. + 8]; row n = token (n / 4), head n % 4
     bf16x8 bq[8];
@@ -126,63 +123,127 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
         const bf16_t* qr = q + ((size_t)(b * M + (real ? n / GQA : 0)) * AH + kvh * GQA + (n % GQA)) * AD;
 #pragma unroll
         for (int kb = 0; kb < 8; kb++) {
-            uint4 v = reinterpret_cast<const uint4*>(qr)[kb * 4 + g];
-            if (!real) v = make_uint4(0, 0, 0, 0);
+            u32x4 v = reinterpret_cast<const u32x4*>(qr)[kb * 4 + g];
+            if (!real) v = u32x4{0, 0, 0, 0};
             bq[kb] = as_bf16x8(v);
         }
     }
-    float m_run = NEG, l_run = 0.f, o[R][4];
+    float m_run = NEG, l_run = 0.f;
+    f32x4 O[16];
 #pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) o[r][e] = 0.f;
+    for (int j = 0; j < 16; j++) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const size_t pbase = ((size_t)slot * AKV + kvh) * Lmax * AD;
+    const bf16_t* kbase = Kp + pbase;
+    const bf16_t* vbase = Vp + pbase;
+    bf16_t* vl = v_s[w];
     const int ntiles = hi > lo ? (hi - lo + 15) / 16 : 0;
-    for (int t = w; t < ntiles; t += 4) {
-        const int key0 = lo + t * 16;
-        tile_step<M>(Kp + pbase + (size_t)key0 * AD, Vp + pbase + (size_t)key0 * AD, AD, min(16, hi - key0), false, bq, m_run,
-                     l_run, o, p_s[w], c_s[w], lane);
+    if (w < ntiles) {
+        // fragment addresses of a tile; keys past `hi` re-read the tile's first key (they are masked / weighted by 0)
+        auto k_ptr = [&](int t) {
+            const int key0 = lo + t * 16;
+            return reinterpret_cast<const u32x4*>(kbase + (size_t)(key0 + n < hi ? key0 + n : key0) * AD) + g;
+        };
+        auto v_ptr = [&](int t, int i) {
+            const int key0 = lo + t * 16, key = key0 + 2 * i + hw;
+            return reinterpret_cast<const u32x4*>(vbase + (size_t)(key < hi ? key : key0) * AD) + cl;
+        };
+        u32x4 a[8], vv[8];
+        {
+            const u32x4* kr = k_ptr(w);
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) a[kb] = kr[kb * 4];
+#pragma unroll
+            for (int i = 0; i < 8; i++) vv[i] = *v_ptr(w, i);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        for (int t = w; t < ntiles; t += 4) {
+            const int tn = t + 4 < ntiles ? t + 4 : t;           // the last step re-reads its own tile
+            const int nvalid = min(16, hi - (lo + t * 16));
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            const u32x4* kr = k_ptr(tn);
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[kb]), bq[kb], acc, 0, 0, 0);
+                a[kb] = kr[kb * 4];
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            float p[4];
+            softmax_tile(acc, nvalid, false, m_run, l_run, p, c_s[w], lane);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                // keys 2i (lower half wavefront) and 2i+1 (upper half), 8 columns per lane
+                *reinterpret_cast<u32x4*>(vl + (2 * i + hw) * VL_LD + 8 * cl) = vv[i];
+                vv[i] = *v_ptr(tn, i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            wave_lds_sync();
+            pv_tile(O, p, vl, c_s[w], lane);
+            wave_lds_sync();
+        }
     }
     if (s == 0 && w == 3) {
-        // the M new keys of this sequence, straight from the inputs (batch.py:143-145), with the causal tail among them
+        // The M new keys of this sequence, straight from the inputs (batch.py:143-145), with the causal rule among them:
+        // key i is visible to query token j only if i <= j.  Not pipelined: it runs once per sequence.
         const bf16_t* kn = k_new + ((size_t)b * M * AKV + kvh) * AD;
         const bf16_t* vn = v_new + ((size_t)b * M * AKV + kvh) * AD;
-        tile_step<M>(kn, vn, (size_t)AKV * AD, M, true, bq, m_run, l_run, o, p_s[w], c_s[w], lane);
+        const size_t stride = (size_t)AKV * AD;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        {
+            const u32x4* kr = reinterpret_cast<const u32x4*>(kn + (size_t)(n < M ? n : 0) * stride);
+            u32x4 a[8];
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) a[kb] = kr[kb * 4 + g];
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[kb]), bq[kb], acc, 0, 0, 0);
+        }
+        float p[4];
+        softmax_tile(acc, M, true, m_run, l_run, p, c_s[w], lane);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int key = 2 * i + hw;                          // rows past the M new keys are zero: their weight is 0
+            u32x4 v = u32x4{0, 0, 0, 0};
+            if (key < M) v = reinterpret_cast<const u32x4*>(vn + (size_t)key * stride)[cl];
+            *reinterpret_cast<u32x4*>(vl + key * VL_LD + 8 * cl) = v;
+        }
+        wave_lds_sync();
+        pv_tile(O, p, vl, c_s[w], lane);
+        wave_lds_sync();
     }
     if (s == 0 && w == 0) {
         // append (batch.py:196-201): row j of this sequence goes to pool position p0 + j
         for (int j = 0; j < M; j++) {
             const uint2 kk = reinterpret_cast<const uint2*>(k_new + ((size_t)(b * M + j) * AKV + kvh) * AD)[lane];
-            const uint2 vv = reinterpret_cast<const uint2*>(v_new + ((size_t)(b * M + j) * AKV + kvh) * AD)[lane];
+            const uint2 vv2 = reinterpret_cast<const uint2*>(v_new + ((size_t)(b * M + j) * AKV + kvh) * AD)[lane];
             reinterpret_cast<uint2*>(Kp + pbase + (size_t)(p0 + j) * AD)[lane] = kk;
-            reinterpret_cast<uint2*>(Vp + pbase + (size_t)(p0 + j) * AD)[lane] = vv;
+            reinterpret_cast<uint2*>(Vp + pbase + (size_t)(p0 + j) * AD)[lane] = vv2;
         }
     }
 
-    // ---- merge the 4 wavefronts (deterministic order)
+    // ---- merge the 4 wavefronts (deterministic order); lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
     if (g == 0) {
         m_s[w][n] = m_run;
         l_s[w][n] = l_run;
     }
-    __syncthreads();
-    float f[R];
+    __syncthreads();                                             // also: every wavefront is done with its V tile
+    float f[4];
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        const float mm = fmaxf(fmaxf(m_s[0][r], m_s[1][r]), fmaxf(m_s[2][r], m_s[3][r]));
-        f[r] = __expf(m_s[w][r] - mm);
+    for (int r = 0; r < 4; r++) {
+        const int row = 4 * g + r;
+        const float mm = fmaxf(fmaxf(m_s[0][row], m_s[1][row]), fmaxf(m_s[2][row], m_s[3][row]));
+        f[r] = __expf(m_s[w][row] - mm);
     }
     for (int ww = 0; ww < 4; ww++) {
-        if (w == ww) {
+        if (w == ww && 4 * g < R) {
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                f32x4* dst = reinterpret_cast<f32x4*>(&o_s[r][lane * 4]);
-                f32x4 cur = ww == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : *dst;
-                cur[0] += o[r][0] * f[r]; cur[1] += o[r][1] * f[r]; cur[2] += o[r][2] * f[r]; cur[3] += o[r][3] * f[r];
-                *dst = cur;
-            }
+            for (int j = 0; j < 16; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float* dst = &o_s[4 * g + r][16 * j + n];
+                    *dst = (ww == 0 ? 0.f : *dst) + O[j][r] * f[r];
+                }
         }
         __syncthreads();
     }
@@ -198,29 +259,58 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(const bf16_t* __restr
     }
 }
 
-// merge of the splits: one workgroup of 256 threads per (sequence, kv head); thread d owns output column d of every row
+// merge of the splits: one workgroup of 256 threads per (sequence, kv head, row).  The per-split factors exp(m_s - m) are
+// computed by one thread each; then wavefront w sums the splits s = w, w+4, ... (a lane owns 4 output columns, four splits'
+// loads in flight) and the four wavefronts are added in order.
+constexpr int MAX_SPLITS = 4096;
 template <int M>
 __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                          const int* __restrict__ slots, const int* __restrict__ pos,
                                                          bf16_t* __restrict__ out, int Lmax, int CH, int nsplit, int n_slots) {
     constexpr int R = 4 * M;
-    const int kvh = blockIdx.x % AKV, b = blockIdx.x / AKV, d = threadIdx.x;
+    __shared__ float fs_s[MAX_SPLITS];
+    __shared__ float red_m[4], red_l[4];
+    __shared__ __align__(16) float acc_s[4][AD];
+    const int r = blockIdx.x % R, bk = blockIdx.x / R, kvh = bk % AKV, b = bk / AKV;
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
     const int slot = slots[b], p0 = pos[b];
     if ((unsigned)slot >= (unsigned)n_slots || p0 < 0 || p0 + M > Lmax) return;
     const int ns = max(1, min(nsplit, (p0 + CH - 1) / CH));
-    const size_t base = (size_t)blockIdx.x * nsplit;
-    for (int r = 0; r < R; r++) {
-        float mm = NEG;
-        for (int s = 0; s < ns; s++) mm = fmaxf(mm, part_ml[((base + s) * R + r) * 2]);
-        float l = 0.f, acc = 0.f;
-        for (int s = 0; s < ns; s++) {
-            const float fs = __expf(part_ml[((base + s) * R + r) * 2] - mm);
-            l += part_ml[((base + s) * R + r) * 2 + 1] * fs;
-            acc += part_o[((base + s) * R + r) * AD + d] * fs;
-        }
-        const float ov = l == 0.f ? acc : acc / l;                                   // batch.py:216
-        out[((size_t)(b * M + r / GQA) * AH + kvh * GQA + (r % GQA)) * AD + d] = f2bf(ov);
+    const size_t base = (size_t)bk * nsplit;
+    const float* ml = part_ml + (base * R + r) * 2;              // split stride 2 R floats
+    const float* po = part_o + (base * R + r) * AD + lane * 4;   // split stride R * AD floats
+    float mx = NEG;
+    for (int s = tid; s < ns; s += 256) mx = fmaxf(mx, ml[(size_t)s * 2 * R]);
+    mx = wave_max(mx);
+    if (lane == 0) red_m[w] = mx;
+    __syncthreads();
+    const float mm = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
+    float lp = 0.f;
+    for (int s = tid; s < ns; s += 256) {
+        const float f = __expf(ml[(size_t)s * 2 * R] - mm);
+        fs_s[s] = f;
+        lp += ml[(size_t)s * 2 * R + 1] * f;
     }
+    lp = wave_sum(lp);
+    if (lane == 0) red_l[w] = lp;
+    __syncthreads();
+    const float l = (red_l[0] + red_l[1]) + (red_l[2] + red_l[3]);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    int s = w;
+    for (; s + 12 < ns; s += 16) {
+        f32x4 ov[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) ov[i] = *reinterpret_cast<const f32x4*>(po + (size_t)(s + 4 * i) * R * AD);
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc += ov[i] * fs_s[s + 4 * i];
+    }
+    for (; s < ns; s += 4) acc += *reinterpret_cast<const f32x4*>(po + (size_t)s * R * AD) * fs_s[s];
+    *reinterpret_cast<f32x4*>(&acc_s[w][lane * 4]) = acc;
+    __syncthreads();
+    const int d = tid;
+    const float a = (acc_s[0][d] + acc_s[1][d]) + (acc_s[2][d] + acc_s[3][d]);
+    const float ov = l == 0.f ? a : a / l;                                           // batch.py:216
+    out[((size_t)(b * M + r / GQA) * AH + kvh * GQA + (r % GQA)) * AD + d] = f2bf(ov);
 }
 
 }  // namespace
@@ -245,9 +335,10 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if (workspace_bytes < qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)) return -6;
     const int nsplit = (Lmax + CH - 1) / CH;
+    if (nsplit > MAX_SPLITS) return QT_ERR_UNSUPPORTED;
     float* part_o = (float*)workspace;
     float* part_ml = part_o + (size_t)B * AKV * nsplit * (4 * M) * AD;
-    const dim3 g1((unsigned)(B * AKV * nsplit)), g2((unsigned)(B * AKV));
+    const dim3 g1((unsigned)(B * AKV * nsplit)), g2((unsigned)(B * AKV * 4 * M));
 #define QT_ATTN_LAUNCH(MM)                                                                                                \
     hipLaunchKernelGGL(attn_partial_kernel<MM>, g1, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)k_new,         \
                        (const bf16_t*)v_new, (bf16_t*)Kp, (bf16_t*)Vp, slots, pos, part_o, part_ml, Lmax, CH, nsplit, n_slots); \

@@ -98,6 +98,10 @@ def test_chunked_prefill_vs_sequential_oracle(qt, dev, T):
     y2, s2 = qt.gdn_nax.gdn_chunked(q, k, v, dproj, to_dev(A_log, dev), to_dev(dtb, dev), to_dev(S0[None], dev))
     check_tensors_equal("gdn_chunked y", y2, y)
     check_tensors_equal("gdn_chunked state", s2, s1)
+    # the output kernel with the gated norm fused in gives the bits of the two separate kernels
+    out3, s3 = qt.gdn_nax.phase_b_norm(dproj, ops, U, gC, to_dev(S0[None], dev), to_dev(gw, dev))
+    check_tensors_equal("fused gated norm", out3, out)
+    check_tensors_equal("fused gated norm state", s3, s1)
 
 
 @pytest.mark.parametrize("T", [512, 2048])
@@ -113,3 +117,9 @@ def test_config2_chunked_prefill(qt, dev, T):
     e2 = check_rel("y rel-L2", to_np(y).reshape(T, 2048), oy, 2e-3, rel_l2)
     e3 = check_rel("gated output rel-L2", to_np(out), oo, 2e-3, rel_l2)
     print(f"T={T}: state {e1:.2e}, y {e2:.2e}, out {e3:.2e}")
+    # the layer core (fused output + norm kernel) returns the same bits, and the conv tail of prefill.py:262-263
+    o4, conv4, s4 = qt.prefill.gdn_core(dproj, to_dev(cs[None], dev, BF16), to_dev(S0[None], dev), to_dev(cw, dev, BF16),
+                                        to_dev(A_log, dev), to_dev(dtb, dev), to_dev(gw, dev))
+    check_tensors_equal("gdn_core output", o4, out)
+    check_tensors_equal("gdn_core state", s4, s1)
+    check_equal("gdn_core conv tail", to_np(conv4)[0], otail)
