@@ -6,7 +6,6 @@ from __future__ import annotations
 import torch
 
 from . import _lib as L
-from .batch import _workspace
 
 BF16 = torch.bfloat16
 
@@ -33,8 +32,6 @@ def scaled_dot_product_attention(q, k, v, *, scale: float, mask="causal"):
         raise ValueError("fewer keys than queries")
     q = q.contiguous()
     out = torch.empty_like(q)
-    nbytes = L.lib().qt_gqa_prefill_workspace_bytes(Lk)
-    ws = _workspace(q.device, nbytes)
-    L.call("qt_gqa_prefill_causal", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(ws), ws.numel(), S, Lk, Lk - S, S * 256,
-           k.stride(1), L.stream())
+    L.call("qt_gqa_prefill_causal", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), None, 0, S, Lk, Lk - S, S * 256, k.stride(1),
+           L.stream())
     return out

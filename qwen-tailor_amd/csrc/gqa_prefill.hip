@@ -2,13 +2,14 @@
 // Replaces the call mx.fast.scaled_dot_product_attention(q, K[:, :, :kv_len], V[:, :, :kv_len], scale=256**-0.5,
 // mask="causal") of the reference's full-attention layers (qwen35/model.py:160-167, qwen35/prefill.py:468).
 //
-// One wavefront owns 16 query rows and keeps everything transposed so that no value ever changes lanes:
-//     S^T[keys x rows] = K_tile . Q^T          (A = K rows straight from HBM / L2, B = Q^T resident in registers)
-//     O^T[d x rows]   += V^T_tile . P^T        (A = rows of V^T, B = P^T)
-// In the accumulator layout lane (n, g) holds rows 4g..4g+3 of column n.  With columns = query rows, the running max, the
-// rescale and the final 1/l of a query row are lane-local, and two S^T accumulators, exponentiated and packed to bf16,
-// ARE the B operand of the P.V MFMA when the key index of a 32-key block is enumerated as 16 (j >> 2) + 4 g + (j & 3).
-// V^T rows are read from a transposed copy of V (qt_gqa_transpose_v, one small pass) so the A operand is contiguous.
+// One workgroup = 16 query rows x the 4 query heads that share a KV head (one head per wavefront), so a K / V tile of 64
+// keys is fetched from HBM once and staged in LDS for all four.  Per tile and wavefront:
+//     S^T[keys x rows] = K_tile . Q^T     A = K rows from LDS, B = Q^T resident in registers (16x16x32 bf16 MFMA)
+//     online softmax in the accumulator layout: lane (row n, group g) holds keys 4g..4g+3 of each 16-key sub-tile
+//     O[rows x 256]   += P . V            A = two exponentiated S^T accumulators packed to bf16 (they ARE the A operand
+//                                         when a 32-key block is enumerated as 16 (j >> 2) + 4 g + (j & 3)),
+//                                         B = V through the transposing LDS load (4 consecutive keys of one column)
+// The next tile travels global -> registers while the current one is consumed; two barriers per tile.
 #include "qt_common.h"
 
 using namespace qt;
@@ -16,114 +17,179 @@ using namespace qt;
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr float SCALE = 0.0625f;       // 256^-0.5
 constexpr float NEG = -3.0e38f;
+constexpr int KT = 64;                 // keys per tile
+constexpr int KS_LD = AD + 8;          // LDS row strides (elements): 528 / 544 bytes spread the rows over the banks
+constexpr int VS_LD = AD + 16;
 
-// V [KV][L][256] -> VT [KV][256][Lp] (keys past L are zero), 64 x 64 tiles through LDS
-__global__ __launch_bounds__(256) void transpose_v_kernel(const bf16_t* __restrict__ V, bf16_t* __restrict__ VT, int L, int Lp,
-                                                          long v_head_stride) {
-    __shared__ bf16_t tile[64][66];
-    const int kvh = blockIdx.z, k0 = blockIdx.x * 64, d0 = blockIdx.y * 64;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    for (int i = ty; i < 64; i += 4) {
-        const int key = k0 + i;
-        tile[i][tx] = key < L ? V[(size_t)kvh * v_head_stride + (size_t)key * AD + d0 + tx] : (bf16_t)0;
-    }
-    __syncthreads();
-    for (int i = ty; i < 64; i += 4) {
-        const int key = k0 + tx;
-        if (key < Lp) VT[((size_t)kvh * AD + d0 + i) * Lp + key] = tile[tx][i];
-    }
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
-                                                           const bf16_t* __restrict__ VT, bf16_t* __restrict__ out, int S, int L,
-                                                           int Lp, int q_pos0, long q_head_stride, long k_head_stride) {
-    const int qt = gridDim.x - 1 - blockIdx.x;                   // long rows first
-    const int h = blockIdx.y, kvh = h / (AH / AKV);
-    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
-    const int r0 = qt * 64 + w * 16;
-    if (r0 >= S) return;
-    const int row = r0 + n;
+                                                           const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
+                                                           int q_pos0, long q_head_stride, long kv_head_stride) {
+    __shared__ __align__(16) bf16_t k_s[KT * KS_LD];
+    __shared__ __align__(16) bf16_t v_s[KT * VS_LD];
+    __shared__ __align__(16) float c_s[4][16];
+    const int rb = gridDim.x - 1 - blockIdx.x;                   // long rows first
+    const int kvh = blockIdx.y;
+    const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int h = kvh * (AH / AKV) + w;
+    const int r0 = rb * 16, row = r0 + n;
     const bool row_ok = row < S;
     const int my_last = q_pos0 + row;                            // last key this query row may see
-    const int kend = min(L, q_pos0 + min(r0 + 15, S - 1) + 1);  // keys any row of this wavefront sees
+    const int kend = min(L, q_pos0 + min(r0 + 15, S - 1) + 1);   // keys any row of this block sees
+    const int ntiles = (kend + KT - 1) / KT;
 
+    // Q^T as the B operand of the score MFMA: lane (row n, group g) holds q[row][32 kb + 8 g .. + 8]
     bf16x8 bq[8];
     {
-        const uint4* qr = reinterpret_cast<const uint4*>(q + (size_t)h * q_head_stride + (size_t)(row_ok ? row : r0) * AD);
+        const u32x4* qr = reinterpret_cast<const u32x4*>(q + (size_t)h * q_head_stride + (size_t)(row_ok ? row : r0) * AD);
 #pragma unroll
         for (int kb = 0; kb < 8; kb++) {
-            uint4 v = qr[kb * 4 + g];
-            if (!row_ok) v = make_uint4(0, 0, 0, 0);
+            u32x4 v = qr[kb * 4 + g];
+            if (!row_ok) v = u32x4{0, 0, 0, 0};
             bq[kb] = __builtin_bit_cast(bf16x8, v);
         }
     }
+    // tile loader: thread (tid >> 5, tid & 31) moves 16 bytes of the rows tid >> 5 + 8 i, i = 0..7, of K and of V
+    const int lr = tid >> 5, lc = tid & 31;
+    const bf16_t* kg = K + (size_t)kvh * kv_head_stride + 8 * lc;
+    const bf16_t* vg = V + (size_t)kvh * kv_head_stride + 8 * lc;
+    u32x4 kr[8], vr[8];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int key = min(t * KT + lr + 8 * i, L - 1);     // rows past the end repeat the last key; they are masked
+            kr[i] = *reinterpret_cast<const u32x4*>(kg + (size_t)key * AD);
+            vr[i] = *reinterpret_cast<const u32x4*>(vg + (size_t)key * AD);
+        }
+    };
+    load_tile(0);
+
+    float m_run = NEG, l_run = 0.f;
     f32x4 O[16];
 #pragma unroll
-    for (int mt = 0; mt < 16; mt++) O[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = NEG, l_run = 0.f;
+    for (int j = 0; j < 16; j++) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const bf16_t* ka = k_s + n * KS_LD + 8 * g;                  // A operand of the scores: row 16 kt + n, columns 32 kb + 8 g
+    // transposing load: within 16 lanes, lane 4q + i receives element i of the 8-byte chunks addressed by lanes q, q+4,
+    // q+8, q+12; lane n of group g points at key 4g + n/4, columns 4 (n%4).. of the block and receives keys 4g..4g+3 of column n
+    const bf16_t* va = v_s + (4 * g + (n >> 2)) * VS_LD + 4 * (n & 3);
 
-    const bf16_t* Kh = K + (size_t)kvh * k_head_stride;
-    const bf16_t* Vh = VT + (size_t)kvh * AD * Lp;
-    for (int k0 = 0; k0 < kend; k0 += 32) {
-        f32x4 acc[2];
+    for (int t = 0; t < ntiles; t++) {
+        __syncthreads();                                         // everyone is done reading the previous tile
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            const int key = min(k0 + 16 * t + n, L - 1);
-            const uint4* kr = reinterpret_cast<const uint4*>(Kh + (size_t)key * AD);
-            uint4 a[8];
+        for (int i = 0; i < 8; i++) {
+            *reinterpret_cast<u32x4*>(k_s + (lr + 8 * i) * KS_LD + 8 * lc) = kr[i];
+            *reinterpret_cast<u32x4*>(v_s + (lr + 8 * i) * VS_LD + 8 * lc) = vr[i];
+        }
+        if (t + 1 < ntiles) load_tile(t + 1);
+        __syncthreads();
+
+        // scores: the 8 K fragments of a 16-key sub-tile are read in one batch, one sub-tile ahead of the MFMAs that use them
+        f32x4 acc[4];
+        bf16x8 Af[2][8];
 #pragma unroll
-            for (int kb = 0; kb < 8; kb++) a[kb] = kr[kb * 4 + g];
-            acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int kb = 0; kb < 8; kb++) Af[0][kb] = *reinterpret_cast<const bf16x8*>(ka + 32 * kb);
+#pragma unroll
+        for (int kt = 0; kt < 4; kt++) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (kt < 3) {
+#pragma unroll
+                for (int kb = 0; kb < 8; kb++)
+                    Af[(kt + 1) & 1][kb] = *reinterpret_cast<const bf16x8*>(ka + 16 * (kt + 1) * KS_LD + 32 * kb);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            acc[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kb = 0; kb < 8; kb++)
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[kb]), bq[kb], acc[t], 0, 0, 0);
+                acc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kt & 1][kb], bq[kb], acc[kt], 0, 0, 0);
         }
-        float s[8], mx = NEG;
+        __builtin_amdgcn_sched_barrier(0);
+        float sc[4][4], mx = NEG;
 #pragma unroll
-        for (int t = 0; t < 2; t++)
+        for (int kt = 0; kt < 4; kt++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int key = k0 + 16 * t + 4 * g + r;
-                s[t * 4 + r] = (key <= my_last && key < L) ? acc[t][r] * SCALE : NEG;
-                mx = fmaxf(mx, s[t * 4 + r]);
+            for (int i = 0; i < 4; i++) {
+                const int key = t * KT + 16 * kt + 4 * g + i;
+                sc[kt][i] = (key <= my_last && key < L) ? acc[kt][i] * SCALE : NEG;
+                mx = fmaxf(mx, sc[kt][i]);
             }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_run, mx);
-        const float corr = __expf(m_run - m_new);
-        float p[8], ps = 0.f;
+        const float corr = __expf(m_run - m_new);                // m_run = NEG initially: exp(-huge) = 0
+        float ps = 0.f;
+        s16x8 P[2];
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            p[i] = s[i] > 0.5f * NEG ? __expf(s[i] - m_new) : 0.f;
-            ps += p[i];
-        }
-        l_run = l_run * corr + ps;
+        for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float pv = sc[kt][i] > 0.5f * NEG ? __expf(sc[kt][i] - m_new) : 0.f;
+                ps += pv;
+                P[kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(pv);
+            }
+        l_run = l_run * corr + ps;                               // this lane's share; summed over g at the end
         m_run = m_new;
-        bf16x8 pb;
+        if (g == 0) c_s[w][n] = corr;
+        wave_lds_sync();
+        const f32x4 c4 = *reinterpret_cast<const f32x4*>(&c_s[w][4 * g]);
+        if (__any(corr != 1.0f)) {                               // wavefront-uniform: most tiles leave every row's max alone
 #pragma unroll
-        for (int i = 0; i < 8; i++) pb[i] = (__bf16)p[i];
-#pragma unroll
-        for (int mt = 0; mt < 16; mt++) {
-            const bf16_t* vr = Vh + (size_t)(16 * mt + n) * Lp + k0 + 4 * g;
-            const uint2 v0 = *reinterpret_cast<const uint2*>(vr), v1 = *reinterpret_cast<const uint2*>(vr + 16);
-            const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(v0.x, v0.y, v1.x, v1.y));
-            O[mt] *= corr;
-            O[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, O[mt], 0, 0, 0);
+            for (int j = 0; j < 16; j++) O[j] *= c4;
         }
+        // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs
+        auto v_frag = [&](int j, int q4) {
+            return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * VS_LD + 16 * j)));
+        };
+        s16x4 Bf[3][4];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            Bf[0][q4] = v_frag(0, q4);
+            Bf[1][q4] = v_frag(1, q4);
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (j + 2 < 16) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) Bf[(j + 2) % 3][q4] = v_frag(j + 2, q4);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                const s16x8 B = __builtin_shufflevector(Bf[j % 3][2 * pp], Bf[j % 3][2 * pp + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[pp]), __builtin_bit_cast(bf16x8, B),
+                                                              O[j], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        wave_lds_sync();                                         // c_s is rewritten by the next tile
     }
+    // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
-    if (row_ok) {
-        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-        bf16_t* orow = out + (size_t)h * q_head_stride + (size_t)row * AD;
+    if (g == 0) c_s[w][n] = l_run;
+    wave_lds_sync();
+    const f32x4 l4 = *reinterpret_cast<const f32x4*>(&c_s[w][4 * g]);
 #pragma unroll
-        for (int mt = 0; mt < 16; mt++) {
-            const uint2 pk = make_uint2(pack_bf(O[mt][0] * inv, O[mt][1] * inv), pack_bf(O[mt][2] * inv, O[mt][3] * inv));
-            *reinterpret_cast<uint2*>(orow + 16 * mt + 4 * g) = pk;
+    for (int r = 0; r < 4; r++) {
+        const int orow = r0 + 4 * g + r;
+        if (orow < S) {
+            const float inv = 1.0f / l4[r];
+            bf16_t* dst = out + (size_t)h * q_head_stride + (size_t)orow * AD + n;
+#pragma unroll
+            for (int j = 0; j < 16; j++) dst[16 * j] = f2bf(O[j][r] * inv);
         }
     }
 }
@@ -132,25 +198,23 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
 
 extern "C" {
 
-// bytes of the transposed-V workspace for L keys
-long qt_gqa_prefill_workspace_bytes(int L) { return L < 0 ? -1 : (long)AKV * AD * (((long)L + 63) / 64 * 64) * 2; }
+// no workspace is needed any more; the entry point keeps its argument (may be null) so that callers do not change
+long qt_gqa_prefill_workspace_bytes(int L) { return L < 0 ? -1 : 0; }
 
 // q, out [8][S][256] bf16 (head stride q_head_stride elements), K, V [2][>=L][256] bf16 (head stride kv_head_stride):
 // query i sits at absolute position q_pos0 + i and sees keys 0 .. q_pos0 + i (< L).
 int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out, void* workspace, long workspace_bytes, int S,
                           int L, int q_pos0, long q_head_stride, long kv_head_stride, hipStream_t stream) {
-    if (!q || !K || !V || !out || !workspace) return QT_ERR_NULL;
+    (void)workspace;
+    (void)workspace_bytes;
+    if (!q || !K || !V || !out) return QT_ERR_NULL;
     if (S < 0 || L < 1 || q_pos0 < 0 || q_head_stride < (long)S * AD || kv_head_stride < (long)L * AD) return QT_ERR_DIM;
     if (S == 0) return QT_OK;
-    for (const void* p : {q, K, V, (const void*)out, (const void*)workspace})
+    for (const void* p : {q, K, V, (const void*)out})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if ((q_head_stride | kv_head_stride) & 7) return QT_ERR_ALIGN;
-    if (workspace_bytes < qt_gqa_prefill_workspace_bytes(L)) return -6;
-    const int Lp = (L + 63) / 64 * 64;
-    hipLaunchKernelGGL(transpose_v_kernel, dim3(Lp / 64, AD / 64, AKV), dim3(256), 0, stream, (const bf16_t*)V, (bf16_t*)workspace, L,
-                       Lp, kv_head_stride);
-    hipLaunchKernelGGL(attn_prefill_kernel, dim3((S + 63) / 64, AH), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
-                       (const bf16_t*)workspace, (bf16_t*)out, S, L, Lp, q_pos0, q_head_stride, kv_head_stride);
+    hipLaunchKernelGGL(attn_prefill_kernel, dim3((S + 15) / 16, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
+                       (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }
