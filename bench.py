@@ -351,7 +351,7 @@ def main():
                                f"rotating over {N_LAYERS} layer pools", "batch": B, "layer_pools": N_LAYERS,
                    "launch": "eager" if args.no_graph else "hip-graph of 18 launches"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": None, "kernel": "gdn_decode_kernel<8>", "bytes_per_launch": decode_bytes(B),
+                     "traffic": None, "kernel": "gdn_decode_wide_kernel<4>" if B >= 64 else "gdn_decode_kernel", "bytes_per_launch": decode_bytes(B),
                      "avg_launch_us": launch_s * 1e6},
         "extras": extras,
     }

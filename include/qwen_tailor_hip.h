@@ -27,7 +27,8 @@ typedef void* qt_stream_t; /* hipStream_t */
 /* batch.deltanet_b (qwen35/batch.py:128-135): one decode token for each of B rows.
  * proj [B,8224] bf16; conv_pool [n_slots*2,3,6144] bf16 (reads buffer slot*2+(pos&1), writes the other one);
  * conv_w [6144*4] bf16; A_log, dt_bias [16] f32; ssm_pool [n_slots,16,128,128] f32 (updated in place);
- * slots, pos [B] int32; y [B,2048] bf16.  rows_per_wg: 0 = choose, else 16/32/64/128 value rows per workgroup. */
+ * slots, pos [B] int32; y [B,2048] bf16.  rows_per_wg: 0 = choose, else 16/32/64/128 value rows per workgroup
+ * (qt_gdn_decode_step also takes 256 / 512 = two / four whole heads per workgroup). */
 int qt_gdn_decode_step(const void* proj, void* conv_pool, const void* conv_w, const float* A_log, const float* dt_bias,
                        float* ssm_pool, const int32_t* slots, const int32_t* pos, void* y, int B, int n_slots,
                        int rows_per_wg, qt_stream_t stream);

@@ -46,7 +46,7 @@ __device__ __forceinline__ void store_window(bf16_t* __restrict__ cs_out, const 
 
 // M chained tokens of one (sequence, head, row split).  Snapshot j of the state goes to st_out + j*st_stride and of the
 // conv window to cs_out + j*cs_stride (strides 0 = update in place).
-template <int RS>
+template <int RS, int HPW = 1>
 __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs_in,
                                            bf16_t* __restrict__ cs_out, size_t cs_stride,
                                            const bf16_t* __restrict__ cw, const float* __restrict__ A_log,
@@ -54,12 +54,18 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
                                            float* st_out, size_t st_stride, bf16_t* __restrict__ y, int M, int h,
                                            int split) {
     constexpr int ROWS = RS * 16;
-    __shared__ double red[4];
-    __shared__ __align__(16) float qk_s[2][DK];
-    __shared__ float v_s[ROWS];
-    __shared__ float gb_s[2];
+    __shared__ double red_a[HPW][4];
+    __shared__ __align__(16) float qk_a[HPW][2][DK];
+    __shared__ float v_a[HPW][ROWS];
+    __shared__ float gb_a[HPW][2];
+    // HPW heads per workgroup: each group of 256 threads runs one head, only the barriers are shared
+    const int sub = HPW > 1 ? (int)(threadIdx.x >> 8) : 0;
+    double* red = red_a[sub];
+    float (*qk_s)[DK] = qk_a[sub];
+    float* v_s = v_a[sub];
+    float* gb_s = gb_a[sub];
 
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, grp = lane >> 4, c = lane & 15;
+    const int tid = threadIdx.x & 255, w = tid >> 6, lane = tid & 63, grp = lane >> 4, c = lane & 15;
     const int row0 = split * ROWS;
     const int which = tid >> 7;                                  // 0: a q channel, 1: a k channel
     const int ch_qk = which * KD + h * DK + (tid & 127);
@@ -182,6 +188,27 @@ __global__ __launch_bounds__(256) void gdn_decode_kernel(const bf16_t* __restric
                    y + (size_t)b * KD, 1, h, split);
 }
 
+// the same step with HPW heads of one row per workgroup (256 threads per head, whole heads only): the workgroup streams
+// HPW * 64 KiB of contiguous state
+template <int HPW>
+__global__ __launch_bounds__(256 * HPW) void gdn_decode_wide_kernel(const bf16_t* __restrict__ proj, bf16_t* conv_pool,
+                                                                    const bf16_t* __restrict__ cw,
+                                                                    const float* __restrict__ A_log,
+                                                                    const float* __restrict__ dt_bias, float* ssm_pool,
+                                                                    const int* __restrict__ slots,
+                                                                    const int* __restrict__ pos, bf16_t* __restrict__ y,
+                                                                    int n_slots) {
+    const unsigned id = xcd_remap(blockIdx.x, gridDim.x);
+    const int b = id / (HV / HPW), h = (id % (HV / HPW)) * HPW + (threadIdx.x >> 8);
+    const int slot = slots[b];
+    if ((unsigned)slot >= (unsigned)n_slots) return;
+    const int par = pos[b] & 1;
+    float* st = ssm_pool + (size_t)slot * HV * DV * DK;
+    gdn_tokens<8, HPW>(proj + (size_t)b * PW, conv_pool + (size_t)(slot * 2 + par) * 3 * CD,
+                       conv_pool + (size_t)(slot * 2 + (par ^ 1)) * 3 * CD, 0, cw, A_log, dt_bias, st, st, 0,
+                       y + (size_t)b * KD, 1, h, 0);
+}
+
 // batch_spec.deltanet_bm (qwen35/batch_spec.py:142-150): M chained tokens per sequence, snapshot pools in place
 template <int RS>
 __global__ __launch_bounds__(256) void gdn_verify_kernel(const bf16_t* __restrict__ proj, bf16_t* conv_pool,
@@ -249,9 +276,20 @@ int qt_gdn_decode_step(const void* proj, void* conv_pool, const void* conv_w, co
     if (B < 0 || n_slots <= 0) return QT_ERR_DIM;
     if (B == 0) return QT_OK;
     if (!aligned16(ssm_pool) || (reinterpret_cast<uintptr_t>(conv_w) & 7u)) return QT_ERR_ALIGN;
-    const int rs = pick_rs(B, rows_per_wg);
-    QT_DISPATCH_RS(rs, gdn_decode_kernel, B, stream, (const bf16_t*)proj, (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log,
-                   dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
+    // Many rows: 2 or 4 whole heads of a row per workgroup (128 / 256 KiB of contiguous state per workgroup); measured at
+    // B = 64: 23.3 us against 26.0 us with one head per workgroup.  Few rows: split heads so the chip still fills.
+    const int hpw = rows_per_wg == 512 ? 4 : rows_per_wg == 256 ? 2 : rows_per_wg != 0 ? 1 : B >= 64 ? 4 : B >= 32 ? 2 : 1;
+    if (hpw == 4) {
+        hipLaunchKernelGGL(gdn_decode_wide_kernel<4>, dim3(B * (HV / 4)), dim3(1024), 0, stream, (const bf16_t*)proj,
+                           (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log, dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
+    } else if (hpw == 2) {
+        hipLaunchKernelGGL(gdn_decode_wide_kernel<2>, dim3(B * (HV / 2)), dim3(512), 0, stream, (const bf16_t*)proj,
+                           (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log, dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
+    } else {
+        const int rs = pick_rs(B, rows_per_wg);
+        QT_DISPATCH_RS(rs, gdn_decode_kernel, B, stream, (const bf16_t*)proj, (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log,
+                       dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
+    }
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

@@ -248,6 +248,13 @@ def test_deltanet_b_layout_of_reference_test(qt, dev):
         check_tensors_equal('torch.equal(conv_pool[s_ * 2 + ((int(pos[b]) & 1) ', conv_pool[s_ * 2 + ((int(pos[b]) & 1) ^ 1)][None], rc)
     check_equal('np.array_equal(to_np(ssm_pool[4]), ssm0[4])', to_np(ssm_pool[4]), ssm0[4])
     check_equal('np.array_equal(to_np(ssm_pool[6]), ssm0[6])', to_np(ssm_pool[6]), ssm0[6])
+    # every workgroup shape (a head split over 8..1 workgroups, 2 or 4 whole heads per workgroup) gives the same bits
+    for rows in (16, 32, 64, 128, 256, 512):
+        cp2, ssm2 = to_dev(cp, dev, BF16), to_dev(ssm0, dev)
+        y2 = qt.batch.deltanet_b(to_dev(proj, dev, BF16), cp2, dcw, dA, ddt, ssm2, to_dev(slots, dev), to_dev(pos, dev), rows_per_wg=rows)
+        check_tensors_equal(f'y rows_per_wg={rows}', y2, y)
+        check_tensors_equal(f'conv pool rows_per_wg={rows}', cp2, conv_pool)
+        check_tensors_equal(f'ssm pool rows_per_wg={rows}', ssm2, ssm_pool)
 
 
 @pytest.mark.parametrize("B", [1, 16, 64])
@@ -287,6 +294,10 @@ def test_deltanet_b_out_of_range_slot_is_skipped(qt, dev):
     proj = to_dev(rand_bf(gen, (2, PW)), dev, BF16)
     qt.batch.deltanet_b(proj, conv, to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev), ssm,
                         torch.tensor([7, -1], dtype=torch.int32, device=dev), torch.tensor([0, 0], dtype=torch.int32, device=dev))
+    for rows in (256, 512):
+        qt.batch.deltanet_b(proj, conv, to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev), ssm,
+                            torch.tensor([7, -1], dtype=torch.int32, device=dev), torch.tensor([0, 0], dtype=torch.int32, device=dev),
+                            rows_per_wg=rows)
     torch.cuda.synchronize()
     check_tensors_equal('torch.equal(ssm, s0)', ssm, s0)
     check_tensors_equal('torch.equal(conv, c0)', conv, c0)
