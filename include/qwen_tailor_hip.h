@@ -98,6 +98,13 @@ long qt_gdn_chunk_gc_bytes(int S);
 long qt_gdn_chunk_snap_bytes(int S);
 int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v, const float* A_log, const float* dt_bias,
                    void* ops, float* U, float* gC, int S, qt_stream_t stream);
+/* qt_gdn_phase_a with qt_gdn_conv_prep fused in (the reference's fused prep kernel, qwen35/gdn_nax.py:394-401 prep_a, with the
+ * conv-state roll of qwen35/prefill.py:262-263): q, k, v are computed from proj [S,8224], conv_state [3,6144] and conv_w
+ * [6144*4] inside the kernel (same bits as qt_gdn_conv_prep).  q, k, v: all three null, or all three [S,16,128] bf16 outputs.
+ * conv_out: null or [3,6144] bf16, receives the new conv window (must not alias conv_state).  silu_table as qt_gdn_conv_prep. */
+int qt_gdn_phase_a_conv(const void* proj, const void* conv_state, const void* conv_w, const void* silu_table, const float* A_log,
+                        const float* dt_bias, void* q, void* k, void* v, void* conv_out, void* ops, float* U, float* gC, int S,
+                        qt_stream_t stream);
 int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
                    void* y, int S, qt_stream_t stream);
 int qt_gdn_phase_b_norm(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,

@@ -31,6 +31,7 @@ _SIGS = {
     "qt_gdn_phase_b_norm": [_vp] * 8 + [_f, _vp, _i, _vp],
     "qt_gqa_prefill_causal": [_vp] * 5 + [_l, _i, _i, _i, _l, _l, _vp],
     "qt_gdn_phase_a": [_vp] * 9 + [_i, _vp],
+    "qt_gdn_phase_a_conv": [_vp] * 13 + [_i, _vp],
 }
 
 

@@ -312,6 +312,9 @@ struct PhaseALds {                       // 68 KiB: two workgroups per CU
     __align__(16) bf16_t VT[DV * KT_LD];
     float Lc[C], beta[C], gam[C], dec[C];
 };
+struct PhaseALdsConv : PhaseALds {       // + the silu_bf16 table of the fused conv: 75 KiB, still two workgroups per CU
+    __align__(16) bf16_t tab[SILU_TAB_SIZE];
+};
 
 __device__ __forceinline__ half8 to_half8(const float (&v)[8]) {
     half8 h;
@@ -323,23 +326,44 @@ __device__ __forceinline__ void unpack4(uint2 w, float* f) {
     f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
 }
 
-// q, k, v [S,16,128] bf16 (convolved, normalized: conv_prep's outputs), proj [S,8224] (gate inputs a, b) -> phase B records
-__global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ qi,
-                                                          const bf16_t* __restrict__ ki, const bf16_t* __restrict__ vi,
+// Stores one token's normalized q, k and v (8 channels of each, bf16 pairs) into the row-major and transposed LDS tiles.
+__device__ __forceinline__ void stage_token(PhaseALds& L, int tl, int cc, const uint4& rq, const uint4& rk, const uint4& rv) {
+    *reinterpret_cast<uint4*>(&L.Qs[tl * QS_LD + cc * 8]) = rq;
+    *reinterpret_cast<uint4*>(&L.Ks[tl * QS_LD + cc * 8]) = rk;
+    const uint32_t kw[4] = {rk.x, rk.y, rk.z, rk.w};
+    const uint32_t vw[4] = {rv.x, rv.y, rv.z, rv.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        L.KT[kt_at(cc * 8 + 2 * e, tl)] = (bf16_t)(kw[e] & 0xffffu);
+        L.KT[kt_at(cc * 8 + 2 * e + 1, tl)] = (bf16_t)(kw[e] >> 16);
+        L.VT[kt_at(cc * 8 + 2 * e, tl)] = (bf16_t)(vw[e] & 0xffffu);
+        L.VT[kt_at(cc * 8 + 2 * e + 1, tl)] = (bf16_t)(vw[e] >> 16);
+    }
+}
+
+// Phase A of one (chunk, head).  FROM_PROJ = false: q, k, v [S,16,128] bf16 are inputs (convolved, normalized: conv_prep's
+// outputs).  FROM_PROJ = true: they are computed here from the projection rows (conv4 + SiLU + q/k norm with the arithmetic of
+// conv_prep_kernel, bit for bit; qwen35/prefill.py:96-134) and, with WRITE_QKV, also stored; the workgroups of the last chunk
+// write the new conv window (the last three input rows, prefill.py:262-263) to conv_out if it is given.
+// proj [S,8224] supplies the gate inputs a, b in both forms.
+template <bool FROM_PROJ, bool WRITE_QKV>
+__global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __restrict__ proj, bf16_t* qi, bf16_t* ki, bf16_t* vi,
+                                                          const bf16_t* __restrict__ cs, const bf16_t* __restrict__ cw,
+                                                          const bf16_t* __restrict__ silu_tab, bf16_t* __restrict__ conv_out,
                                                           const float* __restrict__ A_log, const float* __restrict__ dt_bias,
                                                           _Float16* __restrict__ ops, float* __restrict__ U,
                                                           float* __restrict__ gC, int S) {
-    __shared__ PhaseALds L;
+    __shared__ typename std::conditional<FROM_PROJ, PhaseALdsConv, PhaseALds>::type L;
     const int c = blockIdx.x / HV, h = blockIdx.x % HV, t0 = c * C;
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
     const size_t rec = (size_t)c * HV + h;
     _Float16* op = ops + rec * OP_HALVES;
+    const int gi = tid >> 4, cc = tid & 15;
 
-    // ---- the chunk's q, k, v rows: every load is issued before anything else (a 16-lane group owns a token per round,
-    // a lane 8 consecutive columns); rows past the end are zero (gdn_nax.py:172-174)
-    uint4 raw[4][3];
-    {
-        const int gi = tid >> 4, cc = tid & 15;
+    // ---- the chunk's rows: every load is issued before anything else; rows past the end are zero (gdn_nax.py:172-174)
+    uint4 raw[4][3];                               // !FROM_PROJ: token rr * 16 + gi, a lane 8 consecutive columns
+    uint4 rw[3][7], wt[3][4];                      // FROM_PROJ: input rows 4 gi - 3 .. 4 gi + 3 of 8 channels of q, k, v; their taps
+    if constexpr (!FROM_PROJ) {
 #pragma unroll
         for (int rr = 0; rr < 4; rr++) {
             const int t = t0 + rr * 16 + gi;
@@ -348,6 +372,23 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
             raw[rr][1] = *reinterpret_cast<const uint4*>(ki + o);
             raw[rr][2] = *reinterpret_cast<const uint4*>(vi + o);
             if (t >= S) raw[rr][0] = raw[rr][1] = raw[rr][2] = make_uint4(0, 0, 0, 0);
+        }
+    } else {
+#pragma unroll
+        for (int part = 0; part < 3; part++) {
+            const int ch0 = part * KD + h * DK + cc * 8;
+#pragma unroll
+            for (int e = 0; e < 4; e++) wt[part][e] = *reinterpret_cast<const uint4*>(cw + (size_t)(ch0 + 2 * e) * 4);
+#pragma unroll
+            for (int d = 0; d < 7; d++) {
+                const int tt = min(t0 + 4 * gi - 3 + d, S - 1);
+                rw[part][d] = *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0);
+            }
+        }
+        if (conv_out && c == (S - 1) / C && tid < 3 * 48) {            // new conv window: input rows S-3 .. S-1 of this head's channels
+            const int r = tid / 48, part = (tid % 48) >> 4, ch0 = part * KD + h * DK + (tid & 15) * 8, tt = S - 3 + r;
+            *reinterpret_cast<uint4*>(conv_out + r * CD + ch0) =
+                *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0);
         }
     }
 
@@ -372,22 +413,36 @@ __global__ __launch_bounds__(256) void gdn_phase_a_kernel(const bf16_t* __restri
         L.dec[lane] = expf(tot - lc);
         if (lane == 63) gC[rec] = expf(lc);
     }
-    {
-        const int gi = tid >> 4, cc = tid & 15;
+    if constexpr (!FROM_PROJ) {
 #pragma unroll
-        for (int rr = 0; rr < 4; rr++) {
-            const int tl = rr * 16 + gi;
-            *reinterpret_cast<uint4*>(&L.Qs[tl * QS_LD + cc * 8]) = raw[rr][0];
-            *reinterpret_cast<uint4*>(&L.Ks[tl * QS_LD + cc * 8]) = raw[rr][1];
-            const uint32_t kw[4] = {raw[rr][1].x, raw[rr][1].y, raw[rr][1].z, raw[rr][1].w};
-            const uint32_t vw[4] = {raw[rr][2].x, raw[rr][2].y, raw[rr][2].z, raw[rr][2].w};
+        for (int rr = 0; rr < 4; rr++) stage_token(L, rr * 16 + gi, cc, raw[rr][0], raw[rr][1], raw[rr][2]);
+    } else {
+        silu_table_fill(L.tab, silu_tab, tid, 256);
+        __syncthreads();
+        const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
+        uint4 pk[4][3];
+        float ss[8], rr[8];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                L.KT[kt_at(cc * 8 + 2 * e, tl)] = (bf16_t)(kw[e] & 0xffffu);
-                L.KT[kt_at(cc * 8 + 2 * e + 1, tl)] = (bf16_t)(kw[e] >> 16);
-                L.VT[kt_at(cc * 8 + 2 * e, tl)] = (bf16_t)(vw[e] & 0xffffu);
-                L.VT[kt_at(cc * 8 + 2 * e + 1, tl)] = (bf16_t)(vw[e] >> 16);
+        for (int part = 0; part < 3; part++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const double sq = conv8_silu_packed(L.tab, rw[part][j], rw[part][j + 1], rw[part][j + 2], rw[part][j + 3], wt[part],
+                                                    pk[j][part]);
+                if (part < 2) ss[2 * j + part] = (float)row16_sum_d(sq);
             }
+        rsqrt_rows<8>(ss, qk_eps(), rr, cc);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int tl = 4 * gi + j, t = t0 + tl;
+            uint4 pq = scale8_packed(pk[j][0], rr[2 * j], scq), pkk = scale8_packed(pk[j][1], rr[2 * j + 1], sck), pv = pk[j][2];
+            if (t >= S) pq = pkk = pv = make_uint4(0, 0, 0, 0);
+            if (WRITE_QKV && t < S) {
+                const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
+                *reinterpret_cast<uint4*>(qi + o) = pq;
+                *reinterpret_cast<uint4*>(ki + o) = pkk;
+                *reinterpret_cast<uint4*>(vi + o) = pv;
+            }
+            stage_token(L, tl, cc, pq, pkk, pv);
         }
     }
     __syncthreads();
@@ -622,8 +677,33 @@ int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v
     for (const void* p : {proj, q, k, v, (const void*)ops, (const void*)U})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     const int NC = (S + C - 1) / C;
-    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (const bf16_t*)q,
-                       (const bf16_t*)k, (const bf16_t*)v, A_log, dt_bias, (_Float16*)ops, U, gC, S);
+    hipLaunchKernelGGL((gdn_phase_a_kernel<false, false>), dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (bf16_t*)q,
+                       (bf16_t*)k, (bf16_t*)v, (const bf16_t*)nullptr, (const bf16_t*)nullptr, (const bf16_t*)nullptr,
+                       (bf16_t*)nullptr, A_log, dt_bias, (_Float16*)ops, U, gC, S);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_gdn_phase_a_conv(const void* proj, const void* conv_state, const void* conv_w, const void* silu_table, const float* A_log,
+                        const float* dt_bias, void* q, void* k, void* v, void* conv_out, void* ops, float* U, float* gC, int S,
+                        hipStream_t stream) {
+    if (!proj || !conv_state || !conv_w || !A_log || !dt_bias || !ops || !U || !gC) return QT_ERR_NULL;
+    if ((q || k || v) && !(q && k && v)) return QT_ERR_NULL;
+    if (S < 0) return QT_ERR_DIM;
+    if (S == 0) return QT_OK;
+    for (const void* p : {proj, conv_state, conv_w, silu_table, (const void*)q, (const void*)k, (const void*)v, (const void*)conv_out,
+                          (const void*)ops, (const void*)U})
+        if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
+    if (conv_out == conv_state) return QT_ERR_UNSUPPORTED;          // the old window is still being read when the new one is written
+    const int NC = (S + C - 1) / C;
+    if (q)
+        hipLaunchKernelGGL((gdn_phase_a_kernel<true, true>), dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (bf16_t*)q,
+                           (bf16_t*)k, (bf16_t*)v, (const bf16_t*)conv_state, (const bf16_t*)conv_w, (const bf16_t*)silu_table,
+                           (bf16_t*)conv_out, A_log, dt_bias, (_Float16*)ops, U, gC, S);
+    else
+        hipLaunchKernelGGL((gdn_phase_a_kernel<true, false>), dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj,
+                           (bf16_t*)nullptr, (bf16_t*)nullptr, (bf16_t*)nullptr, (const bf16_t*)conv_state, (const bf16_t*)conv_w,
+                           (const bf16_t*)silu_table, (bf16_t*)conv_out, A_log, dt_bias, (_Float16*)ops, U, gC, S);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

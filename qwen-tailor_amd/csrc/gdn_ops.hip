@@ -70,41 +70,25 @@ __global__ __launch_bounds__(256) void conv_prep_kernel(const bf16_t* __restrict
     silu_table_fill(tab, silu_tab, tid, 256);
     __syncthreads();
     const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
+    uint4 pk[2][3];
+    float ss[4], rr[4];
+#pragma unroll
+    for (int part = 0; part < 3; part++)
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const double sq = conv8_silu_packed(tab, raw[r][part][0], raw[r][part][1], raw[r][part][2], raw[r][part][3], wt[part],
+                                                pk[r][part]);
+            if (part < 2) ss[2 * r + part] = (float)row16_sum_d(sq);
+        }
+    rsqrt_rows<4>(ss, qk_eps(), rr, cc);
 #pragma unroll
     for (int r = 0; r < 2; r++) {
         const int t = tb * CP_TOK + r * 16 + gi;
-        float u[3][8];
-#pragma unroll
-        for (int part = 0; part < 3; part++) {
-            float x[4][8];
-#pragma unroll
-            for (int d = 0; d < 4; d++) unpack8(raw[r][part][d], x[d]);
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const uint4 ww = wt[part][e >> 1];
-                const uint2 wc = (e & 1) ? make_uint2(ww.z, ww.w) : make_uint2(ww.x, ww.y);
-                u[part][e] = conv_silu_tab(tab, x[0][e], x[1][e], x[2][e], x[3][e], wc);
-            }
-        }
-        double sq = 0.0, sk = 0.0;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            sq += (double)u[0][e] * u[0][e];
-            sk += (double)u[1][e] * u[1][e];
-        }
-        const float qr = rsqrt_rn((float)row16_sum_d(sq) / (float)DK + qk_eps());
-        const float kr = rsqrt_rn((float)row16_sum_d(sk) / (float)DK + qk_eps());
         if (t < S) {
             const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
-            uint4 pq, pk, pv;
-            pq.x = pack_bf(BF(BF(u[0][0] * qr) * scq), BF(BF(u[0][1] * qr) * scq)); pq.y = pack_bf(BF(BF(u[0][2] * qr) * scq), BF(BF(u[0][3] * qr) * scq));
-            pq.z = pack_bf(BF(BF(u[0][4] * qr) * scq), BF(BF(u[0][5] * qr) * scq)); pq.w = pack_bf(BF(BF(u[0][6] * qr) * scq), BF(BF(u[0][7] * qr) * scq));
-            pk.x = pack_bf(BF(BF(u[1][0] * kr) * sck), BF(BF(u[1][1] * kr) * sck)); pk.y = pack_bf(BF(BF(u[1][2] * kr) * sck), BF(BF(u[1][3] * kr) * sck));
-            pk.z = pack_bf(BF(BF(u[1][4] * kr) * sck), BF(BF(u[1][5] * kr) * sck)); pk.w = pack_bf(BF(BF(u[1][6] * kr) * sck), BF(BF(u[1][7] * kr) * sck));
-            pv.x = pack_bf(u[2][0], u[2][1]); pv.y = pack_bf(u[2][2], u[2][3]); pv.z = pack_bf(u[2][4], u[2][5]); pv.w = pack_bf(u[2][6], u[2][7]);
-            *reinterpret_cast<uint4*>(q + o) = pq;
-            *reinterpret_cast<uint4*>(k + o) = pk;
-            *reinterpret_cast<uint4*>(v + o) = pv;
+            *reinterpret_cast<uint4*>(q + o) = scale8_packed(pk[r][0], rr[2 * r], scq);
+            *reinterpret_cast<uint4*>(k + o) = scale8_packed(pk[r][1], rr[2 * r + 1], sck);
+            *reinterpret_cast<uint4*>(v + o) = pk[r][2];
         }
     }
 }

@@ -124,9 +124,84 @@ __device__ __forceinline__ float conv_silu_tab(const bf16_t* tab, float w0, floa
     s = s + x * hi_bf(c.y);
     return silu_lookup(tab, f2bf(s));
 }
+// Branch-free form for hot loops: inputs with |x| >= 32 (or NaN) return a placeholder and set `rare`; the caller then
+// re-evaluates that group of channels through conv8_silu_slow, which is kept out of line so that the hot loop stays small.
+__device__ __forceinline__ float silu_lookup_fast(const bf16_t* tab, bf16_t xb, bool& rare) {
+    const unsigned ax = xb & 0x7fffu, idx = ax - SILU_TAB_LO * 128;               // idx wraps for small |x|
+    const bool in_tab = idx < (unsigned)SILU_TAB_N;
+    rare |= ax >= (unsigned)(SILU_TAB_LO * 128 + SILU_TAB_N);
+    const float t = bf2f(tab[(xb >> 15) * SILU_TAB_N + (in_tab ? idx : 0u)]);
+    return in_tab ? t : BF(bf2f(xb) * 0.5f);
+}
+__device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]);
+// conv4 + silu of 8 consecutive channels of one token: rows x0..x3 (oldest first, 8 bf16 each), taps wt (4 bf16 per channel)
+struct F8 { float v[8]; };
+static __device__ __attribute__((noinline)) F8 conv8_silu_slow(uint4 x0, uint4 x1, uint4 x2, uint4 x3, uint4 w0, uint4 w1, uint4 w2,
+                                                               uint4 w3);
+__device__ __forceinline__ void conv8_silu_tab(const bf16_t* tab, const uint4& x0, const uint4& x1, const uint4& x2,
+                                               const uint4& x3, const uint4 (&wt)[4], float (&u)[8]) {
+    float a[8], b[8], c[8], d[8];
+    unpack8(x0, a);
+    unpack8(x1, b);
+    unpack8(x2, c);
+    unpack8(x3, d);
+    bool rare = false;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const uint4 ww = wt[e >> 1];
+        const uint32_t c0 = (e & 1) ? ww.z : ww.x, c1 = (e & 1) ? ww.w : ww.y;
+        float s = a[e] * lo_bf(c0);
+        s = s + b[e] * hi_bf(c0);
+        s = s + c[e] * lo_bf(c1);
+        s = s + d[e] * hi_bf(c1);
+        u[e] = silu_lookup_fast(tab, f2bf(s), rare);
+    }
+    if (__builtin_expect(rare, 0)) {
+        const F8 r = conv8_silu_slow(x0, x1, x2, x3, wt[0], wt[1], wt[2], wt[3]);
+#pragma unroll
+        for (int e = 0; e < 8; e++) u[e] = r.v[e];
+    }
+}
 __device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]) {
     f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
     f[4] = lo_bf(w.z); f[5] = hi_bf(w.z); f[6] = lo_bf(w.w); f[7] = hi_bf(w.w);
+}
+
+static __device__ __attribute__((noinline)) F8 conv8_silu_slow(uint4 x0, uint4 x1, uint4 x2, uint4 x3, uint4 w0, uint4 w1, uint4 w2,
+                                                               uint4 w3) {
+    float a[8], b[8], c[8], d[8];
+    unpack8(x0, a);
+    unpack8(x1, b);
+    unpack8(x2, c);
+    unpack8(x3, d);
+    const uint4 wt[4] = {w0, w1, w2, w3};
+    F8 r;
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+        const uint4 ww = wt[e >> 1];
+        r.v[e] = conv_silu(a[e], b[e], c[e], d[e], make_uint2(ww.x, ww.y));
+        r.v[e + 1] = conv_silu(a[e + 1], b[e + 1], c[e + 1], d[e + 1], make_uint2(ww.z, ww.w));
+    }
+    return r;
+}
+
+// conv4 + silu of 8 channels of one token, packed as bf16 pairs (the values are bf16-exact), and their exact sum of squares
+__device__ __forceinline__ double conv8_silu_packed(const bf16_t* tab, const uint4& x0, const uint4& x1, const uint4& x2,
+                                                    const uint4& x3, const uint4 (&wt)[4], uint4& packed) {
+    float u[8];
+    conv8_silu_tab(tab, x0, x1, x2, x3, wt, u);
+    double sq = 0.0;
+#pragma unroll
+    for (int e = 0; e < 8; e++) sq += (double)u[e] * u[e];
+    packed = make_uint4(pack_bf(u[0], u[1]), pack_bf(u[2], u[3]), pack_bf(u[4], u[5]), pack_bf(u[6], u[7]));
+    return sq;
+}
+// q/k normalization of 8 packed channels: BF(BF(u * r) * sc) (kernels.py:507-510)
+__device__ __forceinline__ uint4 scale8_packed(const uint4& u, float r, float sc) {
+    float f[8];
+    unpack8(u, f);
+    return make_uint4(pack_bf(BF(BF(f[0] * r) * sc), BF(BF(f[1] * r) * sc)), pack_bf(BF(BF(f[2] * r) * sc), BF(BF(f[3] * r) * sc)),
+                      pack_bf(BF(BF(f[4] * r) * sc), BF(BF(f[5] * r) * sc)), pack_bf(BF(BF(f[6] * r) * sc), BF(BF(f[7] * r) * sc)));
 }
 
 constexpr float INV_SCALE = 0.08838834764831845f;                                // 128^-0.5, kernels.py:490
@@ -157,6 +232,26 @@ __device__ __forceinline__ double row16_sum_d(double v) {
     v += dpp_mov_d<0x141>(v);
     v += dpp_mov_d<0x140>(v);
     return v;
+}
+// value of lane I of each 16-lane row, to every lane of that row
+template <int I>
+__device__ __forceinline__ float row16_bcast(float v) { return dpp_mov<0x150 + I>(v); }
+template <int N, int I = 0>
+__device__ __forceinline__ void row16_bcast_all(float v, float (&r)[N]) {
+    if constexpr (I < N) {
+        r[I] = row16_bcast<I>(v);
+        row16_bcast_all<N, I + 1>(v, r);
+    }
+}
+// N <= 16 sums of squares of 128-wide rows (every lane of a 16-lane row holds all N) -> r[i] = rsqrt_rn(ss[i] / 128 + eps).
+// Lane c of the row evaluates entry c % N only and the results are broadcast, so the double-precision rsqrt runs once per lane.
+template <int N>
+__device__ __forceinline__ void rsqrt_rows(const float (&ss)[N], float eps, float (&r)[N], int c) {
+    float mine = ss[0];
+#pragma unroll
+    for (int i = 1; i < N; i++) mine = (c % N == i) ? ss[i] : mine;
+    const float rv = rsqrt_rn(mine / 128.0f + eps);
+    row16_bcast_all<N>(rv, r);
 }
 // total over the whole 64-lane wavefront (every lane gets it)
 __device__ __forceinline__ double wave_sum_d(double v) {

@@ -28,24 +28,33 @@ def _alloc_records(S, dev):
     return ops, U, gC
 
 
-def _phase_a(proj, conv_state, conv_w, A_log, dt_bias, qkv=None, want_qkv=True):
-    """conv_prep (unless q, k, v are given) followed by the phase A kernel.  Returns (q, k, v, ops, U, gC)."""
-    from . import prefill
+def _phase_a(proj, conv_state, conv_w, A_log, dt_bias, qkv=None, want_qkv=True, conv_out=None):
+    """Phase A.  With q, k, v given: the kernel that consumes them.  Otherwise one kernel that convolves and normalizes the
+    projection rows itself (returning q, k, v only if want_qkv) and, if conv_out [3,6144] is given, writes the new conv
+    window there.  Returns (q, k, v, ops, U, gC)."""
     proj = L.dev(proj, BF16, "proj", (None, PW))
     S = proj.shape[0]
     A, dtb = L.f32(A_log, "A_log", (HV,)), L.f32(dt_bias, "dt_bias", (HV,))
+    ops, U, gC = _alloc_records(S, proj.device)
     if qkv is not None:
         q, k, v = (L.dev(t, BF16, name, (S, HV, DK)) for t, name in zip(qkv, "qkv"))
-    else:
-        q, k, v = prefill.conv_prep(proj, conv_state, conv_w)
-    ops, U, gC = _alloc_records(S, proj.device)
-    L.call("qt_gdn_phase_a", L.ptr(proj), L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(A), L.ptr(dtb), L.ptr(ops), L.ptr(U), L.ptr(gC), S,
-           L.stream())
+        L.call("qt_gdn_phase_a", L.ptr(proj), L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(A), L.ptr(dtb), L.ptr(ops), L.ptr(U), L.ptr(gC), S,
+               L.stream())
+        return q, k, v, ops, U, gC
+    cs = L.dev(conv_state, BF16, "conv_state", (3, CD))
+    w = flat_conv_w(conv_w)
+    q = k = v = None
+    if want_qkv:
+        q, k, v = (torch.empty((S, HV, DK), dtype=BF16, device=proj.device) for _ in range(3))
+    if conv_out is not None:
+        conv_out = L.dev(conv_out, BF16, "conv_out", (3, CD))
+    L.call("qt_gdn_phase_a_conv", L.ptr(proj), L.ptr(cs), L.ptr(w), L.ptr(L.silu_table(proj.device)), L.ptr(A), L.ptr(dtb), L.ptr(q),
+           L.ptr(k), L.ptr(v), L.ptr(conv_out), L.ptr(ops), L.ptr(U), L.ptr(gC), S, L.stream())
     return q, k, v, ops, U, gC
 
 
 def prep_a(proj, conv_state, conv_w, A_log, dt_bias, relaxed=True):
-    """conv+silu+qk-norm and phase A (qwen35/gdn_nax.py:394-401; here two launches: the conv kernel, then phase A).
+    """conv+silu+qk-norm and phase A in one launch (qwen35/gdn_nax.py:394-401).
     proj [S,8224], conv_state [3,6144], conv_w [6144,4,1] -> q, k, v [S,16,128] bf16 and the three phase-B records."""
     return _phase_a(proj, conv_state, conv_w, A_log, dt_bias)
 

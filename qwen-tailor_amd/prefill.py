@@ -27,15 +27,16 @@ def gdn_core(proj, conv_state, ssm_state, conv_w, A_log, dt_bias, gnorm, want_qk
     S = proj.shape[0]
     cs = conv_state.reshape(3, CD)
     if GDN_IMPL == "nax":
-        q, k, v, ops, U, gC = gdn_nax._phase_a(proj, cs, conv_w, A_log, dt_bias)
+        new_conv = torch.empty((1, 3, CD), dtype=BF16, device=proj.device)
+        _, _, _, ops, U, gC = gdn_nax._phase_a(proj, cs, conv_w, A_log, dt_bias, want_qkv=want_qkv, conv_out=new_conv[0])
         normed, new_ssm = gdn_nax.phase_b_norm(proj, ops, U, gC, ssm_state, gnorm)
     else:
         q, k, v = conv_prep(proj, cs, conv_w)
         out, new_ssm = gated_delta.gated_delta_update(q[None], k[None], v[None], proj[:, 8208:][None], proj[:, 8192:8208][None],
                                                       A_log, dt_bias, ssm_state.reshape(1, HV, DV, DK))
         normed = gated_norm(out.reshape(S, HV * DV), proj, gnorm)
-    tail = proj[:, :CD]
-    new_conv = (tail[S - 3:] if S >= 3 else torch.cat([cs, tail], dim=0)[-3:])[None].contiguous()   # prefill.py:262-263
+        tail = proj[:, :CD]
+        new_conv = (tail[S - 3:] if S >= 3 else torch.cat([cs, tail], dim=0)[-3:])[None].contiguous()   # prefill.py:262-263
     return normed, new_conv, new_ssm.reshape(1, HV, DV, DK)
 
 

@@ -123,3 +123,20 @@ def test_config2_chunked_prefill(qt, dev, T):
     check_tensors_equal("gdn_core output", o4, out)
     check_tensors_equal("gdn_core state", s4, s1)
     check_equal("gdn_core conv tail", to_np(conv4)[0], otail)
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 5, 64, 65, 200])
+def test_fused_conv_phase_a_equals_separate_kernels(qt, dev, T):
+    """phase A fed by conv_prep's q, k, v and phase A convolving the projection rows itself give the same records, bit for bit;
+    the conv window it leaves is the last three input rows (qwen35/prefill.py:262-263), also when S < 3"""
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(300 + T, T)
+    dproj, dcs, dcw, dA, ddt = to_dev(proj, dev, BF16), to_dev(cs, dev, BF16), to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev)
+    q, k, v = qt.prefill.conv_prep(dproj, dcs, dcw)
+    _, _, _, ops0, U0, gC0 = qt.gdn_nax._phase_a(dproj, None, None, dA, ddt, qkv=(q, k, v))
+    tail = torch.zeros((3, CD), dtype=BF16, device=dev)
+    q1, k1, v1, ops1, U1, gC1 = qt.gdn_nax._phase_a(dproj, dcs, dcw, dA, ddt, conv_out=tail)
+    _, _, _, ops2, U2, gC2 = qt.gdn_nax._phase_a(dproj, dcs, dcw, dA, ddt, want_qkv=False)
+    for name, a, b in (("q", q1, q), ("k", k1, k), ("v", v1, v), ("ops", ops1, ops0), ("U", U1, U0), ("gC", gC1, gC0),
+                       ("ops (no q, k, v stored)", ops2, ops0), ("U (no q, k, v stored)", U2, U0), ("gC (no q, k, v stored)", gC2, gC0)):
+        check_tensors_equal(name, a, b)
+    check_equal("conv tail", to_np(tail), np.concatenate([cs, proj[:, :CD]], axis=0)[-3:])
