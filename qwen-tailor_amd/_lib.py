@@ -71,7 +71,7 @@ _SILU_TABLES = {}
 
 
 def silu_table(dev):
-    """The 7 KiB silu_bf16 table of `dev` (built once per device by the library, owned here: the C ABI keeps no state)."""
+    """The 11 KiB silu_bf16 table of `dev` (built once per device by the library, owned here: the C ABI keeps no state)."""
     t = _SILU_TABLES.get(dev)
     if t is None:
         t = torch.empty(lib().qt_silu_table_bytes() // 2, dtype=torch.bfloat16, device=dev)

@@ -94,9 +94,9 @@ __device__ __forceinline__ float conv_silu(float w0, float w1, float w2, float x
 }
 
 // silu_bf16 is a bf16 -> bf16 map, so kernels that evaluate it many times per thread read it from a table in LDS:
-// 2 signs x 14 exponents (bf16 exponent fields 118..131, 2^-9 <= |x| < 2^5) x 128 mantissas = 3584 entries (7 KiB).
-// Below the range exp(|x|) rounds to 1 and sigmoid_bf16 is exactly 0.5; above it the direct evaluation is used.
-constexpr int SILU_TAB_LO = 118, SILU_TAB_N = 14 * 128, SILU_TAB_SIZE = 2 * SILU_TAB_N;
+// 2 signs x 22 exponents (bf16 exponent fields 110..131, 2^-17 <= |x| < 2^5) x 128 mantissas = 5632 entries (11 KiB).
+// Inputs outside the range (about one in 10^5 for conv sums of unit-variance data) are evaluated directly.
+constexpr int SILU_TAB_LO = 110, SILU_TAB_N = 22 * 128, SILU_TAB_SIZE = 2 * SILU_TAB_N;
 __device__ __forceinline__ bf16_t silu_table_entry(int i) {
     const bf16_t xb = (bf16_t)(((i / SILU_TAB_N) << 15) | (SILU_TAB_LO * 128 + i % SILU_TAB_N));
     return f2bf(silu_bf16(bf2f(xb)));
@@ -124,14 +124,13 @@ __device__ __forceinline__ float conv_silu_tab(const bf16_t* tab, float w0, floa
     s = s + x * hi_bf(c.y);
     return silu_lookup(tab, f2bf(s));
 }
-// Branch-free form for hot loops: inputs with |x| >= 32 (or NaN) return a placeholder and set `rare`; the caller then
-// re-evaluates that group of channels through conv8_silu_slow, which is kept out of line so that the hot loop stays small.
+// Branch-free form for hot loops: inputs outside the table return a placeholder and set `rare`; the caller then re-evaluates
+// that group of channels through conv8_silu_slow, which is kept out of line so that the hot loop stays small.
 __device__ __forceinline__ float silu_lookup_fast(const bf16_t* tab, bf16_t xb, bool& rare) {
-    const unsigned ax = xb & 0x7fffu, idx = ax - SILU_TAB_LO * 128;               // idx wraps for small |x|
+    const unsigned idx = (xb & 0x7fffu) - SILU_TAB_LO * 128;                      // wraps for small |x|
     const bool in_tab = idx < (unsigned)SILU_TAB_N;
-    rare |= ax >= (unsigned)(SILU_TAB_LO * 128 + SILU_TAB_N);
-    const float t = bf2f(tab[(xb >> 15) * SILU_TAB_N + (in_tab ? idx : 0u)]);
-    return in_tab ? t : BF(bf2f(xb) * 0.5f);
+    rare |= !in_tab;
+    return bf2f(tab[(xb >> 15) * SILU_TAB_N + (in_tab ? idx : 0u)]);
 }
 __device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]);
 // conv4 + silu of 8 consecutive channels of one token: rows x0..x3 (oldest first, 8 bf16 each), taps wt (4 bf16 per channel)
