@@ -75,8 +75,9 @@ int qt_gdn_recurrent(const void* q, const void* k, const void* v, const float* g
 
 /* batch.attn_b (qwen35/batch.py:230-237): ragged decode / verify attention, 8 query heads on 2 KV heads, head dim 256.
  * q [B*M,8,256], k_new / v_new [B*M,2,256], pools Kp / Vp [n_slots,2,Lmax,256] bf16 (rows pos[b]..pos[b]+M-1 are appended),
- * out [B*M,8,256].  1 <= M <= 4.  CH = pool keys per split-K workgroup (multiple of 16); workspace of at least
- * qt_gqa_attn_workspace_bytes(B, M, Lmax, CH) bytes, 16-byte aligned, owned by the caller. */
+ * out [B*M,8,256].  1 <= M <= 4, B <= 1024.  The batch's 16-key tiles are spread evenly over one workgroup per CU (split-K
+ * over a flat tile space, so ragged lengths balance); CH = smallest number of pool keys one workgroup takes (multiple of 16).
+ * Workspace of at least qt_gqa_attn_workspace_bytes(B, M, Lmax, CH) bytes, 16-byte aligned, owned by the caller. */
 long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH);
 int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
                        const int32_t* pos, void* out, void* workspace, long workspace_bytes, int B, int M, int Lmax,

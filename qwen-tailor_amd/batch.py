@@ -48,10 +48,9 @@ def _workspace(dev, nbytes):
 
 
 def split_size(Lmax: int, B: int = 16) -> int:
-    """keys per split-K workgroup: aims at roughly 768 workgroups for full pools (about half of that in a ragged batch),
-    a few per CU, each long enough that a wavefront streams several tiles per partial result it writes"""
-    ch = (2 * B * Lmax // 768 + 64) // 128 * 128
-    return max(256, min(1024, ch))
+    """Smallest number of pool keys a split-K workgroup takes.  The kernel spreads the batch's key tiles evenly over one
+    workgroup per CU whatever the mix of lengths; this lower bound only matters for small batches of short sequences."""
+    return 128
 
 
 def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None):

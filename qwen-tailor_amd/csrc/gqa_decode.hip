@@ -3,18 +3,24 @@
 // pos[b] + j of slot slots[b]; it attends the pool keys below pos[b] and the new keys of rows b*M .. b*M + j, which are
 // read from the inputs (never from the pool) and appended to the pool at pos[b] + j.
 //
-// Split-K: workgroup (b, kv head, split s) streams the pool keys [s*CH, min((s+1)*CH, pos[b])) ONCE for all 4*M query
-// rows that share the KV head, so K and V are read from HBM exactly once per step.
-//   scores : S^T[16 keys x 16 rows] = K_tile[16 x 256] . Q^T[256 x 16] on bf16 MFMA (16x16x32), K straight from HBM
+// Split-K over one flat tile space: segment sg = (sequence b, kv head) owns max(1, ceil(pos[b] / 16)) tiles of 16 pool keys,
+// the segments are laid end to end, and each of the launch's workgroups takes the same number of consecutive tiles (it may
+// cross segment borders: it then emits one partial result per segment it touches).  Every workgroup therefore streams the
+// same number of bytes whatever the mix of sequence lengths, K and V are read from HBM exactly once per step for all 4*M
+// query rows that share the KV head, and the launch is one round of resident workgroups (one per CU).
+//   loads  : a K or V tile (16 keys x 512 bytes) is fetched as whole rows, two rows per wavefront-wide load (nontemporal),
+//            and parked row-major in LDS
+//   scores : S^T[16 keys x 16 rows] = K_tile[16 x 256] . Q^T[256 x 16] on bf16 MFMA (16x16x32), K fragments from LDS
 //   P . V  : O[16 rows x 256] += P[16 x 16 keys] . V[16 keys x 256] on bf16 MFMA (16x16x16): the transposed scores in
-//            their accumulator layout ARE the A operand; the V tile is parked row-major in LDS and read back through the
-//            transposing LDS load (ds_read_b64_tr_b16), which delivers the B operand (4 consecutive keys of one column).
+//            their accumulator layout ARE the A operand; the V tile is read back through the transposing LDS load
+//            (ds_read_b64_tr_b16), which delivers the B operand (4 consecutive keys of one column).
 //            P is split into two bf16 terms (p = hi + lo, error 2^-17), so the product keeps fp32-like accuracy.
-// Each wavefront walks its tiles with a one-tile-deep register FIFO: the registers of a K (V) fragment are refilled with
-// the next tile's fragment right after the MFMA (LDS store) that consumed them, so a tile's loads fly during the previous
-// tile's arithmetic.  The loop issues loads only, in the order of their use, which keeps every vmcnt wait partial.
+// Each wavefront walks its tiles with a one-tile-deep register FIFO: a register is refilled with the next tile's row right
+// after the LDS store that consumed it, so a tile's loads fly during the previous tile's arithmetic.  The loop issues
+// loads only, in the order of their use, which keeps every vmcnt wait partial.
 // Each wavefront keeps its own online-softmax state (m, l, O); the 4 wavefronts of a workgroup are merged through LDS and
-// the workgroup writes one unnormalised partial (m, l, O) per row; a second kernel merges the splits (batch.py:203-221).
+// the workgroup writes one unnormalised partial (m, l, O) per row and segment; a second kernel merges the partials
+// (batch.py:203-221).
 #include "qt_common.h"
 
 using namespace qt;
@@ -30,6 +36,7 @@ constexpr int GQA = AH / AKV;          // 4 query heads per KV head
 constexpr float SCALE = 0.0625f;       // 256^-0.5, batch.py:177
 constexpr float NEG = -3.0e38f;
 constexpr int VL_LD = AD + 16;         // row stride (elements) of the V tile in LDS: 544 bytes spread the 16 rows over the banks
+constexpr int KL_LD = AD + 8;          // row stride of the K tile: 528 bytes, the 16 rows of a fragment read start 4 banks apart
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 __device__ __forceinline__ void wave_lds_sync() {
@@ -93,28 +100,80 @@ __device__ __forceinline__ void pv_tile(f32x4 (&O)[16], const float (&p)[4], con
     }
 }
 
-// partial results of one workgroup: part_o [(b*KV + kvh)*nsplit + s][4*M rows][256] f32 (unnormalised),
-// part_ml [...][4*M][2] = (running max, running sum)
+constexpr int MAX_SEG = 2048;          // segments (2 per sequence) a launch can hold
+
+// Exclusive prefix of the segments' tile counts -> seg_start[0 .. nseg] (LDS); returns the total.  Rows whose slot or position
+// is out of range own no tiles (they are skipped by both kernels).  Every thread of the workgroup must call it.
+template <int M>
+__device__ __forceinline__ int build_segments(int* seg_start, const int* __restrict__ slots, const int* __restrict__ pos, int nseg,
+                                              int Lmax, int n_slots) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    for (int sg = tid; sg < nseg; sg += 256) {
+        const int b = sg / AKV, slot = slots[b], p0 = pos[b];
+        const bool ok = (unsigned)slot < (unsigned)n_slots && p0 >= 0 && p0 + M <= Lmax;
+        seg_start[sg + 1] = ok ? max(1, (p0 + 15) >> 4) : 0;
+    }
+    if (tid == 0) seg_start[0] = 0;
+    __syncthreads();
+    if (tid < 64) {
+        int carry = 0;
+        for (int base = 1; base <= nseg; base += 64) {
+            const int i = base + lane;
+            int v = i <= nseg ? seg_start[i] : 0;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int o = __shfl_up(v, d, 64);
+                if (lane >= d) v += o;
+            }
+            if (i <= nseg) seg_start[i] = v + carry;
+            carry += __shfl(v, 63, 64);
+        }
+    }
+    __syncthreads();
+    return seg_start[nseg];
+}
+// tiles per workgroup for `total` tiles spread over nwg workgroups, at least min_tiles
+__device__ __forceinline__ int tiles_per_wg(int total, int nwg, int min_tiles) { return max(min_tiles, (total + nwg - 1) / nwg); }
+
+// partial results: slot id = workgroup + segment (unique, and consecutive for the workgroups that share a segment);
+// part_o [slot][4*M rows][256] f32 (unnormalised), part_ml [slot][4*M][2] = (running max, running sum)
 template <int M>
 __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_new,
                                                            const bf16_t* __restrict__ v_new, bf16_t* Kp, bf16_t* Vp,
                                                            const int* __restrict__ slots, const int* __restrict__ pos,
-                                                           float* __restrict__ part_o, float* __restrict__ part_ml, int Lmax,
-                                                           int CH, int nsplit, int n_slots) {
+                                                           float* __restrict__ part_o, float* __restrict__ part_ml, int B,
+                                                           int Lmax, int min_tiles, int n_slots) {
     constexpr int R = 4 * M;
+    __shared__ int seg_start[MAX_SEG + 1];
     __shared__ __align__(16) bf16_t v_s[4][16 * VL_LD];          // one V tile per wavefront; reused for the merged O below
+    __shared__ __align__(16) bf16_t k_s[4][16 * KL_LD];          // one K tile per wavefront
     __shared__ __align__(16) float c_s[4][16];
     __shared__ float m_s[4][16], l_s[4][16];
     static_assert(sizeof(bf16_t) * 4 * 16 * VL_LD >= sizeof(float) * 16 * AD, "the merged O tile must fit into the V tiles");
     float (*o_s)[AD] = reinterpret_cast<float (*)[AD]>(&v_s[0][0]);
 
-    const int s = blockIdx.x % nsplit, bk = blockIdx.x / nsplit, kvh = bk % AKV, b = bk / AKV;
-    const int slot = slots[b], p0 = pos[b];
-    if ((unsigned)slot >= (unsigned)n_slots || p0 < 0 || p0 + M > Lmax) return;
-    const int lo = s * CH, hi = min(lo + CH, p0);
-    if (s > 0 && lo >= p0) return;                               // nothing to do for this split (split 0 always runs)
+    const int nseg = B * AKV;
+    const int total = build_segments<M>(seg_start, slots, pos, nseg, Lmax, n_slots);
+    const int per = tiles_per_wg(total, gridDim.x, min_tiles);
+    const int wt0 = blockIdx.x * per, wt1 = min(wt0 + per, total);
+    if (wt0 >= wt1) return;
+    int sg0 = 0;                                                 // the segment that holds tile wt0 (uniform binary search)
+    for (int lo_ = 0, hi_ = nseg; lo_ < hi_;) {
+        const int mid = (lo_ + hi_) >> 1;
+        if (seg_start[mid + 1] <= wt0) lo_ = mid + 1; else hi_ = mid;
+        sg0 = lo_;
+    }
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int hw = lane >> 5, cl = lane & 31;
+
+  for (int sg = sg0; sg < nseg && seg_start[sg] < wt1; sg++) {
+    const int ss = seg_start[sg], se = seg_start[sg + 1];
+    if (se == ss) continue;                                      // a skipped row
+    const int kvh = sg % AKV, b = sg / AKV;
+    const int slot = slots[b], p0 = pos[b];
+    const bool first = wt0 <= ss;                                // this workgroup holds the segment's first tile
+    const int lo = (max(wt0, ss) - ss) * 16, hi = min((min(wt1, se) - ss) * 16, p0);
+    const size_t pslot = (size_t)blockIdx.x + sg;
 
     // Q^T as the MFMA B operand: lane (row n, group g) holds q[row n][32 kb + 8 g .. + 8]; row n = token (n / 4), head n % 4
     bf16x8 bq[8];
@@ -137,52 +196,53 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     const bf16_t* kbase = Kp + pbase;
     const bf16_t* vbase = Vp + pbase;
     bf16_t* vl = v_s[w];
+    bf16_t* kl = k_s[w];
     const int ntiles = hi > lo ? (hi - lo + 15) / 16 : 0;
     if (w < ntiles) {
-        // fragment addresses of a tile; keys past `hi` re-read the tile's first key (they are masked / weighted by 0)
-        auto k_ptr = [&](int t) {
-            const int key0 = lo + t * 16;
-            return reinterpret_cast<const u32x4*>(kbase + (size_t)(key0 + n < hi ? key0 + n : key0) * AD) + g;
-        };
-        auto v_ptr = [&](int t, int i) {
+        // Row addresses of a tile: key 2i (lower half wavefront) / 2i + 1 (upper half), 8 columns per lane, so one load covers
+        // two whole 512-byte rows (a wavefront-wide load of 16 rows x 64 bytes streams about 15 % slower from HBM).  Keys past
+        // `hi` re-read the tile's first key (they are masked / weighted by 0).
+        auto row_ptr = [&](const bf16_t* base, int t, int i) {
             const int key0 = lo + t * 16, key = key0 + 2 * i + hw;
-            return reinterpret_cast<const u32x4*>(vbase + (size_t)(key < hi ? key : key0) * AD) + cl;
+            return reinterpret_cast<const u32x4*>(base + (size_t)(key < hi ? key : key0) * AD) + cl;
         };
         u32x4 a[8], vv[8];
-        {
-            const u32x4* kr = k_ptr(w);
 #pragma unroll
-            for (int kb = 0; kb < 8; kb++) a[kb] = kr[kb * 4];
+        for (int i = 0; i < 8; i++) a[i] = __builtin_nontemporal_load(row_ptr(kbase, w, i));
 #pragma unroll
-            for (int i = 0; i < 8; i++) vv[i] = *v_ptr(w, i);
-        }
+        for (int i = 0; i < 8; i++) vv[i] = __builtin_nontemporal_load(row_ptr(vbase, w, i));
         __builtin_amdgcn_sched_barrier(0);
         for (int t = w; t < ntiles; t += 4) {
             const int tn = t + 4 < ntiles ? t + 4 : t;           // the last step re-reads its own tile
             const int nvalid = min(16, hi - (lo + t * 16));
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            const u32x4* kr = k_ptr(tn);
+            // park both tiles row-major in LDS; every register is refilled with the next tile's row right after its store
 #pragma unroll
-            for (int kb = 0; kb < 8; kb++) {
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[kb]), bq[kb], acc, 0, 0, 0);
-                a[kb] = kr[kb * 4];
+            for (int i = 0; i < 8; i++) {
+                *reinterpret_cast<u32x4*>(kl + (2 * i + hw) * KL_LD + 8 * cl) = a[i];
+                a[i] = __builtin_nontemporal_load(row_ptr(kbase, tn, i));
                 __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                *reinterpret_cast<u32x4*>(vl + (2 * i + hw) * VL_LD + 8 * cl) = vv[i];
+                vv[i] = __builtin_nontemporal_load(row_ptr(vbase, tn, i));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            wave_lds_sync();
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) {                     // A operand: lane (key n, group g) holds k[key n][32 kb + 8 g .. + 8]
+                const u32x4 ka = *reinterpret_cast<const u32x4*>(kl + n * KL_LD + 32 * kb + 8 * g);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(ka), bq[kb], acc, 0, 0, 0);
             }
             float p[4];
             softmax_tile(acc, nvalid, false, m_run, l_run, p, c_s[w], lane);
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                // keys 2i (lower half wavefront) and 2i+1 (upper half), 8 columns per lane
-                *reinterpret_cast<u32x4*>(vl + (2 * i + hw) * VL_LD + 8 * cl) = vv[i];
-                vv[i] = *v_ptr(tn, i);
-                __builtin_amdgcn_sched_barrier(0);
-            }
             wave_lds_sync();
             pv_tile(O, p, vl, c_s[w], lane);
             wave_lds_sync();
         }
     }
-    if (s == 0 && w == 3) {
+    if (first && w == 3) {
         // The M new keys of this sequence, straight from the inputs (batch.py:143-145), with the causal rule among them:
         // key i is visible to query token j only if i <= j.  Not pipelined: it runs once per sequence.
         const bf16_t* kn = k_new + ((size_t)b * M * AKV + kvh) * AD;
@@ -210,7 +270,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
         pv_tile(O, p, vl, c_s[w], lane);
         wave_lds_sync();
     }
-    if (s == 0 && w == 0) {
+    if (first && w == 0) {
         // append (batch.py:196-201): row j of this sequence goes to pool position p0 + j
         for (int j = 0; j < M; j++) {
             const uint2 kk = reinterpret_cast<const uint2*>(k_new + ((size_t)(b * M + j) * AKV + kvh) * AD)[lane];
@@ -247,38 +307,44 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
         }
         __syncthreads();
     }
-    float* po = part_o + (size_t)blockIdx.x * R * AD;
+    float* po = part_o + pslot * R * AD;
     for (int i = tid; i < R * AD / 4; i += 256)
         reinterpret_cast<f32x4*>(po)[i] = reinterpret_cast<const f32x4*>(&o_s[0][0])[i];
     if (tid < R) {
         const float mm = fmaxf(fmaxf(m_s[0][tid], m_s[1][tid]), fmaxf(m_s[2][tid], m_s[3][tid]));
         float ll = 0.f;
         for (int ww = 0; ww < 4; ww++) ll += l_s[ww][tid] * __expf(m_s[ww][tid] - mm);
-        part_ml[((size_t)blockIdx.x * R + tid) * 2] = mm;
-        part_ml[((size_t)blockIdx.x * R + tid) * 2 + 1] = ll;
+        part_ml[(pslot * R + tid) * 2] = mm;
+        part_ml[(pslot * R + tid) * 2 + 1] = ll;
     }
+    __syncthreads();                                             // the LDS tiles are reused by the next segment
+  }
 }
 
-// merge of the splits: one workgroup of 256 threads per (sequence, kv head, row).  The per-split factors exp(m_s - m) are
-// computed by one thread each; then wavefront w sums the splits s = w, w+4, ... (a lane owns 4 output columns, four splits'
-// loads in flight) and the four wavefronts are added in order.
+// merge of the partial results: one workgroup of 256 threads per (segment, row).  The per-partial factors exp(m_s - m) are
+// computed by one thread each; then wavefront w sums the partials s = w, w+4, ... (a lane owns 4 output columns, four
+// partials' loads in flight) and the four wavefronts are added in order.
 constexpr int MAX_SPLITS = 4096;
 template <int M>
 __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                          const int* __restrict__ slots, const int* __restrict__ pos,
-                                                         bf16_t* __restrict__ out, int Lmax, int CH, int nsplit, int n_slots) {
+                                                         bf16_t* __restrict__ out, int B, int Lmax, int nwg, int min_tiles,
+                                                         int n_slots) {
     constexpr int R = 4 * M;
+    __shared__ int seg_start[MAX_SEG + 1];
     __shared__ float fs_s[MAX_SPLITS];
     __shared__ float red_m[4], red_l[4];
     __shared__ __align__(16) float acc_s[4][AD];
-    const int r = blockIdx.x % R, bk = blockIdx.x / R, kvh = bk % AKV, b = bk / AKV;
+    const int r = blockIdx.x % R, sg = blockIdx.x / R, kvh = sg % AKV, b = sg / AKV;
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
-    const int slot = slots[b], p0 = pos[b];
-    if ((unsigned)slot >= (unsigned)n_slots || p0 < 0 || p0 + M > Lmax) return;
-    const int ns = max(1, min(nsplit, (p0 + CH - 1) / CH));
-    const size_t base = (size_t)bk * nsplit;
-    const float* ml = part_ml + (base * R + r) * 2;              // split stride 2 R floats
-    const float* po = part_o + (base * R + r) * AD + lane * 4;   // split stride R * AD floats
+    const int total = build_segments<M>(seg_start, slots, pos, B * AKV, Lmax, n_slots);
+    const int ss = seg_start[sg], se = seg_start[sg + 1];
+    if (se == ss) return;                                        // a skipped row
+    const int per = tiles_per_wg(total, nwg, min_tiles);
+    const int wg0 = ss / per, ns = (se - 1) / per - wg0 + 1;     // the workgroups that hold tiles of this segment
+    const size_t base = (size_t)wg0 + sg;                        // their partials sit in consecutive slots
+    const float* ml = part_ml + (base * R + r) * 2;              // slot stride 2 R floats
+    const float* po = part_o + (base * R + r) * AD + lane * 4;   // slot stride R * AD floats
     float mx = NEG;
     for (int s = tid; s < ns; s += 256) mx = fmaxf(mx, ml[(size_t)s * 2 * R]);
     mx = wave_max(mx);
@@ -317,11 +383,25 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
 
 extern "C" {
 
-// bytes of workspace qt_gqa_attn_decode needs for (B sequences, M rows each, pool length Lmax, split size CH)
+constexpr int MAX_WG = 1024;           // upper bound of the partial kernel's grid (one workgroup per CU)
+
+static int partial_grid() {            // one workgroup per CU of the current device: measured faster than two (the stream is
+                                       // bandwidth-bound with 64 KiB in flight per CU; a second workgroup only adds queueing)
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    return cus < MAX_WG ? cus : MAX_WG;
+}
+
+// bytes of workspace qt_gqa_attn_decode needs for (B sequences, M rows each, pool length Lmax); CH is accepted for callers
+// written against the fixed-split form and does not change the size
 long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH) {
     if (B < 0 || M < 1 || Lmax < 1 || CH < 16) return -1;
-    const long nsplit = (Lmax + CH - 1) / CH;
-    return (long)B * AKV * nsplit * (4 * M) * (AD + 2) * 4;
+    return ((long)MAX_WG + (long)B * AKV) * (4 * M) * (AD + 2) * 4;
 }
 
 int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
@@ -329,21 +409,23 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
                        int n_slots, int CH, hipStream_t stream) {
     if (!q || !k_new || !v_new || !Kp || !Vp || !slots || !pos || !out || !workspace) return QT_ERR_NULL;
     if (B < 0 || Lmax < 1 || n_slots < 1 || CH < 16 || CH % 16) return QT_ERR_DIM;
-    if (M < 1 || M > 4) return QT_ERR_UNSUPPORTED;
+    if (M < 1 || M > 4 || B * AKV > MAX_SEG) return QT_ERR_UNSUPPORTED;
     if (B == 0) return QT_OK;
     for (const void* p : {q, k_new, v_new, (const void*)Kp, (const void*)Vp, (const void*)workspace})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if (workspace_bytes < qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)) return -6;
-    const int nsplit = (Lmax + CH - 1) / CH;
-    if (nsplit > MAX_SPLITS) return QT_ERR_UNSUPPORTED;
+    const int min_tiles = CH / 16;                               // a workgroup takes at least CH keys
+    const long max_tiles = (long)B * AKV * ((Lmax + 15) / 16);
+    const long want = (max_tiles + min_tiles - 1) / min_tiles;
+    const int nwg = (int)(want < partial_grid() ? want : partial_grid());
     float* part_o = (float*)workspace;
-    float* part_ml = part_o + (size_t)B * AKV * nsplit * (4 * M) * AD;
-    const dim3 g1((unsigned)(B * AKV * nsplit)), g2((unsigned)(B * AKV * 4 * M));
+    float* part_ml = part_o + ((size_t)MAX_WG + (size_t)B * AKV) * (4 * M) * AD;
+    const dim3 g1((unsigned)nwg), g2((unsigned)(B * AKV * 4 * M));
 #define QT_ATTN_LAUNCH(MM)                                                                                                \
     hipLaunchKernelGGL(attn_partial_kernel<MM>, g1, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)k_new,         \
-                       (const bf16_t*)v_new, (bf16_t*)Kp, (bf16_t*)Vp, slots, pos, part_o, part_ml, Lmax, CH, nsplit, n_slots); \
-    hipLaunchKernelGGL(attn_merge_kernel<MM>, g2, dim3(256), 0, stream, part_o, part_ml, slots, pos, (bf16_t*)out, Lmax, CH, \
-                       nsplit, n_slots);
+                       (const bf16_t*)v_new, (bf16_t*)Kp, (bf16_t*)Vp, slots, pos, part_o, part_ml, B, Lmax, min_tiles, n_slots); \
+    hipLaunchKernelGGL(attn_merge_kernel<MM>, g2, dim3(256), 0, stream, part_o, part_ml, slots, pos, (bf16_t*)out, B, Lmax, nwg, \
+                       min_tiles, n_slots);
     switch (M) {
         case 1: QT_ATTN_LAUNCH(1) break;
         case 2: QT_ATTN_LAUNCH(2) break;
