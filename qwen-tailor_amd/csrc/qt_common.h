@@ -125,7 +125,7 @@ __device__ __forceinline__ float conv_silu_tab(const bf16_t* tab, float w0, floa
     return silu_lookup(tab, f2bf(s));
 }
 // Branch-free form for hot loops: inputs outside the table return a placeholder and set `rare`; the caller then re-evaluates
-// that group of channels through conv8_silu_slow, which is kept out of line so that the hot loop stays small.
+// that group of channels through conv8_silu_slow in one unlikely block (one branch per 8 channels instead of one per channel).
 __device__ __forceinline__ float silu_lookup_fast(const bf16_t* tab, bf16_t xb, bool& rare) {
     const unsigned idx = (xb & 0x7fffu) - SILU_TAB_LO * 128;                      // wraps for small |x|
     const bool in_tab = idx < (unsigned)SILU_TAB_N;
@@ -135,7 +135,7 @@ __device__ __forceinline__ float silu_lookup_fast(const bf16_t* tab, bf16_t xb, 
 __device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]);
 // conv4 + silu of 8 consecutive channels of one token: rows x0..x3 (oldest first, 8 bf16 each), taps wt (4 bf16 per channel)
 struct F8 { float v[8]; };
-static __device__ __attribute__((noinline)) F8 conv8_silu_slow(uint4 x0, uint4 x1, uint4 x2, uint4 x3, uint4 w0, uint4 w1, uint4 w2,
+static __device__ __attribute__((always_inline)) inline F8 conv8_silu_slow(uint4 x0, uint4 x1, uint4 x2, uint4 x3, uint4 w0, uint4 w1, uint4 w2,
                                                                uint4 w3);
 __device__ __forceinline__ void conv8_silu_tab(const bf16_t* tab, const uint4& x0, const uint4& x1, const uint4& x2,
                                                const uint4& x3, const uint4 (&wt)[4], float (&u)[8]) {
@@ -166,7 +166,7 @@ __device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]) {
     f[4] = lo_bf(w.z); f[5] = hi_bf(w.z); f[6] = lo_bf(w.w); f[7] = hi_bf(w.w);
 }
 
-static __device__ __attribute__((noinline)) F8 conv8_silu_slow(uint4 x0, uint4 x1, uint4 x2, uint4 x3, uint4 w0, uint4 w1, uint4 w2,
+static __device__ __attribute__((always_inline)) inline F8 conv8_silu_slow(uint4 x0, uint4 x1, uint4 x2, uint4 x3, uint4 w0, uint4 w1, uint4 w2,
                                                                uint4 w3) {
     float a[8], b[8], c[8], d[8];
     unpack8(x0, a);
