@@ -21,6 +21,11 @@ if ROOT not in sys.path:
 HV, DK, DV, CD, PW = 16, 128, 128, 6144, 8224
 N_LAYERS = 18
 HBM_PEAK_GBS = 8000.0
+# HBM bytes of one B = 64 decode launch measured with rocprofv3 --pmc (FETCH_SIZE 34 563.5 KiB x 1.9993 + WRITE_SIZE 68 142.9 KiB,
+# scale factors from a 64 MiB copy; profiles/gdn_decode_wide_kernel_B64.md).  Reported as `roofline.traffic` for that batch only.
+DECODE_TRAFFIC_B64 = int((34563.5 * 1.9993 + 68142.9) * 1024)
+# same for the three kernels of the T = 2048 prefill (profiles/gdn_prefill_T2048.md)
+PREFILL_TRAFFIC_T2048 = int(((17328.8 + 16941.0 + 23758.5) * 1.9993 + 49204 + 25600 + 8192) * 1024)
 
 
 def decode_bytes(B):
@@ -109,10 +114,10 @@ def time_graph(torch, fn, reps=200, inner=10):
             for _ in range(inner):
                 fn()
     torch.cuda.synchronize()
-    for _ in range(3):
+    n = max(1, reps // inner)
+    for _ in range(max(3, n // 2)):                   # warm-up replays: clocks and caches settle before the timed region
         g.replay()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    n = max(1, reps // inner)
     torch.cuda.synchronize()
     e0.record()
     for _ in range(n):
@@ -137,16 +142,14 @@ def bench_prefill(torch, qt, dev, T, seed=1002):
     dtb = (torch.randn(HV, generator=g) * 0.1).to(dev)
     gw = torch.ones(DV, device=dev)
     S0 = (torch.randn((1, HV, DV, DK), generator=g) * 0.02).to(dev)
-    q, k, v, ops, U, gC = qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb)
-    y, _ = qt.gdn_nax.phase_b(proj, None, None, ops, U, gC, S0)
+    _, _, _, ops, U, gC = qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb, want_qkv=False)
     t_all = time_graph(torch, lambda: qt.prefill.gdn_core(proj, cs, S0, cw, A, dtb, gw), reps=60, inner=3)
-    t_a = time_graph(torch, lambda: qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb), reps=60, inner=3)
-    t_b = time_graph(torch, lambda: qt.gdn_nax.phase_b(proj, None, None, ops, U, gC, S0), reps=60, inner=3)
-    t_n = time_graph(torch, lambda: qt.prefill.gated_norm(y, proj, gw), reps=60, inner=3)
+    t_a = time_graph(torch, lambda: qt.gdn_nax._phase_a(proj, cs[0], cw, A, dtb, want_qkv=False), reps=60, inner=3)
+    t_b = time_graph(torch, lambda: qt.gdn_nax.phase_b_norm(proj, ops, U, gC, S0, gw), reps=60, inner=3)
     flop = GDN_FLOP_PER_TOKEN * T
     hbm = T * PW * 2 + T * 2048 * 2 + 2 * HV * DV * DK * 4          # compulsory: projection rows in, gated output out, state in + out
-    return {"T": T, "tok_per_s": T / t_all, "us": t_all * 1e6, "phase_a_us": t_a * 1e6, "phase_b_us": t_b * 1e6,
-            "gated_norm_us": t_n * 1e6, "mfma_tflops": flop / t_all / 1e12, "mfma_frac": flop / t_all / 1e12 / MFMA_PEAK_TFLOPS,
+    return {"T": T, "tok_per_s": T / t_all, "us": t_all * 1e6, "conv_phase_a_us": t_a * 1e6,
+            "chain_output_norm_us": t_b * 1e6, "mfma_tflops": flop / t_all / 1e12, "mfma_frac": flop / t_all / 1e12 / MFMA_PEAK_TFLOPS,
             "compulsory_hbm_GBps": hbm / t_all / 1e9}
 
 
@@ -235,7 +238,7 @@ def cpu_baseline(B, budget_s=12.0):
         C.decode_step(proj, conv, cw, A_log, dtb, ssm, slots, pos + n + 1, acc64=False, nthreads=threads)
         n += 1
         el = time.perf_counter() - t0
-        if el >= budget_s or n >= 5000:
+        if el >= budget_s or n >= 20000:
             break
     return {"value": n / el, "unit": "steps/s", "cores": threads, "kind": "port",
             "sample": f"{n} decode steps at B={B} on one layer pool, C restatement of the reference step (oracle/gdn_oracle.c), "
@@ -351,7 +354,7 @@ def main():
                                f"rotating over {N_LAYERS} layer pools", "batch": B, "layer_pools": N_LAYERS,
                    "launch": "eager" if args.no_graph else "hip-graph of 18 launches"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": None, "kernel": "gdn_decode_wide_kernel<4>" if B >= 64 else "gdn_decode_kernel", "bytes_per_launch": decode_bytes(B),
+                     "traffic": DECODE_TRAFFIC_B64 if B == 64 else None, "kernel": "gdn_decode_wide_kernel<4>" if B >= 64 else "gdn_decode_kernel", "bytes_per_launch": decode_bytes(B),
                      "avg_launch_us": launch_s * 1e6},
         "extras": extras,
     }
@@ -361,7 +364,7 @@ def main():
                             "config": {"workload": "configs[2]: conv + chunked GDN (chunk 64) + gated RMSNorm, B=1, T=2048, 16 heads, "
                                                    "nonzero initial state"},
                             "roofline": {"bound": "mfma", "achieved": p2k["mfma_tflops"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                         "frac": p2k["mfma_frac"], "traffic": None}}
+                                         "frac": p2k["mfma_frac"], "traffic": PREFILL_TRAFFIC_T2048}}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B)
     print(json.dumps(out))
