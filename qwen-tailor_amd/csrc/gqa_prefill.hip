@@ -2,14 +2,17 @@
 // Replaces the call mx.fast.scaled_dot_product_attention(q, K[:, :, :kv_len], V[:, :, :kv_len], scale=256**-0.5,
 // mask="causal") of the reference's full-attention layers (qwen35/model.py:160-167, qwen35/prefill.py:468).
 //
-// One workgroup = 16 query rows x the 4 query heads that share a KV head (one head per wavefront), so a K / V tile of 64
-// keys is fetched from HBM once and staged in LDS for all four.  Per tile and wavefront:
+// One workgroup = 32 query rows x the 4 query heads that share a KV head: wavefront w owns the 16 rows of block w >> 1 for
+// the two heads 2 (w & 1), 2 (w & 1) + 1, so a K / V tile of 64 keys is fetched from HBM once and staged in LDS for all of
+// them, and every K or V fragment a wavefront reads from LDS feeds two MFMAs (one per head): the kernel is bound by MFMA
+// issue and LDS bandwidth in equal parts instead of by LDS bandwidth alone.  Per tile and wavefront:
 //     S^T[keys x rows] = K_tile . Q^T     A = K rows from LDS, B = Q^T resident in registers (16x16x32 bf16 MFMA)
 //     online softmax in the accumulator layout: lane (row n, group g) holds keys 4g..4g+3 of each 16-key sub-tile
 //     O[rows x 256]   += P . V            A = two exponentiated S^T accumulators packed to bf16 (they ARE the A operand
 //                                         when a 32-key block is enumerated as 16 (j >> 2) + 4 g + (j & 3)),
 //                                         B = V through the transposing LDS load (4 consecutive keys of one column)
-// The next tile travels global -> registers while the current one is consumed; two barriers per tile.
+// The next tile travels global -> registers while the current one is consumed; two barriers per tile.  A wavefront runs
+// at one per SIMD and keeps about 400 registers (Q^T of two heads, two 16 x 256 accumulators, the tile in flight).
 #include "qt_common.h"
 
 using namespace qt;
@@ -34,31 +37,38 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-__global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
+// NH = heads per wavefront: 2 (32 query rows per workgroup, as described above) for long sequences; 1 (16 rows per workgroup,
+// one head per wavefront: twice the workgroups, LDS-bound) when the launch would otherwise leave CUs idle.
+template <int NH>
+__global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
                                                            const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
                                                            int q_pos0, long q_head_stride, long kv_head_stride) {
     __shared__ __align__(16) bf16_t k_s[KT * KS_LD];
     __shared__ __align__(16) bf16_t v_s[KT * VS_LD];
-    __shared__ __align__(16) float c_s[4][16];
+    __shared__ __align__(16) float c_s[4][2][16];
+    constexpr int RB = 16 * NH;
     const int rb = gridDim.x - 1 - blockIdx.x;                   // long rows first
     const int kvh = blockIdx.y;
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
-    const int h = kvh * (AH / AKV) + w;
-    const int r0 = rb * 16, row = r0 + n;
+    const int h0 = kvh * (AH / AKV) + (NH == 2 ? 2 * (w & 1) : w);       // this wavefront's heads: h0 (, h0 + 1)
+    const int r0 = rb * RB + (NH == 2 ? 16 * (w >> 1) : 0), row = r0 + n;   // this wavefront's 16 rows
     const bool row_ok = row < S;
     const int my_last = q_pos0 + row;                            // last key this query row may see
-    const int kend = min(L, q_pos0 + min(r0 + 15, S - 1) + 1);   // keys any row of this block sees
+    const int kend = min(L, q_pos0 + min(rb * RB + RB - 1, S - 1) + 1);        // keys any row of the workgroup sees
     const int ntiles = (kend + KT - 1) / KT;
+    const int kend_w = r0 < S ? min(L, q_pos0 + min(r0 + 15, S - 1) + 1) : 0;  // keys any row of this wavefront sees
+    const int ntiles_w = (kend_w + KT - 1) / KT;
 
-    // Q^T as the B operand of the score MFMA: lane (row n, group g) holds q[row][32 kb + 8 g .. + 8]
-    bf16x8 bq[8];
-    {
-        const u32x4* qr = reinterpret_cast<const u32x4*>(q + (size_t)h * q_head_stride + (size_t)(row_ok ? row : r0) * AD);
+    // Q^T as the B operand of the score MFMA: lane (row n, group g) holds q[row][32 kb + 8 g .. + 8], for both heads
+    bf16x8 bq[NH][8];
+#pragma unroll
+    for (int hh = 0; hh < NH; hh++) {
+        const u32x4* qr = reinterpret_cast<const u32x4*>(q + (size_t)(h0 + hh) * q_head_stride + (size_t)(row_ok ? row : 0) * AD);
 #pragma unroll
         for (int kb = 0; kb < 8; kb++) {
             u32x4 v = qr[kb * 4 + g];
             if (!row_ok) v = u32x4{0, 0, 0, 0};
-            bq[kb] = __builtin_bit_cast(bf16x8, v);
+            bq[hh][kb] = __builtin_bit_cast(bf16x8, v);
         }
     }
     // tile loader: thread (tid >> 5, tid & 31) moves 16 bytes of the rows tid >> 5 + 8 i, i = 0..7, of K and of V
@@ -76,10 +86,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
     };
     load_tile(0);
 
-    float m_run = NEG, l_run = 0.f;
-    f32x4 O[16];
+    float m_run[NH], l_run[NH];
+    f32x4 O[NH][16];
 #pragma unroll
-    for (int j = 0; j < 16; j++) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int hh = 0; hh < NH; hh++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) O[hh][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int hh = 0; hh < NH; hh++) m_run[hh] = NEG, l_run[hh] = 0.f;
     const bf16_t* ka = k_s + n * KS_LD + 8 * g;                  // A operand of the scores: row 16 kt + n, columns 32 kb + 8 g
     // transposing load: within 16 lanes, lane 4q + i receives element i of the 8-byte chunks addressed by lanes q, q+4,
     // q+8, q+12; lane n of group g points at key 4g + n/4, columns 4 (n%4).. of the block and receives keys 4g..4g+3 of column n
@@ -94,60 +108,67 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
         }
         if (t + 1 < ntiles) load_tile(t + 1);
         __syncthreads();
+        if (t >= ntiles_w) continue;                             // wavefront-uniform: the upper row block may see one tile more
 
-        // scores: the 8 K fragments of a 16-key sub-tile are read in one batch, one sub-tile ahead of the MFMAs that use them
-        f32x4 acc[4];
-        bf16x8 Af[2][8];
-#pragma unroll
-        for (int kb = 0; kb < 8; kb++) Af[0][kb] = *reinterpret_cast<const bf16x8*>(ka + 32 * kb);
+        // scores: each K fragment multiplies the Q^T of both heads (the compiler overlaps the next sub-tile's LDS reads with
+        // these MFMAs as registers allow)
+        f32x4 acc[NH][4];
+        bf16x8 Af[8];
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
-            __builtin_amdgcn_sched_barrier(0);
-            if (kt < 3) {
 #pragma unroll
-                for (int kb = 0; kb < 8; kb++)
-                    Af[(kt + 1) & 1][kb] = *reinterpret_cast<const bf16x8*>(ka + 16 * (kt + 1) * KS_LD + 32 * kb);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            acc[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int kb = 0; kb < 8; kb++) Af[kb] = *reinterpret_cast<const bf16x8*>(ka + 16 * kt * KS_LD + 32 * kb);
+#pragma unroll
+            for (int hh = 0; hh < NH; hh++) acc[hh][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kb = 0; kb < 8; kb++)
-                acc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kt & 1][kb], bq[kb], acc[kt], 0, 0, 0);
+#pragma unroll
+                for (int hh = 0; hh < NH; hh++)
+                    acc[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kb], bq[hh][kb], acc[hh][kt], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        float sc[4][4], mx = NEG;
+        s16x8 P[NH][2];
+        bool rescale = false;
 #pragma unroll
-        for (int kt = 0; kt < 4; kt++)
+        for (int hh = 0; hh < NH; hh++) {
+            float sc[4][4], mx = NEG;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int key = t * KT + 16 * kt + 4 * g + i;
-                sc[kt][i] = (key <= my_last && key < L) ? acc[kt][i] * SCALE : NEG;
-                mx = fmaxf(mx, sc[kt][i]);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        const float corr = __expf(m_run - m_new);                // m_run = NEG initially: exp(-huge) = 0
-        float ps = 0.f;
-        s16x8 P[2];
+            for (int kt = 0; kt < 4; kt++)
 #pragma unroll
-        for (int kt = 0; kt < 4; kt++)
+                for (int i = 0; i < 4; i++) {
+                    const int key = t * KT + 16 * kt + 4 * g + i;
+                    sc[kt][i] = (key <= my_last && key < L) ? acc[hh][kt][i] * SCALE : NEG;
+                    mx = fmaxf(mx, sc[kt][i]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run[hh], mx);
+            const float corr = __expf(m_run[hh] - m_new);        // m_run = NEG initially: exp(-huge) = 0
+            float ps = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float pv = sc[kt][i] > 0.5f * NEG ? __expf(sc[kt][i] - m_new) : 0.f;
-                ps += pv;
-                P[kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(pv);
-            }
-        l_run = l_run * corr + ps;                               // this lane's share; summed over g at the end
-        m_run = m_new;
-        if (g == 0) c_s[w][n] = corr;
-        wave_lds_sync();
-        const f32x4 c4 = *reinterpret_cast<const f32x4*>(&c_s[w][4 * g]);
-        if (__any(corr != 1.0f)) {                               // wavefront-uniform: most tiles leave every row's max alone
+            for (int kt = 0; kt < 4; kt++)
 #pragma unroll
-            for (int j = 0; j < 16; j++) O[j] *= c4;
+                for (int i = 0; i < 4; i++) {
+                    const float pv = sc[kt][i] > 0.5f * NEG ? __expf(sc[kt][i] - m_new) : 0.f;
+                    ps += pv;
+                    P[hh][kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(pv);
+                }
+            l_run[hh] = l_run[hh] * corr + ps;                   // this lane's share; summed over g at the end
+            m_run[hh] = m_new;
+            if (g == 0) c_s[w][hh][n] = corr;
+            rescale |= corr != 1.0f;
         }
-        // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs
+        wave_lds_sync();
+        if (__any(rescale)) {                                    // wavefront-uniform: most tiles leave every row's max alone
+#pragma unroll
+            for (int hh = 0; hh < NH; hh++) {
+                const f32x4 c4 = *reinterpret_cast<const f32x4*>(&c_s[w][hh][4 * g]);
+#pragma unroll
+                for (int j = 0; j < 16; j++) O[hh][j] *= c4;
+            }
+        }
+        // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs and serve
+        // both heads
         auto v_frag = [&](int j, int q4) {
             return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                 (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * VS_LD + 16 * j)));
@@ -169,27 +190,36 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const bf16_t* __restr
 #pragma unroll
             for (int pp = 0; pp < 2; pp++) {
                 const s16x8 B = __builtin_shufflevector(Bf[j % 3][2 * pp], Bf[j % 3][2 * pp + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                O[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[pp]), __builtin_bit_cast(bf16x8, B),
-                                                              O[j], 0, 0, 0);
+#pragma unroll
+                for (int hh = 0; hh < NH; hh++)
+                    O[hh][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[hh][pp]),
+                                                                      __builtin_bit_cast(bf16x8, B), O[hh][j], 0, 0, 0);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
         wave_lds_sync();                                         // c_s is rewritten by the next tile
     }
     // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
-    if (g == 0) c_s[w][n] = l_run;
+#pragma unroll
+    for (int hh = 0; hh < NH; hh++) {
+        float l = l_run[hh];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        if (g == 0) c_s[w][hh][n] = l;
+    }
     wave_lds_sync();
-    const f32x4 l4 = *reinterpret_cast<const f32x4*>(&c_s[w][4 * g]);
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int orow = r0 + 4 * g + r;
-        if (orow < S) {
-            const float inv = 1.0f / l4[r];
-            bf16_t* dst = out + (size_t)h * q_head_stride + (size_t)orow * AD + n;
+    for (int hh = 0; hh < NH; hh++) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&c_s[w][hh][4 * g]);
 #pragma unroll
-            for (int j = 0; j < 16; j++) dst[16 * j] = f2bf(O[j][r] * inv);
+        for (int r = 0; r < 4; r++) {
+            const int orow = r0 + 4 * g + r;
+            if (orow < S) {
+                const float inv = 1.0f / l4[r];
+                bf16_t* dst = out + (size_t)(h0 + hh) * q_head_stride + (size_t)orow * AD + n;
+#pragma unroll
+                for (int j = 0; j < 16; j++) dst[16 * j] = f2bf(O[hh][j][r] * inv);
+            }
         }
     }
 }
@@ -213,8 +243,13 @@ int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out
     for (const void* p : {q, K, V, (const void*)out})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if ((q_head_stride | kv_head_stride) & 7) return QT_ERR_ALIGN;
-    hipLaunchKernelGGL(attn_prefill_kernel, dim3((S + 15) / 16, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
-                       (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride);
+    // two heads per wavefront once 32-row blocks alone give every CU at least two workgroups; below that, 16-row blocks
+    if ((S + 31) / 32 * AKV >= 512)
+        hipLaunchKernelGGL(attn_prefill_kernel<2>, dim3((S + 31) / 32, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
+                           (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride);
+    else
+        hipLaunchKernelGGL(attn_prefill_kernel<1>, dim3((S + 15) / 16, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
+                           (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

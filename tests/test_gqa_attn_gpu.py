@@ -151,3 +151,22 @@ def test_prefill_causal_2048(qt, dev):
     with pytest.raises(ValueError):
         qt.attention.scaled_dot_product_attention(to_dev(q, dev, BF16)[None], to_dev(K, dev, BF16)[None], to_dev(V, dev, BF16)[None],
                                                   scale=256 ** -0.5, mask=None)
+
+
+def test_prefill_causal_8192_two_heads_per_wavefront(qt, dev):
+    """S = 8192 (BASELINE's long prefill; the launch uses 32-row workgroups with two heads per wavefront): a sample of query
+    rows, including block borders and the first / last rows, against the float64 oracle evaluated for those rows only"""
+    rng = np.random.default_rng(8192)
+    S = 8192
+    g = torch.Generator().manual_seed(8192)
+    q = torch.randn((8, S, 256), generator=g).bfloat16()
+    K = torch.randn((2, S, 256), generator=g).bfloat16()
+    V = torch.randn((2, S, 256), generator=g).bfloat16()
+    o = to_np(qt.attention.scaled_dot_product_attention(q.to(dev)[None], K.to(dev)[None], V.to(dev)[None], scale=256 ** -0.5,
+                                                        mask="causal"))[0]
+    rows = sorted(set([0, 1, 15, 16, 31, 32, 33, 63, 64, 65, 4095, 4096, 8159, 8160, 8176, 8191] + [int(r) for r in rng.integers(0, S, 40)]))
+    qn, Kn, Vn = q.float().numpy(), K.float().numpy(), V.float().numpy()
+    for r in rows:
+        ref = O.sdpa_causal(qn[:, r:r + 1], Kn[:, :r + 1], Vn[:, :r + 1])            # the row at position r sees keys 0..r
+        check_attn(f"S=8192 row {r}", o[:, r:r + 1], ref)
+    check_equal("row 0 == v[0]", o[:, 0], np.repeat(Vn[:, 0], 4, axis=0))
