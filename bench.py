@@ -217,6 +217,28 @@ def bench_attn_prefill(torch, qt, dev, S=2048, seed=7):
     return {"S": S, "us": t * 1e6, "tflops": flop / t / 1e12, "mfma_frac": flop / t / 1e12 / MFMA_PEAK_TFLOPS}
 
 
+def bench_state_admission(torch, qt, dev, pos=2048, Lmax=4096, slots=8):
+    """Admission of one prefilled sequence into its slot (Pools.load, qwen35/batch.py:431-447): 18 layers of recurrent state
+    (1 MiB + 36 KiB each) and 6 layers of K / V rows (pos x 2 heads x 512 B each, twice), 60 strided copies."""
+    cfg = qt.model.Cfg()
+    P = qt.batch.Pools(cfg, slots, Lmax, device=dev)
+    nl, na = len(P.conv), len(P.K)
+    bf = torch.bfloat16
+    state = {"conv": [torch.zeros((1, 3, CD), dtype=bf, device=dev) for _ in range(nl)],
+             "ssm": [torch.zeros((1, HV, DV, DK), device=dev) for _ in range(nl)],
+             "kv": [(torch.zeros((1, cfg.n_kv, pos, cfg.head_dim), dtype=bf, device=dev),
+                     torch.zeros((1, cfg.n_kv, pos, cfg.head_dim), dtype=bf, device=dev)) for _ in range(na)]}
+    it = [0]
+
+    def step():
+        P.load(it[0] % slots, state, pos)
+        it[0] += 1
+    t = time_graph(torch, step, reps=slots * 6, inner=slots)
+    nbytes = 2 * (nl * (HV * DV * DK * 4 + 3 * CD * 2) + na * 2 * cfg.n_kv * pos * cfg.head_dim * 2)      # read + written
+    return {"pos": pos, "copies": 2 * nl + 2 * na, "us": t * 1e6, "bytes": nbytes, "GBps": nbytes / t / 1e9,
+            "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
+
+
 def cpu_baseline(B, budget_s=12.0):
     """The C restatement of the decode step (float accumulation) timed on this host's cores: a reported baseline only."""
     import numpy as np
@@ -343,7 +365,8 @@ def main():
         extras["attn_decode_config3"] = bench_attn(torch, qt, dev, 16, 1, 512, 32768, 1003)
         torch.cuda.empty_cache()
         extras["attn_verify_config4"] = bench_attn(torch, qt, dev, 16, 4, 1024, 8192, 1004)
-        extras["attn_prefill_causal"] = bench_attn_prefill(torch, qt, dev)
+        extras["attn_prefill_causal"] = [bench_attn_prefill(torch, qt, dev, S) for S in (2048, 8192)]
+        extras["state_admission"] = bench_state_admission(torch, qt, dev)
 
     out = {
         "metric": "GDN decode steps/s @B=64 (% HBM peak); GDN prefill tok/s @2048 (% MFMA)",

@@ -120,6 +120,19 @@ long qt_gqa_prefill_workspace_bytes(int L);
 int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out, void* workspace, long workspace_bytes, int S,
                           int L, int q_pos0, long q_head_stride, long kv_head_stride, qt_stream_t stream);
 
+/* batch.blit (qwen35/batch.py:365-372), the in-place strided copy behind Pools.load / read (batch.py:431-462) and the
+ * scheduler's plain <-> speculative state moves (qwen35/serve.py:310-348):
+ *     dst.flat[d0 + y*dstride + i] = src.flat[s0 + y*sstride + i]   for i < n, y < ny   (offsets and strides in elements)
+ * elem_size = 2 (bf16) or 4 (f32); ny <= 65535; the ranges written must not overlap the ranges read. */
+int qt_blit(void* dst, const void* src, int elem_size, long n, long d0, long s0, long ny, long dstride, long sstride,
+            qt_stream_t stream);
+
+/* `count` qt_blit copies in one launch (a sequence's admission is 48 of them: Pools.load, qwen35/batch.py:431-447).
+ * dst[k], src[k]: device base pointers (the arrays themselves are host memory); meta[7k .. 7k+6] (host memory) =
+ * { elem_size, n, d0, s0, ny, dstride, sstride } as for qt_blit.  Every copy must be 16-byte granular (base pointers, and
+ * n, d0, s0, dstride, sstride in bytes), otherwise -2 and nothing is launched. */
+int qt_blit_batch(void* const* dst, const void* const* src, const long* meta, int count, qt_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

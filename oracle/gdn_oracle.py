@@ -373,3 +373,15 @@ def sdpa_causal(q, K, V, q_pos0=None):
         w = np.exp(sc - sc.max(-1, keepdims=True))
         o[h] = BF((w @ V[kvh] / w.sum(-1, keepdims=True)).astype(np.float32))
     return o
+
+
+# ------------------------------------------------------------------------------------------------
+# state admission (batch.py:349-372): the strided in-place copy
+# ------------------------------------------------------------------------------------------------
+def blit(dst, src, n, d0, s0, ny=1, dstride=0, sstride=0):
+    """dst.flat[d0 + y*dstride + i] = src.flat[s0 + y*sstride + i] for i < n, y < ny, in place on the numpy array `dst`
+    (qwen35/batch.py:349-372, one element per thread of a (n, ny) grid)."""
+    d, s = dst.reshape(-1), np.asarray(src).reshape(-1)
+    for y in range(ny):
+        d[d0 + y * dstride:d0 + y * dstride + n] = s[s0 + y * sstride:s0 + y * sstride + n]
+    return dst

@@ -32,6 +32,8 @@ _SIGS = {
     "qt_gqa_prefill_causal": [_vp] * 5 + [_l, _i, _i, _i, _l, _l, _vp],
     "qt_gdn_phase_a": [_vp] * 9 + [_i, _vp],
     "qt_gdn_phase_a_conv": [_vp] * 13 + [_i, _vp],
+    "qt_blit": [_vp, _vp, _i, _l, _l, _l, _l, _l, _l, _vp],
+    "qt_blit_batch": [_vp, _vp, _vp, _i, _vp],
 }
 
 

@@ -90,6 +90,47 @@ def gnorm_rows(y, proj, gw, eps=1e-6):
     return out
 
 
+def blit(dst, src, n, d0, s0, ny=1, dstride=0, sstride=0):
+    """dst.flat[d0 + y*dstride + i] = src.flat[s0 + y*sstride + i] for i < n, y < ny, in place (qwen35/batch.py:365-372).
+    dst and src are contiguous device tensors of the same dtype (bf16 or float32); returns dst."""
+    if dst.dtype != src.dtype or dst.dtype not in (BF16, torch.float32):
+        raise TypeError(f"blit: bf16 or float32 tensors of one dtype expected, got {dst.dtype} and {src.dtype}")
+    dst, src = L.dev(dst, dst.dtype, "dst"), L.dev(src, src.dtype, "src")
+    n, d0, s0, ny, dstride, sstride = (int(x) for x in (n, d0, s0, ny, dstride, sstride))
+    if n < 0 or ny < 0 or min(d0, s0, dstride, sstride) < 0:
+        raise ValueError("blit: negative size, offset or stride")
+    if n and ny and (d0 + (ny - 1) * dstride + n > dst.numel() or s0 + (ny - 1) * sstride + n > src.numel()):
+        raise ValueError("blit: the copy leaves the source or the destination")
+    L.call("qt_blit", L.ptr(dst), L.ptr(src), dst.element_size(), n, d0, s0, ny, dstride, sstride, L.stream())
+    return dst
+
+
+def blit_batch(jobs):
+    """Several blits in one launch: jobs = [(dst, src, n, d0, s0, ny, dstride, sstride), ...] with the arguments of blit.
+    Every copy must be 16-byte granular (a ValueError says which one is not)."""
+    import ctypes
+    k = len(jobs)
+    if k == 0:
+        return
+    dsts, srcs, meta = (ctypes.c_void_p * k)(), (ctypes.c_void_p * k)(), (ctypes.c_long * (7 * k))()
+    for i, (dst, src, n, d0, s0, ny, dstride, sstride) in enumerate(jobs):
+        if dst.dtype != src.dtype or dst.dtype not in (BF16, torch.float32):
+            raise TypeError(f"blit_batch: job {i}: bf16 or float32 tensors of one dtype expected")
+        L.dev(dst, dst.dtype, "dst"), L.dev(src, src.dtype, "src")
+        n, d0, s0, ny, dstride, sstride = (int(x) for x in (n, d0, s0, ny, dstride, sstride))
+        if n < 0 or ny < 0 or min(d0, s0, dstride, sstride) < 0:
+            raise ValueError(f"blit_batch: job {i}: negative size, offset or stride")
+        if n and ny and (d0 + (ny - 1) * dstride + n > dst.numel() or s0 + (ny - 1) * sstride + n > src.numel()):
+            raise ValueError(f"blit_batch: job {i}: the copy leaves the source or the destination")
+        dsts[i], srcs[i] = dst.data_ptr(), src.data_ptr()
+        meta[7 * i:7 * i + 7] = [dst.element_size(), n, d0, s0, ny, dstride, sstride]
+    rc = L.lib().qt_blit_batch(dsts, srcs, meta, k, L.stream())
+    if rc == -2:
+        raise ValueError("blit_batch: every copy must be 16-byte granular (base pointers, sizes, offsets, strides)")
+    if rc:
+        raise RuntimeError(f"qt_blit_batch failed: {L.ERRORS.get(rc, rc)}")
+
+
 class Pools:
     """Slot-major state pools of the batched decode step (qwen35/batch.py:405-462)."""
 
@@ -119,15 +160,19 @@ class Pools:
 
     def load(self, slot: int, state: dict, pos: int):
         """Copy a prefilled single-sequence state (kv [1,2,max_len,256] pairs, conv [1,3,6144], ssm [1,16,128,128], valid after
-        `pos` tokens) into `slot`, in place (qwen35/batch.py:431-447)."""
+        `pos` tokens) into `slot`, in place, with the strided copy kernel (qwen35/batch.py:431-447)."""
         assert 0 <= slot < self.S and 0 < pos <= self.Lmax, (slot, pos)
         par = pos & 1
+        jobs = []
         for i, (c, s) in enumerate(zip(state["conv"], state["ssm"])):
-            self.conv[i][slot * 2 + par].copy_(c.reshape(3, CD))
-            self.ssm[i][slot].copy_(s.reshape(HV, DV, DK))
+            jobs.append((self.conv[i], c, CD * 3, (slot * 2 + par) * 3 * CD, 0, 1, 0, 0))
+            jobs.append((self.ssm[i], s, HV * DV * DK, slot * HV * DV * DK, 0, 1, 0, 0))
+        nkv, D = self.cfg.n_kv, self.cfg.head_dim
         for i, (K, V) in enumerate(state["kv"]):
-            self.K[i][slot, :, :pos].copy_(K[0, :, :pos])
-            self.V[i][slot, :, :pos].copy_(V[0, :, :pos])
+            smax = K.shape[2]
+            for pool, src in ((self.K[i], K), (self.V[i], V)):
+                jobs.append((pool, src, pos * D, slot * nkv * self.Lmax * D, 0, nkv, self.Lmax * D, smax * D))
+        blit_batch(jobs)                                         # one launch for the whole sequence (the reference issues 48 blits)
 
     def read(self, slot: int, pos: int, max_len: int | None = None):
         """The slot's state as a single-sequence state dict of fresh tensors (qwen35/batch.py:449-462)."""

@@ -50,3 +50,28 @@ class SpecPools:
     def entry_bytes(cfg: Cfg, M: int):
         nl = sum(cfg.is_linear(i) for i in range(cfg.layers))
         return nl * M * (HV * DV * DK * 4 + 2 * 3 * CD * 2)
+
+
+def to_spec(P, SP, slot: int, pos: int, ss: int):
+    """Plain -> speculative (the state moves of qwen35/serve.py:310-330): the sequence in `slot` of the plain pools `P`, with
+    `pos` tokens in its state, goes into snapshot 0 / conv buffer 0 of entry `ss` of the snapshot pools `SP`, for every
+    GatedDeltaNet layer.  The caller then runs the entry with par = 0, sel = 0."""
+    from .batch import blit_batch
+    M = SP.M
+    jobs = []
+    for i in range(len(SP.conv)):
+        jobs.append((SP.conv[i], P.conv[i], 3 * CD, (ss * 2 * M) * 3 * CD, (slot * 2 + (pos & 1)) * 3 * CD, 1, 0, 0))
+        jobs.append((SP.ssm[i], P.ssm[i], HV * DV * DK, ss * M * HV * DV * DK, slot * HV * DV * DK, 1, 0, 0))
+    blit_batch(jobs)
+
+
+def to_plain(P, SP, slot: int, pos: int, ss: int, par: int, n: int):
+    """Speculative -> plain (qwen35/serve.py:332-348): the live snapshot `n` of entry `ss` (conv buffer `par`, the one the
+    last round wrote) goes back into `slot` of the plain pools, whose state then holds `pos` tokens."""
+    from .batch import blit_batch
+    M = SP.M
+    jobs = []
+    for i in range(len(SP.conv)):
+        jobs.append((P.ssm[i], SP.ssm[i], HV * DV * DK, slot * HV * DV * DK, (ss * M + n) * HV * DV * DK, 1, 0, 0))
+        jobs.append((P.conv[i], SP.conv[i], 3 * CD, (slot * 2 + (pos & 1)) * 3 * CD, ((ss * 2 + par) * M + n) * 3 * CD, 1, 0, 0))
+    blit_batch(jobs)

@@ -31,6 +31,22 @@ constexpr int KT = 64;                 // keys per tile
 constexpr int KS_LD = AD + 8;          // LDS row strides (elements): 528 / 544 bytes spread the rows over the banks
 constexpr int VS_LD = AD + 16;
 
+// AP_MARK(i): per-tile phase time stamps for profiling builds (QT_ATTN_PREFILL_PROF defines ap_prof_buf[workgroup][wave][8],
+// accumulated shader-clock ticks per phase); compiles to nothing otherwise
+#ifdef QT_ATTN_PREFILL_PROF
+__device__ long long* ap_prof_buf;
+#define AP_MARK(i)                                                                                              \
+    do {                                                                                                        \
+        const long long now_ = clock64();                                                                       \
+        if ((threadIdx.x & 63) == 0) ap_prof_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6)) * 8 + (i)] += now_ - ap_last_; \
+        ap_last_ = now_;                                                                                        \
+    } while (0)
+#define AP_INIT() long long ap_last_ = clock64()
+#else
+#define AP_MARK(i)
+#define AP_INIT()
+#endif
+
 __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -99,8 +115,11 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
     // q+8, q+12; lane n of group g points at key 4g + n/4, columns 4 (n%4).. of the block and receives keys 4g..4g+3 of column n
     const bf16_t* va = v_s + (4 * g + (n >> 2)) * VS_LD + 4 * (n & 3);
 
+    AP_INIT();
     for (int t = 0; t < ntiles; t++) {
+        AP_MARK(0);
         __syncthreads();                                         // everyone is done reading the previous tile
+        AP_MARK(1);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             *reinterpret_cast<u32x4*>(k_s + (lr + 8 * i) * KS_LD + 8 * lc) = kr[i];
@@ -108,6 +127,7 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
         }
         if (t + 1 < ntiles) load_tile(t + 1);
         __syncthreads();
+        AP_MARK(2);
         if (t >= ntiles_w) continue;                             // wavefront-uniform: the upper row block may see one tile more
 
         // scores: each K fragment multiplies the Q^T of both heads (the compiler overlaps the next sub-tile's LDS reads with
@@ -127,6 +147,7 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
                     acc[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kb], bq[hh][kb], acc[hh][kt], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
+        AP_MARK(3);
         s16x8 P[NH][2];
         bool rescale = false;
 #pragma unroll
@@ -159,6 +180,7 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
             rescale |= corr != 1.0f;
         }
         wave_lds_sync();
+        AP_MARK(4);
         if (__any(rescale)) {                                    // wavefront-uniform: most tiles leave every row's max alone
 #pragma unroll
             for (int hh = 0; hh < NH; hh++) {
@@ -167,6 +189,7 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
                 for (int j = 0; j < 16; j++) O[hh][j] *= c4;
             }
         }
+        AP_MARK(5);
         // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs and serve
         // both heads
         auto v_frag = [&](int j, int q4) {
@@ -197,6 +220,7 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        AP_MARK(6);
         wave_lds_sync();                                         // c_s is rewritten by the next tile
     }
     // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n

@@ -1,0 +1,136 @@
+// In-place strided copies between state containers for gfx950: admission of a prefilled sequence into its slot, migration
+// between the plain pools and the snapshot pools.  Replaces the Metal kernel blit_{ctype} (qwen35/batch.py:349-372) behind
+// batch.blit, which Pools.load / read (batch.py:431-462) and the scheduler's _to_spec / _to_plain (qwen35/serve.py:310-348) use:
+//     dst.flat[d0 + y * dstride + i] = src.flat[s0 + y * sstride + i]      for i < n, y < ny
+// The copy is pure HBM traffic (n * ny elements read and written once).  Rows whose byte offsets and length are multiples
+// of 16 move as 16-byte vectors, a lane per vector, 4 vectors in flight per lane; anything else moves element by element.
+#include "qt_common.h"
+
+namespace {
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+// one workgroup copies up to 256 * 4 vectors of one row y; grid = (ceil(nvec / 1024), ny)
+__global__ __launch_bounds__(256) void blit_vec_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, long nvec,
+                                                       long d0, long s0, long dstride, long sstride) {
+    const long y = blockIdx.y;
+    u32x4* d = dst + d0 + y * dstride;
+    const u32x4* s = src + s0 + y * sstride;
+    const long i0 = (long)blockIdx.x * 1024 + threadIdx.x;
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (i0 + k * 256 < nvec) v[k] = __builtin_nontemporal_load(s + i0 + k * 256);
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (i0 + k * 256 < nvec) __builtin_nontemporal_store(v[k], d + i0 + k * 256);
+}
+
+// Many copies in one launch: a sequence's admission moves 48 separate pieces (18 layers of conv window and recurrent state,
+// 6 layers of K and V rows); launched one by one they cost a launch each (about 3 us), far more than their bytes.  The jobs
+// travel by value in the kernel arguments; all sizes, offsets and strides are in 16-byte vectors.
+struct BlitJob {
+    u32x4* dst;
+    const u32x4* src;
+    long nvec, ny, dstride, sstride;
+};
+constexpr int MAX_JOBS = 64;           // 64 x 48 bytes of kernel arguments
+struct BlitJobs {
+    BlitJob job[MAX_JOBS];
+};
+// grid = (x, number of jobs): the x workgroups of a job walk its (row, 1024-vector block) pairs with a grid stride
+__global__ __launch_bounds__(256) void blit_batch_kernel(const BlitJobs jobs) {
+    const BlitJob& j = jobs.job[blockIdx.y];
+    const long blocks_per_row = (j.nvec + 1023) / 1024, nblocks = blocks_per_row * j.ny;
+    for (long b = blockIdx.x; b < nblocks; b += gridDim.x) {
+        const long y = b / blocks_per_row, i0 = (b % blocks_per_row) * 1024 + threadIdx.x;
+        u32x4* d = j.dst + y * j.dstride;
+        const u32x4* s = j.src + y * j.sstride;
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            if (i0 + k * 256 < j.nvec) v[k] = __builtin_nontemporal_load(s + i0 + k * 256);
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            if (i0 + k * 256 < j.nvec) __builtin_nontemporal_store(v[k], d + i0 + k * 256);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void blit_elem_kernel(T* __restrict__ dst, const T* __restrict__ src, long n, long d0, long s0,
+                                                        long dstride, long sstride) {
+    const long y = blockIdx.y, i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[d0 + y * dstride + i] = src[s0 + y * sstride + i];
+}
+
+}  // namespace
+
+extern "C" {
+
+// elem_size 2 (bf16) or 4 (f32); n, d0, s0, dstride, sstride in elements.  The ranges written must not overlap the ranges read.
+int qt_blit(void* dst, const void* src, int elem_size, long n, long d0, long s0, long ny, long dstride, long sstride,
+            hipStream_t stream) {
+    if (!dst || !src) return QT_ERR_NULL;
+    if (elem_size != 2 && elem_size != 4) return QT_ERR_UNSUPPORTED;
+    if (n < 0 || ny < 0 || d0 < 0 || s0 < 0 || dstride < 0 || sstride < 0 || ny > 65535) return QT_ERR_DIM;
+    if (n == 0 || ny == 0) return QT_OK;
+    const long e = elem_size;
+    const bool vec = ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u) == 0 &&
+                     ((n * e) | (d0 * e) | (s0 * e) | (dstride * e) | (sstride * e)) % 16 == 0;
+    if (vec) {
+        const long per = 16 / e, nvec = n / per;
+        hipLaunchKernelGGL(blit_vec_kernel, dim3((unsigned)((nvec + 1023) / 1024), (unsigned)ny), dim3(256), 0, stream, (u32x4*)dst,
+                           (const u32x4*)src, nvec, d0 / per, s0 / per, dstride / per, sstride / per);
+    } else if (elem_size == 2) {
+        hipLaunchKernelGGL(blit_elem_kernel<uint16_t>, dim3((unsigned)((n + 255) / 256), (unsigned)ny), dim3(256), 0, stream,
+                           (uint16_t*)dst, (const uint16_t*)src, n, d0, s0, dstride, sstride);
+    } else {
+        hipLaunchKernelGGL(blit_elem_kernel<uint32_t>, dim3((unsigned)((n + 255) / 256), (unsigned)ny), dim3(256), 0, stream,
+                           (uint32_t*)dst, (const uint32_t*)src, n, d0, s0, dstride, sstride);
+    }
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+// `count` copies in one launch per 64 of them.  dst[k] / src[k] are device base pointers (host arrays), meta[7 k .. 7 k + 6] =
+// { elem_size, n, d0, s0, ny, dstride, sstride } as for qt_blit (host array).  Every job must be 16-byte granular (pointers,
+// n, offsets and strides as bytes); otherwise QT_ERR_ALIGN and nothing is launched.
+int qt_blit_batch(void* const* dst, const void* const* src, const long* meta, int count, hipStream_t stream) {
+    if (!dst || !src || !meta) return QT_ERR_NULL;
+    if (count < 0) return QT_ERR_DIM;
+    for (int k = 0; k < count; k++) {
+        const long* m = meta + 7 * k;
+        const long e = m[0];
+        if (!dst[k] || !src[k]) return QT_ERR_NULL;
+        if (e != 2 && e != 4) return QT_ERR_UNSUPPORTED;
+        for (int i = 1; i < 7; i++)
+            if (m[i] < 0) return QT_ERR_DIM;
+        if (((reinterpret_cast<uintptr_t>(dst[k]) | reinterpret_cast<uintptr_t>(src[k])) & 15u) ||
+            ((m[1] * e) | (m[2] * e) | (m[3] * e) | (m[5] * e) | (m[6] * e)) % 16)
+            return QT_ERR_ALIGN;
+    }
+    for (int k0 = 0; k0 < count; k0 += MAX_JOBS) {
+        BlitJobs jobs;
+        const int nj = count - k0 < MAX_JOBS ? count - k0 : MAX_JOBS;
+        long most = 1;
+        for (int k = 0; k < nj; k++) {
+            const long* m = meta + 7 * (k0 + k);
+            const long per = 16 / m[0];
+            BlitJob& j = jobs.job[k];
+            j.dst = (u32x4*)dst[k0 + k] + m[2] / per;
+            j.src = (const u32x4*)src[k0 + k] + m[3] / per;
+            j.nvec = m[1] / per;
+            j.ny = m[4];
+            j.dstride = m[5] / per;
+            j.sstride = m[6] / per;
+            const long nb = (j.nvec + 1023) / 1024 * j.ny;
+            if (nb > most) most = nb;
+        }
+        for (int k = nj; k < MAX_JOBS; k++) jobs.job[k] = BlitJob{nullptr, nullptr, 0, 0, 0, 0};
+        hipLaunchKernelGGL(blit_batch_kernel, dim3((unsigned)(most < 256 ? most : 256), (unsigned)nj), dim3(256), 0, stream, jobs);
+        QT_CHECK_LAUNCH();
+    }
+    return QT_OK;
+}
+
+}  // extern "C"

@@ -76,14 +76,10 @@ def test_pools_shapes_and_byte_accounting():
     assert qt.batch.Pools.slot_bytes(cfg, 64, double_conv=False) == 18 * (16 * 128 * 128 * 4 + 3 * 6144 * 2) + 6 * 2 * 2 * 64 * 256 * 2
     st = {"conv": [torch.randn(1, 3, 6144).bfloat16() for _ in range(18)], "ssm": [torch.randn(1, 16, 128, 128) for _ in range(18)],
           "kv": [(torch.randn(1, 2, 64, 256).bfloat16(), torch.randn(1, 2, 64, 256).bfloat16()) for _ in range(6)]}
-    P.load(2, st, 37)                                       # tests/batch.py:102-112: load -> read round trip, other slots stay zero
-    back = P.read(2, 37, 64)
-    assert all(torch.equal(a, b) for a, b in zip(back["ssm"], st["ssm"]))
-    assert all(torch.equal(a, b) for a, b in zip(back["conv"], st["conv"]))
-    assert all(torch.equal(a[0][:, :, :37], b[0][:, :, :37]) and torch.equal(a[1][:, :, :37], b[1][:, :, :37])
-               for a, b in zip(back["kv"], st["kv"]))
-    assert all(float(x[0].abs().max()) == 0 and float(x[1].abs().max()) == 0 for x in P.ssm + P.K)
-    assert torch.equal(P.conv[0][2 * 2 + 1], st["conv"][0][0]) and float(P.conv[0][2 * 2].abs().max()) == 0   # parity pos & 1
+    # the load -> read round trip (tests/batch.py:102-112) runs the copy kernel: tests/test_state_blit_gpu.py; without a GPU
+    # the operator must fail loudly rather than copy on the host
+    with pytest.raises(TypeError):
+        P.load(2, st, 37)
     with pytest.raises(AssertionError):
         P.load(3, st, 1)                                    # the trash slot cannot be loaded (batch.py:434)
     SP = qt.batch_spec.SpecPools(cfg, 2, 3, 4, 64, device="cpu")
