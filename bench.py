@@ -239,6 +239,20 @@ def bench_state_admission(torch, qt, dev, pos=2048, Lmax=4096, slots=8):
             "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
 
 
+def bench_attn_glue(torch, qt, dev, R=2048, seed=5):
+    """q / k RMSNorm + partial RoPE + split (qkv_prep) and the output gate over R rows (R = 2048: one prefill's rows)"""
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    qkv = torch.randn((R, 5120), generator=g).to(bf).to(dev)
+    qn, kn = torch.ones(256, dtype=bf, device=dev), torch.ones(256, dtype=bf, device=dev)
+    pos = torch.zeros(1, dtype=torch.int32, device=dev)
+    o = torch.randn((R, 8, 256), generator=g).to(bf).to(dev)
+    t1 = time_graph(torch, lambda: qt.attention.qkv_prep(qkv, qn, kn, pos, M=R), reps=60, inner=3)
+    t2 = time_graph(torch, lambda: qt.attention.out_gate(o, qkv), reps=60, inner=3)
+    b1, b2 = R * (3072 + 3072) * 2, R * (2048 * 3) * 2          # q, k, v columns in + out; o, gate in + out
+    return {"rows": R, "qkv_prep_us": t1 * 1e6, "qkv_prep_GBps": b1 / t1 / 1e9, "out_gate_us": t2 * 1e6, "out_gate_GBps": b2 / t2 / 1e9}
+
+
 def cpu_baseline(B, budget_s=12.0):
     """The C restatement of the decode step (float accumulation) timed on this host's cores: a reported baseline only."""
     import numpy as np
@@ -367,6 +381,7 @@ def main():
         extras["attn_verify_config4"] = bench_attn(torch, qt, dev, 16, 4, 1024, 8192, 1004)
         extras["attn_prefill_causal"] = [bench_attn_prefill(torch, qt, dev, S) for S in (2048, 8192)]
         extras["state_admission"] = bench_state_admission(torch, qt, dev)
+        extras["attn_glue"] = bench_attn_glue(torch, qt, dev)
 
     out = {
         "metric": "GDN decode steps/s @B=64 (% HBM peak); GDN prefill tok/s @2048 (% MFMA)",

@@ -120,6 +120,15 @@ long qt_gqa_prefill_workspace_bytes(int L);
 int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out, void* workspace, long workspace_bytes, int S,
                           int L, int q_pos0, long q_head_stride, long kv_head_stride, qt_stream_t stream);
 
+/* The elementwise steps either side of the attention kernels in a full-attention layer (qwen35/batch.py:505-513,
+ * qwen35/model.py:154-169).  qkv [R,5120] bf16 = [(q_h[256] | gate_h[256]) for 8 heads | k[2][256] | v[2][256]].
+ * qt_attn_qkv_prep: q [R,8,256], k [R,2,256] = rope(rms_norm(., q_norm / k_norm [256] bf16, eps), position), v [R,2,256] = v;
+ * rotary embedding of the first 64 features, half-split pairing, theta 1e7; row r = b*M + j sits at position pos[b] + j.
+ * qt_attn_out_gate: out [R,2048] = o [R,8,256] * sigmoid(gate). */
+int qt_attn_qkv_prep(const void* qkv, const void* q_norm, const void* k_norm, const int32_t* pos, void* q, void* k, void* v, long R,
+                     int M, float eps, qt_stream_t stream);
+int qt_attn_out_gate(const void* o, const void* qkv, void* out, long R, qt_stream_t stream);
+
 /* batch.blit (qwen35/batch.py:365-372), the in-place strided copy behind Pools.load / read (batch.py:431-462) and the
  * scheduler's plain <-> speculative state moves (qwen35/serve.py:310-348):
  *     dst.flat[d0 + y*dstride + i] = src.flat[s0 + y*sstride + i]   for i < n, y < ny   (offsets and strides in elements)

@@ -385,3 +385,54 @@ def blit(dst, src, n, d0, s0, ny=1, dstride=0, sstride=0):
     for y in range(ny):
         d[d0 + y * dstride:d0 + y * dstride + n] = s[s0 + y * sstride:s0 + y * sstride + n]
     return dst
+
+
+# ------------------------------------------------------------------------------------------------
+# attention glue (batch.py:505-513, model.py:154-169): q / k RMSNorm, partial rotary embedding, output gate
+# ------------------------------------------------------------------------------------------------
+ROPE_DIM, ROPE_THETA, QKV_W = 64, 1e7, 8 * 512 + 2 * 2 * 256
+
+
+def rope_freqs():
+    """freq_i = float32(theta^(-2 i / dims)), i < dims / 2 (mx.fast.rope(..., traditional=False, base=1e7), model.py:163)"""
+    return np.array([np.float32(ROPE_THETA ** (-2.0 * i / ROPE_DIM)) for i in range(ROPE_DIM // 2)], np.float32)
+
+
+def rms_norm_rows(x, w, eps=1e-6):
+    """mx.fast.rms_norm on rows of 256 (model.py:160-161): exact sum of squares, x * inv rounded to bf16, times the bf16 weight,
+    rounded to bf16."""
+    x = np.asarray(x, np.float32)
+    ss = (x.astype(np.float64) ** 2).sum(-1, keepdims=True).astype(np.float32)
+    inv = rsqrt32((ss / F32(x.shape[-1]) + F32(eps)).astype(np.float32))
+    return BF((np.asarray(w, np.float32) * BF((x * inv).astype(np.float32))).astype(np.float32))
+
+
+def rope_rows(x, pos):
+    """Half-split rotary embedding of the first 64 of 256 features (mx.fast.rope, traditional=False): x [..., 256], pos
+    broadcastable to x.shape[:-1].  Products and sums are rounded to float32 one by one, the result to bf16."""
+    x = np.asarray(x, np.float32).copy()
+    th = (np.asarray(pos, np.float32)[..., None] * rope_freqs()).astype(np.float32)
+    c, s = np.cos(th.astype(np.float64)).astype(np.float32), np.sin(th.astype(np.float64)).astype(np.float32)
+    x1, x2 = x[..., :32].copy(), x[..., 32:64].copy()
+    x[..., :32] = BF(((x1 * c).astype(np.float32) - (x2 * s).astype(np.float32)).astype(np.float32))
+    x[..., 32:64] = BF(((x1 * s).astype(np.float32) + (x2 * c).astype(np.float32)).astype(np.float32))
+    return x
+
+
+def attn_qkv_prep(qkv, q_norm, k_norm, pos, M=1, eps=1e-6):
+    """qkv [R,5120] = [(q_h | gate_h) x 8 | k x 2 | v x 2] -> q [R,8,256], k [R,2,256] (normed + roped), v [R,2,256]
+    (batch.py:505-512); row r = b*M + j sits at position pos[b] + j."""
+    qkv = np.asarray(qkv, np.float32)
+    R = qkv.shape[0]
+    p = (np.repeat(np.asarray(pos), M) + np.tile(np.arange(M), R // M)).astype(np.float32)
+    q = qkv[:, :4096].reshape(R, 8, 512)[:, :, :256]
+    k = qkv[:, 4096:4608].reshape(R, 2, 256)
+    v = qkv[:, 4608:].reshape(R, 2, 256).copy()
+    return rope_rows(rms_norm_rows(q, q_norm, eps), p[:, None]), rope_rows(rms_norm_rows(k, k_norm, eps), p[:, None]), v
+
+
+def attn_out_gate(o, qkv):
+    """o [R,8,256] * sigmoid(gate) with gate_h = qkv[:, h*512+256 : (h+1)*512] (batch.py:513) -> [R,2048]"""
+    o = np.asarray(o, np.float32).reshape(-1, 8, 256)
+    gate = np.asarray(qkv, np.float32)[:, :4096].reshape(-1, 8, 512)[:, :, 256:]
+    return BF((o * sigmoid_bf16(gate)).astype(np.float32)).reshape(-1, 2048)

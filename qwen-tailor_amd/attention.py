@@ -35,3 +35,33 @@ def scaled_dot_product_attention(q, k, v, *, scale: float, mask="causal"):
     L.call("qt_gqa_prefill_causal", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), None, 0, S, Lk, Lk - S, S * 256, k.stride(1),
            L.stream())
     return out
+
+
+QKV_W = 8 * 512 + 2 * 2 * 256
+
+
+def qkv_prep(qkv, q_norm, k_norm, pos, M=1, eps=1e-6):
+    """The steps between the qkv projection and the attention kernel of a full-attention layer (qwen35/batch.py:505-512,
+    qwen35/model.py:154-164): split the 5120-wide rows into q / gate / k / v, RMS-normalise q and k per head (weights [256]
+    bf16), rotate their first 64 features to the row's position.  qkv [R,5120] bf16, pos int32 [R / M] (row b*M + j sits at
+    pos[b] + j).  Returns q [R,8,256], k [R,2,256], v [R,2,256] bf16; the gate stays in qkv (out_gate reads it there)."""
+    qkv = L.dev(qkv, BF16, "qkv", (None, QKV_W))
+    R = qkv.shape[0]
+    if M < 1 or R % M:
+        raise ValueError(f"qkv_prep: M = {M} must divide the number of rows ({R})")
+    pos = L.i32(pos, "pos", R // M)
+    qn, kn = L.dev(q_norm, BF16, "q_norm", (256,)), L.dev(k_norm, BF16, "k_norm", (256,))
+    q = torch.empty((R, 8, 256), dtype=BF16, device=qkv.device)
+    k, v = (torch.empty((R, 2, 256), dtype=BF16, device=qkv.device) for _ in range(2))
+    L.call("qt_attn_qkv_prep", L.ptr(qkv), L.ptr(qn), L.ptr(kn), L.ptr(pos), L.ptr(q), L.ptr(k), L.ptr(v), R, M, float(eps), L.stream())
+    return q, k, v
+
+
+def out_gate(o, qkv):
+    """o * sigmoid(gate) (qwen35/batch.py:513): o [R,8,256] bf16, qkv [R,5120] bf16 -> [R,2048] bf16"""
+    qkv = L.dev(qkv, BF16, "qkv", (None, QKV_W))
+    R = qkv.shape[0]
+    o = L.dev(o, BF16, "o", (R, 8, 256))
+    out = torch.empty((R, 2048), dtype=BF16, device=qkv.device)
+    L.call("qt_attn_out_gate", L.ptr(o), L.ptr(qkv), L.ptr(out), R, L.stream())
+    return out

@@ -170,3 +170,41 @@ def test_prefill_causal_8192_two_heads_per_wavefront(qt, dev):
         ref = O.sdpa_causal(qn[:, r:r + 1], Kn[:, :r + 1], Vn[:, :r + 1])            # the row at position r sees keys 0..r
         check_attn(f"S=8192 row {r}", o[:, r:r + 1], ref)
     check_equal("row 0 == v[0]", o[:, 0], np.repeat(Vn[:, 0], 4, axis=0))
+
+
+# ------------------------------------------------------------------------------------- glue either side of the attention kernels
+@pytest.mark.parametrize("R,M", [(1, 1), (5, 1), (8, 4), (64, 1)])
+def test_qkv_prep_and_out_gate_bit_exact(qt, dev, R, M):
+    """q / k RMSNorm + partial RoPE + v split, and o * sigmoid(gate) (batch.py:505-513): every bf16 value equals the oracle's"""
+    rng = np.random.default_rng(100 * R + M)
+    qkv = bf(rng.standard_normal((R, O.QKV_W)) * 2)
+    qn, kn = bf(1 + 0.2 * rng.standard_normal(256)), bf(1 + 0.2 * rng.standard_normal(256))
+    pos = rng.integers(0, 32768, R // M).astype(np.int32)
+    pos[0] = 0
+    dq = to_dev(qkv, dev, BF16)
+    q, k, v = qt.attention.qkv_prep(dq, to_dev(qn, dev, BF16), to_dev(kn, dev, BF16), to_dev(pos, dev), M)
+    oq, ok, ov = O.attn_qkv_prep(qkv, qn, kn, pos, M)
+    check_equal("q", to_np(q), oq)
+    check_equal("k", to_np(k), ok)
+    check_equal("v", to_np(v), ov)
+    o = bf(rng.standard_normal((R, 8, 256)))
+    check_equal("gated output", to_np(qt.attention.out_gate(to_dev(o, dev, BF16), dq)), O.attn_out_gate(o, qkv))
+
+
+def test_attention_layer_core_decode_rows(qt, dev):
+    """qkv_prep -> attn_b -> out_gate on 5 decode rows against the same chain of oracle functions (a full-attention layer between
+    its qkv and o_proj projections, batch.py:504-514)"""
+    rng = np.random.default_rng(77)
+    B, Lmax = 5, 256
+    slots, pos = np.array([3, 0, 4, 1, 2], np.int32), np.array([0, 1, 100, 255 - 1, 17], np.int32)
+    qkv = bf(rng.standard_normal((B, O.QKV_W)))
+    qn, kn = bf(1 + 0.1 * rng.standard_normal(256)), bf(1 + 0.1 * rng.standard_normal(256))
+    Kp, Vp = bf(rng.standard_normal((6, 2, Lmax, 256))), bf(rng.standard_normal((6, 2, Lmax, 256)))
+    dq, dK, dV = to_dev(qkv, dev, BF16), to_dev(Kp, dev, BF16), to_dev(Vp, dev, BF16)
+    q, k, v = qt.attention.qkv_prep(dq, to_dev(qn, dev, BF16), to_dev(kn, dev, BF16), to_dev(pos, dev))
+    o = qt.batch.attn_b(q, k, v, dK, dV, to_dev(slots, dev), to_dev(pos, dev))
+    out = qt.attention.out_gate(o, dq)
+    oq, ok, ov = O.attn_qkv_prep(qkv, qn, kn, pos)
+    oo = O.attn_b(oq, ok, ov, Kp, Vp, slots, pos, 1)
+    check_rel("layer core", to_np(out), O.attn_out_gate(oo, qkv), 1e-2, rel_max)
+    check_equal("appended K", to_np(dK), Kp)                                   # the oracle appended the same rows in place

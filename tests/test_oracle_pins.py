@@ -457,3 +457,76 @@ def test_sdpa_causal_vs_torch():
         torch.from_numpy(q.astype(np.float64))[None], torch.from_numpy(K.astype(np.float64)).repeat_interleave(4, 0)[None],
         torch.from_numpy(V.astype(np.float64)).repeat_interleave(4, 0)[None], is_causal=True, scale=256 ** -0.5)[0].numpy()
     assert np.all(np.abs(o - r) <= 0.51 * ulp_bf16(r) + 1e-9)
+
+
+# ------------------------------------------------------------------------------------------------
+# attention glue and the state copy: library routines, closed forms, invariants
+# ------------------------------------------------------------------------------------------------
+def test_rms_norm_rows_vs_torch():
+    """the q / k RMSNorm reduces to torch.nn.functional.rms_norm in float64, up to its two bf16 roundings"""
+    rng = np.random.default_rng(0)
+    x = bf(rng.standard_normal((5, 8, 256)) * 3)
+    w = bf(1 + 0.2 * rng.standard_normal(256))
+    got = O.rms_norm_rows(x, w, 1e-6)
+    ref = torch.nn.functional.rms_norm(torch.from_numpy(x).double(), (256,), torch.from_numpy(w).double(), 1e-6).numpy()
+    assert np.all(np.abs(got - ref) <= 2.0 * ulp_bf16(ref) + 1e-30)             # two bf16 roundings (of x * inv, then of w * that)
+    one = O.rms_norm_rows(np.full((1, 256), 2.0, np.float32), np.ones(256, np.float32), 0.0)
+    assert np.array_equal(one, np.ones((1, 256), np.float32))                   # constant row: x / |x|
+
+
+def test_rope_rows_closed_forms():
+    rng = np.random.default_rng(1)
+    x = bf(rng.standard_normal((7, 2, 256)))
+    f = O.rope_freqs()
+    assert f[0] == 1.0 and abs(float(f[16]) - 1e7 ** -0.5) < 1e-9 and np.all(np.diff(f) < 0)      # theta^(-2i/64)
+    assert np.array_equal(O.rope_rows(x, np.zeros((7, 1))), x)                                    # position 0: identity
+    y = O.rope_rows(x, np.arange(7, dtype=np.float32)[:, None] * 100 + 3)
+    assert np.array_equal(y[..., 64:], x[..., 64:])                                               # features >= 64 pass through
+    n0 = x[..., :32] ** 2 + x[..., 32:64] ** 2                                                    # a rotation keeps the pair norms
+    n1 = y[..., :32] ** 2 + y[..., 32:64] ** 2
+    assert np.abs(n1 - n0).max() <= 0.02 * n0.max()
+    # pairing is (i, i + 32): a unit vector on feature i at position p lands on (cos, sin)(p * f_i) of features i, i + 32
+    e = np.zeros((1, 256), np.float32)
+    e[0, 5] = 1.0
+    r = O.rope_rows(e, np.array([[11.0]]))[0]
+    assert abs(r[5] - np.cos(11 * float(f[5]))) < 4e-3 and abs(r[37] - np.sin(11 * float(f[5]))) < 4e-3 and np.count_nonzero(r) == 2
+    # relative-position property: <rope(q, p), rope(k, p')> depends on p - p' only (float64 check of the formula, no rounding)
+    q, k = rng.standard_normal(256), rng.standard_normal(256)
+    def rot(v, p):
+        v = v.copy()
+        c, s = np.cos(p * f.astype(np.float64)), np.sin(p * f.astype(np.float64))
+        v[:32], v[32:64] = v[:32] * c - v[32:64] * s, v[:32] * s + v[32:64] * c
+        return v
+    assert abs(rot(q, 17.0) @ rot(k, 5.0) - rot(q, 112.0) @ rot(k, 100.0)) < 1e-9
+
+
+def test_attn_qkv_prep_and_gate_layout():
+    rng = np.random.default_rng(2)
+    R, M = 6, 2
+    qkv = bf(rng.standard_normal((R, O.QKV_W)))
+    qn, kn = bf(1 + 0.1 * rng.standard_normal(256)), bf(1 + 0.1 * rng.standard_normal(256))
+    pos = np.array([4, 0, 1000], np.int32)
+    q, k, v = O.attn_qkv_prep(qkv, qn, kn, pos, M)
+    assert q.shape == (R, 8, 256) and k.shape == (R, 2, 256) and v.shape == (R, 2, 256)
+    assert np.array_equal(v, qkv[:, 4608:].reshape(R, 2, 256))
+    # row 2 = sequence 1, token 0, position 0: no rotation, only the norm; head 3 reads columns 3*512 .. 3*512+255
+    assert np.array_equal(q[2, 3], O.rms_norm_rows(qkv[2, 3 * 512:3 * 512 + 256][None], qn)[0])
+    assert np.array_equal(k[2, 1], O.rms_norm_rows(qkv[2, 4096 + 256:4096 + 512][None], kn)[0])
+    # row 1 = sequence 0, token 1 sits at position 5
+    assert np.array_equal(q[1, 0], O.rope_rows(O.rms_norm_rows(qkv[1, :256][None], qn), np.array([[5.0]]))[0])
+    o = bf(rng.standard_normal((R, 8, 256)))
+    g = O.attn_out_gate(o, qkv)
+    ref = o.astype(np.float64) / (1 + np.exp(-qkv[:, :4096].reshape(R, 8, 512)[:, :, 256:].astype(np.float64)))
+    assert np.abs(g.reshape(R, 8, 256) - ref).max() <= 0.02 * np.abs(ref).max()
+
+
+def test_blit_is_a_strided_copy():
+    rng = np.random.default_rng(3)
+    dst, src = rng.standard_normal(400).astype(np.float32), rng.standard_normal(300).astype(np.float32)
+    d0 = dst.copy()
+    O.blit(dst, src, 10, 7, 3, ny=3, dstride=100, sstride=50)
+    want = d0.copy()
+    for y in range(3):
+        for i in range(10):
+            want[7 + y * 100 + i] = src[3 + y * 50 + i]
+    assert np.array_equal(dst, want)
