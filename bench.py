@@ -132,7 +132,7 @@ GDN_FLOP_PER_TOKEN = 2621440.0        # 16 heads x (4 C^2 dk + 4 C^2 dv + 6 C dk
 
 
 def bench_prefill(torch, qt, dev, T, seed=1002):
-    """BASELINE config 2: conv + chunked GDN (chunk 64) + gated RMSNorm over T tokens from a nonzero state"""
+    """benchmark config 2: conv + chunked GDN (chunk 64) + gated RMSNorm over T tokens from a nonzero state"""
     g = torch.Generator().manual_seed(seed)
     bf = torch.bfloat16
     proj = torch.randn((T, PW), generator=g).to(bf).to(dev)
@@ -154,7 +154,7 @@ def bench_prefill(torch, qt, dev, T, seed=1002):
 
 
 def bench_verify_gdn(torch, qt, dev, B=16, M=4, seed=1004):
-    """BASELINE config 4, GDN half: B sequences x M draft tokens, a state snapshot after every token"""
+    """benchmark config 4, GDN half: B sequences x M draft tokens, a state snapshot after every token"""
     g = torch.Generator().manual_seed(seed)
     bf = torch.bfloat16
     pools = [((torch.randn((B + 1, M, HV, DV, DK), generator=g) * 0.02).to(dev), torch.randn(((B + 1) * 2, M, 3, CD), generator=g).to(bf).to(dev))
@@ -178,7 +178,7 @@ def bench_verify_gdn(torch, qt, dev, B=16, M=4, seed=1004):
 
 
 def bench_attn(torch, qt, dev, B, M, lo, hi, seed):
-    """BASELINE configs 3 / 4 (attention half): ragged KV lengths uniform in [lo, hi], M query rows per sequence"""
+    """benchmark configs 3 / 4 (attention half): ragged KV lengths uniform in [lo, hi], M query rows per sequence"""
     import numpy as np
     rng = np.random.default_rng(seed)
     Lmax = hi + 8

@@ -1,5 +1,5 @@
 """GPU parity of the chunked (C = 64) GatedDeltaNet prefill against the sequential CPU oracle.
-Tolerance (BASELINE north star): final state and outputs within 2e-3 relative of the sequential reference."""
+Tolerance (the stated target): final state and outputs within 2e-3 relative of the sequential reference."""
 import numpy as np
 import pytest
 import torch
@@ -19,7 +19,7 @@ def qt():
 
 
 def gdn_inputs(seed, T, state_scale=0.02):
-    """q, k (normalized), v, a, b as BASELINE config 0 draws them, plus layer parameters and an initial state"""
+    """q, k (normalized), v, a, b as benchmark config 0 draws them, plus layer parameters and an initial state"""
     gen = torch.Generator().manual_seed(seed)
     cw, A_log, dtb, gw = layer_params(seed)
     q, k = O.normalize_qk(rand_bf(gen, (T, 16, 128)), rand_bf(gen, (T, 16, 128)))
@@ -106,7 +106,7 @@ def test_chunked_prefill_vs_sequential_oracle(qt, dev, T):
 
 @pytest.mark.parametrize("T", [512, 2048])
 def test_config2_chunked_prefill(qt, dev, T):
-    """BASELINE config 2: B=1, chunk 64, nonzero initial state ~N(0,0.02) (prefix-cache resume), conv first, gated norm last"""
+    """benchmark config 2: B=1, chunk 64, nonzero initial state ~N(0,0.02) (prefix-cache resume), conv first, gated norm last"""
     proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(1002, T)
     dproj = to_dev(proj, dev, BF16)
     q, k, v, ops, U, gC = qt.gdn_nax.prep_a(dproj, to_dev(cs, dev, BF16), to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev))

@@ -1,6 +1,6 @@
 """GPU parity of the fused GatedDeltaNet decode / verify step and its stand-alone pieces against the CPU oracle.
 
-Tolerances (BASELINE north star): fp32 state within 1e-4 relative per decode step; everything the elementwise prologue
+Tolerances (the stated target): fp32 state within 1e-4 relative per decode step; everything the elementwise prologue
 produces (conv windows, q, k, v, gates, gated norm) is bit-exact by construction of the arithmetic contract; bf16 outputs
 of float32 dot products within 1 bf16 ulp."""
 import numpy as np
@@ -139,7 +139,7 @@ def test_gated_delta_update_gqa_heads_and_errors(qt, dev):
 
 
 def test_config0_token_by_token(qt, dev):
-    """BASELINE config 0: one layer, B=1, T=256 run token by token from a zero state; per-step state error <= 1e-4."""
+    """benchmark config 0: one layer, B=1, T=256 run token by token from a zero state; per-step state error <= 1e-4."""
     gen = torch.Generator().manual_seed(1000)
     T = 256
     A_log = (torch.rand(16, generator=gen) * 2.7).numpy()
@@ -259,7 +259,7 @@ def test_deltanet_b_layout_of_reference_test(qt, dev):
 
 @pytest.mark.parametrize("B", [1, 16, 64])
 def test_deltanet_b_config1_steps(qt, dev, B):
-    """BASELINE config 1 (B in {1,16,64}): consecutive steps with advancing positions; state ~ N(0,0.02).  The C oracle steps
+    """benchmark config 1 (B in {1,16,64}): consecutive steps with advancing positions; state ~ N(0,0.02).  The C oracle steps
     alongside from its own state (free running) and must stay within 1e-4 relative at every step."""
     gen = torch.Generator().manual_seed(1001)
     cw, A_log, dtb, gw = layer_params(9)

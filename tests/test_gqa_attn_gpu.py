@@ -1,5 +1,5 @@
 """GPU parity of the ragged GQA hd256 decode / verify attention against the CPU oracle (float64 softmax attention).
-Tolerance (BASELINE north star): bf16 attention outputs within 1e-2 relative."""
+Tolerance (the stated target): bf16 attention outputs within 1e-2 relative."""
 import numpy as np
 import pytest
 import torch
@@ -88,7 +88,7 @@ def test_attn_b_out_of_range_rows_are_skipped(qt, dev):
 
 
 def test_attn_b_config3_ragged_long(qt, dev):
-    """BASELINE config 3: B=16, one query each, ragged KV lengths uniform in [512, 32768] (seed 1003)"""
+    """benchmark config 3: B=16, one query each, ragged KV lengths uniform in [512, 32768] (seed 1003)"""
     rng = np.random.default_rng(1003)
     B, Lmax = 16, 32768
     pos = rng.integers(512, 32768, B).astype(np.int32)                          # keys already in the pool (+1 new)
@@ -114,7 +114,7 @@ def test_attn_b_config3_ragged_long(qt, dev):
 
 
 def test_attn_b_config4_verify_mix(qt, dev):
-    """BASELINE config 4 (attention half): B=16 x M=4, KV lengths uniform in [1024, 8192], 4-token causal tail"""
+    """benchmark config 4 (attention half): B=16 x M=4, KV lengths uniform in [1024, 8192], 4-token causal tail"""
     rng = np.random.default_rng(1004)
     B, M, Lmax = 16, 4, 8192 + 8
     pos = rng.integers(1024, 8192, B).astype(np.int32)
@@ -154,7 +154,7 @@ def test_prefill_causal_2048(qt, dev):
 
 
 def test_prefill_causal_8192_two_heads_per_wavefront(qt, dev):
-    """S = 8192 (BASELINE's long prefill; the launch uses 32-row workgroups with two heads per wavefront): a sample of query
+    """S = 8192 (the long-prefill benchmark size; the launch uses 32-row workgroups with two heads per wavefront): a sample of query
     rows, including block borders and the first / last rows, against the float64 oracle evaluated for those rows only"""
     rng = np.random.default_rng(8192)
     S = 8192

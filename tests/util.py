@@ -1,4 +1,4 @@
-"""Shared helpers of the parity tests: seeded inputs in the shapes of the BASELINE configs, bf16 <-> numpy conversions
+"""Shared helpers of the parity tests: seeded inputs in the shapes of the benchmark configs, bf16 <-> numpy conversions
 and the error measures the tolerances are written in."""
 import numpy as np
 import torch
