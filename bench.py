@@ -360,6 +360,26 @@ def main():
 
     extras = {}
     if not args.no_extras:
+        # the serving step of one layer: decode step + gated RMSNorm, as two launches and as the fused launch
+        gw = torch.ones(DV, device=dev)
+        it = [0]
+
+        def two():
+            l = it[0] % N_LAYERS
+            it[0] += 1
+            y = qt.batch.deltanet_b(st["proj"][l & 3], st["conv"][l], st["cw"][l], st["A_log"][l], st["dtb"][l], st["ssm"][l], st["slots"],
+                                    st["pos"][0])
+            qt.batch.gnorm_rows(y, st["proj"][l & 3], gw)
+
+        def one():
+            l = it[0] % N_LAYERS
+            it[0] += 1
+            qt.batch.deltanet_b_gnorm(st["proj"][l & 3], st["conv"][l], st["cw"][l], st["A_log"][l], st["dtb"][l], st["ssm"][l], st["slots"],
+                                      st["pos"][0], gw)
+        t2 = time_graph(torch, two, reps=N_LAYERS * 20, inner=N_LAYERS)
+        t1 = time_graph(torch, one, reps=N_LAYERS * 20, inner=N_LAYERS)
+        extras["decode_plus_gated_norm"] = {"two_launches_us": t2 * 1e6, "fused_us": t1 * 1e6,
+                                            "fused_GBps": (decode_bytes(B) + B * 2048 * 2) / t1 / 1e9}
         w1, d1 = time_decode(torch, qt, st, B, 1, args.steps, args.warmup, use_graph=not args.no_graph)
         extras["single_pool_cache_resident"] = {"steps_per_s": args.steps / w1, "GBps": decode_bytes(B) / (d1 / args.steps) / 1e9}
         if not args.no_graph:

@@ -33,6 +33,13 @@ int qt_gdn_decode_step(const void* proj, void* conv_pool, const void* conv_w, co
                        float* ssm_pool, const int32_t* slots, const int32_t* pos, void* y, int B, int n_slots,
                        int rows_per_wg, qt_stream_t stream);
 
+/* qt_gdn_decode_step followed by qt_gated_rmsnorm (batch.deltanet_b + batch.gnorm_rows, qwen35/batch.py:128-135, 338-343) in one
+ * launch: out [B,2048] bf16 = gated RMSNorm of the step's outputs with z = proj[:,6144:8192] and weight gw [128] f32 (same bits
+ * as the two launches); the un-normalised outputs are not stored. */
+int qt_gdn_decode_step_gnorm(const void* proj, void* conv_pool, const void* conv_w, const float* A_log, const float* dt_bias,
+                             float* ssm_pool, const int32_t* slots, const int32_t* pos, const float* gw, float eps, void* out, int B,
+                             int n_slots, qt_stream_t stream);
+
 /* batch_spec.deltanet_bm (qwen35/batch_spec.py:142-150): M chained tokens for each of B sequences, a state snapshot
  * after every token.  proj [B*M,8224]; conv_pool [n_entries*2,M,3,6144]; ssm_pool [n_entries,M,16,128,128];
  * sslots, sels, pars [B] int32 (pool entry, snapshot to start from, conv buffer to read); y [B*M,2048].  1 <= M <= 16. */

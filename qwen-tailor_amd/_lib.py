@@ -18,6 +18,7 @@ ERRORS = {-1: "bad dimension", -2: "misaligned pointer", -3: "null pointer", -4:
 
 _SIGS = {
     "qt_gdn_decode_step": [_vp] * 9 + [_i, _i, _i, _vp],
+    "qt_gdn_decode_step_gnorm": [_vp] * 9 + [_f, _vp, _i, _i, _vp],
     "qt_gdn_verify_step": [_vp] * 10 + [_i, _i, _i, _i, _vp],
     "qt_gdn_deltanet": [_vp] * 10 + [_i, _i, _i, _vp],
     "qt_gdn_gates": [_vp, _vp, _l, _l, _vp, _vp, _vp, _vp, _vp, _l, _i, _vp],

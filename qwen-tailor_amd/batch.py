@@ -47,6 +47,24 @@ def _workspace(dev, nbytes):
     return buf
 
 
+def deltanet_b_gnorm(proj, conv_pool, conv_w, A_log, dt_bias, ssm_pool, slots, pos, gw, eps=1e-6):
+    """deltanet_b followed by gnorm_rows (qwen35/batch.py:128-135, 338-343; the two calls of the reference's decode step,
+    batch.py:497-499) in one launch.  Returns the gated-norm output [B, 2048] bf16 (the same bits as the two calls); pools are
+    updated in place as by deltanet_b."""
+    proj = L.dev(proj, BF16, "proj", (None, PW))
+    B = proj.shape[0]
+    ssm_pool = L.dev(ssm_pool, torch.float32, "ssm_pool", (None, HV, DV, DK))
+    n_slots = ssm_pool.shape[0]
+    conv_pool = L.dev(conv_pool, BF16, "conv_pool", (n_slots * 2, 3, CD))
+    slots, pos = L.i32(slots, "slots", B), L.i32(pos, "pos", B)
+    w = flat_conv_w(conv_w)
+    A, dtb, gw = L.f32(A_log, "A_log", (HV,)), L.f32(dt_bias, "dt_bias", (HV,)), L.f32(gw, "gw", (DV,))
+    out = torch.empty((B, HV * DV), dtype=BF16, device=proj.device)
+    L.call("qt_gdn_decode_step_gnorm", L.ptr(proj), L.ptr(conv_pool), L.ptr(w), L.ptr(A), L.ptr(dtb), L.ptr(ssm_pool), L.ptr(slots),
+           L.ptr(pos), L.ptr(gw), float(eps), L.ptr(out), B, n_slots, L.stream())
+    return out
+
+
 def split_size(Lmax: int, B: int = 16) -> int:
     """Smallest number of pool keys a split-K workgroup takes.  The kernel spreads the batch's key tiles evenly over one
     workgroup per CU whatever the mix of lengths; this lower bound only matters for small batches of short sequences."""

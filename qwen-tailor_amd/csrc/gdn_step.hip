@@ -46,13 +46,17 @@ __device__ __forceinline__ void store_window(bf16_t* __restrict__ cs_out, const 
 
 // M chained tokens of one (sequence, head, row split).  Snapshot j of the state goes to st_out + j*st_stride and of the
 // conv window to cs_out + j*cs_stride (strides 0 = update in place).
-template <int RS, int HPW = 1>
+// NORM (whole heads only, RS = 8): y receives the gated RMSNorm of the head's 128 outputs, BF(z sigmoid(z) gw (y inv)) with
+// z = proj[6144 + h*128 + row] (qwen35/batch.py:321-331), instead of the outputs themselves: same bits as the stand-alone
+// norm kernel applied to the stored outputs.
+template <int RS, int HPW = 1, bool NORM = false>
 __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs_in,
                                            bf16_t* __restrict__ cs_out, size_t cs_stride,
                                            const bf16_t* __restrict__ cw, const float* __restrict__ A_log,
                                            const float* __restrict__ dt_bias, const float* st_in,
                                            float* st_out, size_t st_stride, bf16_t* __restrict__ y, int M, int h,
-                                           int split) {
+                                           int split, const float* __restrict__ gw = nullptr, float eps = 0.f) {
+    static_assert(!NORM || RS == 8, "the fused norm needs the whole head in one group of 256 threads");
     constexpr int ROWS = RS * 16;
     __shared__ double red_a[HPW][4];
     __shared__ __align__(16) float qk_a[HPW][2][DK];
@@ -82,6 +86,13 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
     const int gl = lane < 3 ? lane : 0;
     float gx = bf2f(proj[CD + KD + HV * (gl == 1 ? 1 : 0) + h]);       // lane 1: a;  lanes 0, 2: b
     const float gA = A_log[h], gdt = dt_bias[h];
+    // fused norm: lane c < 8 of a 16-lane group finishes the group's row i = c (row c*16 + w*4 + grp of the head)
+    const int nrow = (c & 7) * 16 + w * 4 + grp;
+    float nz = 0.f, ngw = 0.f;
+    if (NORM) {
+        nz = bf2f(proj[CD + h * DV + nrow]);
+        ngw = gw[nrow];
+    }
     __builtin_amdgcn_sched_barrier(0);           // keep the small loads ahead of the state loads in issue order
 
     f4 s[RS][2];
@@ -146,6 +157,7 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
 
         f4* so4 = reinterpret_cast<f4*>(st_out + (size_t)j * st_stride + ((size_t)h * DV + row0) * DK);
         bf16_t* yo = y + (size_t)j * KD + h * DV + row0;
+        float yb[RS];
 #pragma unroll
         for (int i = 0; i < RS; i++) {
             const int row = i * 16 + w * 4 + grp;
@@ -155,7 +167,27 @@ __device__ __forceinline__ void gdn_tokens(const bf16_t* __restrict__ proj, cons
             s[i][1] = f4{sv[4], sv[5], sv[6], sv[7]};
             __builtin_nontemporal_store(s[i][0], so4 + row * (DK / 4) + c);
             __builtin_nontemporal_store(s[i][1], so4 + row * (DK / 4) + 16 + c);
-            if (c == 0) yo[row] = f2bf(yv);
+            if (!NORM) {
+                if (c == 0) yo[row] = f2bf(yv);
+            } else {
+                yb[i] = BF(yv);
+            }
+        }
+        if (NORM) {
+            // sum of squares of the head's 128 stored outputs: this lane's 8 rows, the wavefront's 4 groups, the 4 wavefronts
+            double ss = 0.0;
+#pragma unroll
+            for (int i = 0; i < RS; i++) ss += (double)yb[i] * yb[i];
+            ss += __shfl_xor(ss, 16, 64);
+            ss += __shfl_xor(ss, 32, 64);
+            __syncthreads();                                     // `red` was last read in the prologue
+            if (lane == 0) red[w] = ss;
+            __syncthreads();
+            const float inv = rsqrt_rn((float)((red[0] + red[1]) + (red[2] + red[3])) / 128.f + eps);
+            float mine = yb[0];
+#pragma unroll
+            for (int i = 1; i < RS; i++) mine = ((c & 7) == i) ? yb[i] : mine;
+            if (c < 8) yo[nrow] = gated_out(nz, ngw * (mine * inv));
         }
     }
 }
@@ -190,23 +222,24 @@ __global__ __launch_bounds__(256) void gdn_decode_kernel(const bf16_t* __restric
 
 // the same step with HPW heads of one row per workgroup (256 threads per head, whole heads only): the workgroup streams
 // HPW * 64 KiB of contiguous state
-template <int HPW>
+template <int HPW, bool NORM = false>
 __global__ __launch_bounds__(256 * HPW) void gdn_decode_wide_kernel(const bf16_t* __restrict__ proj, bf16_t* conv_pool,
                                                                     const bf16_t* __restrict__ cw,
                                                                     const float* __restrict__ A_log,
                                                                     const float* __restrict__ dt_bias, float* ssm_pool,
                                                                     const int* __restrict__ slots,
                                                                     const int* __restrict__ pos, bf16_t* __restrict__ y,
-                                                                    int n_slots) {
+                                                                    int n_slots, const float* __restrict__ gw = nullptr,
+                                                                    float eps = 0.f) {
     const unsigned id = xcd_remap(blockIdx.x, gridDim.x);
     const int b = id / (HV / HPW), h = (id % (HV / HPW)) * HPW + (threadIdx.x >> 8);
     const int slot = slots[b];
     if ((unsigned)slot >= (unsigned)n_slots) return;
     const int par = pos[b] & 1;
     float* st = ssm_pool + (size_t)slot * HV * DV * DK;
-    gdn_tokens<8, HPW>(proj + (size_t)b * PW, conv_pool + (size_t)(slot * 2 + par) * 3 * CD,
-                       conv_pool + (size_t)(slot * 2 + (par ^ 1)) * 3 * CD, 0, cw, A_log, dt_bias, st, st, 0,
-                       y + (size_t)b * KD, 1, h, 0);
+    gdn_tokens<8, HPW, NORM>(proj + (size_t)b * PW, conv_pool + (size_t)(slot * 2 + par) * 3 * CD,
+                             conv_pool + (size_t)(slot * 2 + (par ^ 1)) * 3 * CD, 0, cw, A_log, dt_bias, st, st, 0,
+                             y + (size_t)b * KD, 1, h, 0, gw, eps);
 }
 
 // batch_spec.deltanet_bm (qwen35/batch_spec.py:142-150): M chained tokens per sequence, snapshot pools in place
@@ -290,6 +323,25 @@ int qt_gdn_decode_step(const void* proj, void* conv_pool, const void* conv_w, co
         QT_DISPATCH_RS(rs, gdn_decode_kernel, B, stream, (const bf16_t*)proj, (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log,
                        dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
     }
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+// batch.deltanet_b followed by batch.gnorm_rows (qwen35/batch.py:128-135, 338-343) in one launch: `out` receives the gated
+// RMSNorm of the step's outputs (same bits as the two launches), the outputs themselves are not stored.
+int qt_gdn_decode_step_gnorm(const void* proj, void* conv_pool, const void* conv_w, const float* A_log, const float* dt_bias,
+                             float* ssm_pool, const int32_t* slots, const int32_t* pos, const float* gw, float eps, void* out, int B,
+                             int n_slots, hipStream_t stream) {
+    if (!proj || !conv_pool || !conv_w || !A_log || !dt_bias || !ssm_pool || !slots || !pos || !gw || !out) return QT_ERR_NULL;
+    if (B < 0 || n_slots <= 0) return QT_ERR_DIM;
+    if (B == 0) return QT_OK;
+    if (!aligned16(ssm_pool) || (reinterpret_cast<uintptr_t>(conv_w) & 7u)) return QT_ERR_ALIGN;
+#define QT_GNORM_LAUNCH(HPW_)                                                                                                  \
+    hipLaunchKernelGGL((gdn_decode_wide_kernel<HPW_, true>), dim3(B * (HV / HPW_)), dim3(256 * HPW_), 0, stream, (const bf16_t*)proj, \
+                       (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log, dt_bias, ssm_pool, slots, pos, (bf16_t*)out, n_slots, gw, eps)
+    if (B >= 64) QT_GNORM_LAUNCH(4);
+    else if (B >= 32) QT_GNORM_LAUNCH(2);
+    else QT_GNORM_LAUNCH(1);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

@@ -333,3 +333,27 @@ def test_deltanet_bm_layout_of_reference_test(qt, dev):
             check_tensors_equal('torch.equal(ssm_pool[s_], sr)', ssm_pool[s_], sr)
         for e in (2, 3, 6):
             check_equal('np.array_equal(to_np(ssm_pool[e]), sp[e])', to_np(ssm_pool[e]), sp[e])
+
+
+@pytest.mark.parametrize("B", [1, 5, 32, 64])
+def test_deltanet_b_gnorm_equals_two_launches(qt, dev, B):
+    """the decode step with the gated RMSNorm fused in == deltanet_b followed by gnorm_rows (batch.py:497-499), bit for bit,
+    for each workgroup shape the batch size selects (1, 2 or 4 heads per workgroup)"""
+    gen = torch.Generator().manual_seed(200 + B)
+    cw, A_log, dtb, gw = layer_params(20 + B)
+    S = B + 2
+    ssm = (torch.randn((S + 1, 16, 128, 128), generator=gen) * 0.05).numpy()
+    cp = rand_bf(gen, ((S + 1) * 2, 3, CD))
+    slots = torch.randperm(S, generator=gen).numpy().astype(np.int32)[:B]
+    pos = torch.randint(0, 500, (B,), generator=gen).numpy().astype(np.int32)
+    proj = to_dev(rand_bf(gen, (B, PW), 1.5), dev, BF16)
+    dcw, dA, ddt, dgw = to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev), to_dev(gw, dev)
+    c1, s1 = to_dev(cp, dev, BF16), to_dev(ssm, dev)
+    y = qt.batch.deltanet_b(proj, c1, dcw, dA, ddt, s1, to_dev(slots, dev), to_dev(pos, dev))
+    want = qt.batch.gnorm_rows(y, proj, dgw)
+    c2, s2 = to_dev(cp, dev, BF16), to_dev(ssm, dev)
+    got = qt.batch.deltanet_b_gnorm(proj, c2, dcw, dA, ddt, s2, to_dev(slots, dev), to_dev(pos, dev), dgw)
+    check_tensors_equal("gated-norm output", got, want)
+    check_tensors_equal("conv pool", c2, c1)
+    check_tensors_equal("ssm pool", s2, s1)
+    check_equal("against the oracle", to_np(got), O.gated_norm(to_np(y), to_np(proj), gw))
