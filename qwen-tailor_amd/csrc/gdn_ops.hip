@@ -41,54 +41,51 @@ __global__ __launch_bounds__(256) void normalize_qk_kernel(const bf16_t* __restr
 }
 
 // conv_prep (qwen35/prefill.py:96-134, 228-238): proj [S,8224], cs [3,6144] -> q, k, v [S,16,128].
-// A workgroup of 256 threads handles 32 consecutive tokens of one head: a 16-lane group owns one token per round (two
-// rounds), a lane 8 consecutive channels of q, of k and of v; all row loads of both rounds are issued before the first
-// conv, SiLU comes from the LDS table, the sum of squares is reduced over the 16 lanes of the group.
-constexpr int CP_TOK = 32;
-__global__ __launch_bounds__(256) void conv_prep_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs,
-                                                        const bf16_t* __restrict__ cw, const bf16_t* __restrict__ silu_tab,
-                                                        bf16_t* __restrict__ q, bf16_t* __restrict__ k, bf16_t* __restrict__ v,
-                                                        int S) {
+// A workgroup of 256 threads handles 64 consecutive tokens of one head: a 16-lane group owns 4 consecutive tokens (their 7
+// input rows are loaded once and shared by the 4 sliding windows), a lane 8 consecutive channels of q, of k and of v; all row
+// loads are issued before the first conv, SiLU comes from the LDS table, the sums of squares are reduced over the 16 lanes of
+// the group and the 8 reciprocal square roots are evaluated one per lane.
+constexpr int CP_TOK = 64;
+__global__ __launch_bounds__(256, 2) void conv_prep_kernel(const bf16_t* __restrict__ proj, const bf16_t* __restrict__ cs,
+                                                           const bf16_t* __restrict__ cw, const bf16_t* __restrict__ silu_tab,
+                                                           bf16_t* __restrict__ q, bf16_t* __restrict__ k, bf16_t* __restrict__ v,
+                                                           int S) {
     __shared__ __align__(16) bf16_t tab[SILU_TAB_SIZE];
     const int tb = blockIdx.x / HV, h = blockIdx.x % HV, tid = threadIdx.x, gi = tid >> 4, cc = tid & 15;
-    uint4 raw[2][3][4], wt[3][4];
+    const int t0 = tb * CP_TOK + 4 * gi;
+    uint4 rw[3][7], wt[3][4];
 #pragma unroll
     for (int part = 0; part < 3; part++) {
         const int ch0 = part * KD + h * DK + cc * 8;
 #pragma unroll
         for (int e = 0; e < 4; e++) wt[part][e] = *reinterpret_cast<const uint4*>(cw + (size_t)(ch0 + 2 * e) * 4);
 #pragma unroll
-        for (int r = 0; r < 2; r++) {
-            const int t = min(tb * CP_TOK + r * 16 + gi, S - 1);               // rows past the end are computed and dropped
-#pragma unroll
-            for (int d = 0; d < 4; d++) {
-                const int tt = t - 3 + d;
-                raw[r][part][d] = *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0);
-            }
+        for (int d = 0; d < 7; d++) {
+            const int tt = min(t0 - 3 + d, S - 1);                             // rows past the end are computed and dropped
+            rw[part][d] = *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0);
         }
     }
     silu_table_fill(tab, silu_tab, tid, 256);
     __syncthreads();
     const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
-    uint4 pk[2][3];
-    float ss[4], rr[4];
+    uint4 pk[4][3];
+    float ss[8], rr[8];
 #pragma unroll
     for (int part = 0; part < 3; part++)
 #pragma unroll
-        for (int r = 0; r < 2; r++) {
-            const double sq = conv8_silu_packed(tab, raw[r][part][0], raw[r][part][1], raw[r][part][2], raw[r][part][3], wt[part],
-                                                pk[r][part]);
-            if (part < 2) ss[2 * r + part] = (float)row16_sum_d(sq);
+        for (int j = 0; j < 4; j++) {
+            const double sq = conv8_silu_packed(tab, rw[part][j], rw[part][j + 1], rw[part][j + 2], rw[part][j + 3], wt[part], pk[j][part]);
+            if (part < 2) ss[2 * j + part] = (float)row16_sum_d(sq);
         }
-    rsqrt_rows<4>(ss, qk_eps(), rr, cc);
+    rsqrt_rows<8>(ss, qk_eps(), rr, cc);
 #pragma unroll
-    for (int r = 0; r < 2; r++) {
-        const int t = tb * CP_TOK + r * 16 + gi;
+    for (int j = 0; j < 4; j++) {
+        const int t = t0 + j;
         if (t < S) {
             const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
-            *reinterpret_cast<uint4*>(q + o) = scale8_packed(pk[r][0], rr[2 * r], scq);
-            *reinterpret_cast<uint4*>(k + o) = scale8_packed(pk[r][1], rr[2 * r + 1], sck);
-            *reinterpret_cast<uint4*>(v + o) = pk[r][2];
+            *reinterpret_cast<uint4*>(q + o) = scale8_packed(pk[j][0], rr[2 * j], scq);
+            *reinterpret_cast<uint4*>(k + o) = scale8_packed(pk[j][1], rr[2 * j + 1], sck);
+            *reinterpret_cast<uint4*>(v + o) = pk[j][2];
         }
     }
 }

@@ -52,6 +52,18 @@ def test_null_and_dimension_errors_from_the_c_abi():
     assert lib.qt_gqa_attn_workspace_bytes(16, 1, 32768, 1024) == (1024 + 16 * 2) * 4 * 258 * 4
     assert lib.qt_gqa_attn_workspace_bytes(1, 0, 16, 16) == -1
     assert lib.qt_normalize_qk(ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16), 1, 64, z) == -4
+    p16 = ctypes.c_void_p(16)
+    assert lib.qt_gdn_decode_step_gnorm(z, z, z, z, z, z, z, z, z, 1e-6, z, 1, 1, z) == -3
+    assert lib.qt_blit(z, p16, 2, 8, 0, 0, 1, 0, 0, z) == -3
+    assert lib.qt_blit(p16, p16, 3, 8, 0, 0, 1, 0, 0, z) == -4                       # element size 2 or 4 only
+    assert lib.qt_blit(p16, p16, 2, -1, 0, 0, 1, 0, 0, z) == -1
+    assert lib.qt_blit(p16, p16, 2, 0, 0, 0, 1, 0, 0, z) == 0                        # nothing to copy: no launch
+    assert lib.qt_attn_qkv_prep(p16, p16, p16, p16, p16, p16, p16, 6, 4, 1e-6, z) == -1      # M must divide the rows
+    assert lib.qt_attn_qkv_prep(p16, p16, p16, z, p16, p16, p16, 4, 4, 1e-6, z) == -3
+    assert lib.qt_attn_out_gate(p16, ctypes.c_void_p(8), p16, 1, z) == -2
+    assert lib.qt_gdn_phase_a_conv(p16, p16, p16, p16, p16, p16, p16, z, z, z, p16, p16, p16, 64, z) == -3   # q without k, v
+    assert lib.qt_gdn_phase_a_conv(p16, p16, p16, p16, p16, p16, z, z, z, p16, p16, p16, p16, 64, z) == -4   # conv_out aliases conv_state
+    assert lib.qt_gqa_attn_decode(p16, p16, p16, p16, p16, p16, p16, p16, p16, 1 << 40, 2000, 1, 64, 1, 128, z) == -4   # B * 2 > 2048 segments
 
 
 def test_product_does_not_import_the_oracle():

@@ -58,6 +58,12 @@ def test_oracle_reproduces_fixtures():
     o = O.attn_b(unbits(z["q"]), unbits(z["kn"]), unbits(z["vn"]), unbits(z["Kp"]), unbits(z["Vp"]), z["slots"], z["pos"], int(z["M"]))
     check_equal("attn_b", o, unbits(z["o"]))
     check_equal("sdpa_causal", O.sdpa_causal(unbits(z["qc"]), unbits(z["Kc"]), unbits(z["Vc"])), unbits(z["oc"]))
+    z = np.load(os.path.join(G, "attn_glue.npz"))
+    q, k, v = O.attn_qkv_prep(unbits(z["qkv"]), unbits(z["q_norm"]), unbits(z["k_norm"]), z["pos"], int(z["M"]))
+    check_equal("glue q", q, unbits(z["q"]))
+    check_equal("glue k", k, unbits(z["k"]))
+    check_equal("glue v", v, unbits(z["v"]))
+    check_equal("glue gate", O.attn_out_gate(unbits(z["o"]), unbits(z["qkv"])), unbits(z["gated"]))
 
 
 @pytest.fixture(scope="module")
@@ -106,3 +112,14 @@ def test_attention_matches_fixture(qt, dev):
     check_rel("attn_b", to_np(o), unbits(z["o"]), 1e-2, rel_l2)
     oc = qt.attention.scaled_dot_product_attention(d("qc")[None], d("Kc")[None], d("Vc")[None], scale=256 ** -0.5, mask="causal")
     check_rel("causal prefill", to_np(oc)[0], unbits(z["oc"]), 1e-2, rel_l2)
+
+
+@pytest.mark.gpu
+def test_attention_glue_matches_fixture(qt, dev):
+    z = np.load(os.path.join(G, "attn_glue.npz"))
+    d = lambda name: to_dev(unbits(z[name]), dev, BF16)
+    q, k, v = qt.attention.qkv_prep(d("qkv"), d("q_norm"), d("k_norm"), to_dev(z["pos"], dev), int(z["M"]))
+    check_equal("q", to_np(q), unbits(z["q"]))
+    check_equal("k", to_np(k), unbits(z["k"]))
+    check_equal("v", to_np(v), unbits(z["v"]))
+    check_equal("gated output", to_np(qt.attention.out_gate(d("o"), d("qkv"))), unbits(z["gated"]))
