@@ -256,28 +256,33 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
         float gwv[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) gwv[j] = gw[cc * 8 + j];
+        // the four rows of this 16-lane group: all sums of squares first, then one reciprocal square root per lane
+        uint4 yv4[4];
+        float ss4[4], inv4[4];
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int row = it * 16 + (threadIdx.x >> 4);
+            yv4[it] = *reinterpret_cast<const uint4*>(&ys[row * YS_LD + cc * 8]);
+            float yy[8];
+            unpack8(yv4[it], yy);
+            double ss = 0.0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
+            ss4[it] = (float)row16_sum_d(ss);
+        }
+        rsqrt_rows<4>(ss4, eps, inv4, cc);
 #pragma unroll
         for (int it = 0; it < 4; it++) {
             const int row = it * 16 + (threadIdx.x >> 4);
             const int t = c * C + row;
             if (t >= S) continue;                                               // whole 16-lane groups leave together
-            const uint4 yv = *reinterpret_cast<const uint4*>(&ys[row * YS_LD + cc * 8]);
             const uint4 zv = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
-            const uint32_t yw[4] = {yv.x, yv.y, yv.z, yv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
             float yy[8], zz[8];
-            double ss = 0.0;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                yy[2 * j] = lo_bf(yw[j]);
-                yy[2 * j + 1] = hi_bf(yw[j]);
-                zz[2 * j] = lo_bf(zw[j]);
-                zz[2 * j + 1] = hi_bf(zw[j]);
-                ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
-            }
-            const float inv = rsqrt_rn((float)row16_sum_d(ss) / 128.f + eps);
+            unpack8(yv4[it], yy);
+            unpack8(zv, zz);
             uint32_t o[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv));
+            for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv4[it]));
             reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV)[cc] =
                 make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
         }

@@ -95,36 +95,49 @@ __global__ __launch_bounds__(256) void silu_table_kernel(bf16_t* __restrict__ ta
     if (i < SILU_TAB_SIZE) tab[i] = silu_table_entry(i);
 }
 
-// gated RMSNorm (qwen35/batch.py:304-343, qwen35/prefill.py:137-157): 16 lanes per (row, head), 8 elements per lane.
+// gated RMSNorm (qwen35/batch.py:304-343, qwen35/prefill.py:137-157): 16 lanes per (row, head), 8 elements per lane; a
+// workgroup takes GN_ROWS rows (all loads first), and the GN_ROWS double-precision reciprocal square roots of a 16-lane group
+// are evaluated one per lane instead of all by every lane.  GN_ROWS = 4 for many rows (the kernel is then bound by those
+// evaluations), 1 for few (bound by the latency of one workgroup).
+template <int GN_ROWS>
 __global__ __launch_bounds__(256) void gated_norm_kernel(const bf16_t* __restrict__ y, const bf16_t* __restrict__ proj,
                                                          const float* __restrict__ gw, bf16_t* __restrict__ out, long rows,
                                                          float eps) {
-    const long grp = (long)blockIdx.x * 16 + (threadIdx.x >> 4);       // (row, head)
-    const int c = threadIdx.x & 15;
-    if (grp >= rows * HV) return;
-    const long row = grp / HV;
-    const int h = (int)(grp % HV);
-    const uint4 yv = reinterpret_cast<const uint4*>(y + row * KD + h * DV)[c];
-    const uint4 zv = reinterpret_cast<const uint4*>(proj + row * PW + CD + h * DV)[c];
-    const uint32_t yw[4] = {yv.x, yv.y, yv.z, yv.w}, zw[4] = {zv.x, zv.y, zv.z, zv.w};
-    float yy[8], zz[8];
-    double ss = 0.0;
+    const int h = threadIdx.x >> 4, c = threadIdx.x & 15;
+    const long row0 = (long)blockIdx.x * GN_ROWS;
+    uint4 yv[GN_ROWS], zv[GN_ROWS];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        yy[2 * j] = lo_bf(yw[j]);
-        yy[2 * j + 1] = hi_bf(yw[j]);
-        zz[2 * j] = lo_bf(zw[j]);
-        zz[2 * j + 1] = hi_bf(zw[j]);
-        ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
+    for (int it = 0; it < GN_ROWS; it++) {
+        const long row = row0 + it < rows ? row0 + it : rows - 1;              // rows past the end are computed and dropped
+        yv[it] = reinterpret_cast<const uint4*>(y + row * KD + h * DV)[c];
+        zv[it] = reinterpret_cast<const uint4*>(proj + row * PW + CD + h * DV)[c];
     }
-    const float inv = rsqrt_rn((float)row16_sum_d(ss) / 128.f + eps);
-    uint32_t o[8];
+    float gwv[8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-        o[j] = gated_out(zz[j], gw[c * 8 + j] * (yy[j] * inv));
+    for (int j = 0; j < 8; j++) gwv[j] = gw[c * 8 + j];
+    float ss[GN_ROWS], inv[GN_ROWS];
+#pragma unroll
+    for (int it = 0; it < GN_ROWS; it++) {
+        float yy[8];
+        unpack8(yv[it], yy);
+        double s2 = 0.0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) s2 += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
+        ss[it] = (float)row16_sum_d(s2);
     }
-    uint4 ov = make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
-    reinterpret_cast<uint4*>(out + row * KD + h * DV)[c] = ov;
+    rsqrt_rows<GN_ROWS>(ss, eps, inv, c);
+#pragma unroll
+    for (int it = 0; it < GN_ROWS; it++) {
+        if (row0 + it >= rows) break;
+        float yy[8], zz[8];
+        unpack8(yv[it], yy);
+        unpack8(zv[it], zz);
+        uint32_t o[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv[it]));
+        reinterpret_cast<uint4*>(out + (row0 + it) * KD + h * DV)[c] =
+            make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
+    }
 }
 
 // gated_delta_update's kernel (qwen35/gated_delta.py:33-137): T sequential tokens with q, k, v, g, beta given.
@@ -230,8 +243,12 @@ int qt_gated_rmsnorm(const void* y, const void* proj, const float* gw, void* out
     if (rows < 0) return QT_ERR_DIM;
     if (rows == 0) return QT_OK;
     if (!al(y, 16) || !al(proj, 16) || !al(out, 16)) return QT_ERR_ALIGN;
-    hipLaunchKernelGGL(gated_norm_kernel, dim3((unsigned)rows), dim3(256), 0, stream, (const bf16_t*)y, (const bf16_t*)proj, gw,
-                       (bf16_t*)out, rows, eps);
+    if (rows >= 4096)
+        hipLaunchKernelGGL(gated_norm_kernel<4>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, (const bf16_t*)y,
+                           (const bf16_t*)proj, gw, (bf16_t*)out, rows, eps);
+    else
+        hipLaunchKernelGGL(gated_norm_kernel<1>, dim3((unsigned)rows), dim3(256), 0, stream, (const bf16_t*)y, (const bf16_t*)proj, gw,
+                           (bf16_t*)out, rows, eps);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

@@ -76,10 +76,12 @@ __device__ __forceinline__ float softplus_bf16(float x) {                       
 // float exp and does not round it; here both exps are float with <= 1 ulp error.
 __device__ __forceinline__ float log_decay(float A_log, float av) { return -expf(A_log) * softplus_bf16(av); }
 __device__ __forceinline__ float decay_gate(float A_log, float av) { return expf(log_decay(A_log, av)); }
-// z * sigmoid(z) * n rounded to bf16 once (kernels.py:134-137): z/(1+exp32(-z)) * n
+// z * sigmoid(z) * n rounded to bf16 once (kernels.py:134-137): z/(1+exp32(-z)) * n.  The fast path uses the hardware
+// reciprocal and float exp (a few ulp off in total); a result within 16 float ulp of a bf16 rounding boundary, or a large |z|,
+// takes the exact path (IEEE divide, double-precision exp).
 __device__ __forceinline__ bf16_t gated_out(float z, float n) {
-    float o = __fdiv_rn(z, 1.0f + expf(-z)) * n;
-    if (__builtin_expect(near_bf16_tie(o, 8) || fabsf(z) > 80.0f, 0)) o = __fdiv_rn(z, 1.0f + exp32(-z)) * n;
+    float o = z * __builtin_amdgcn_rcpf(1.0f + expf(-z)) * n;
+    if (__builtin_expect(near_bf16_tie(o, 16) || fabsf(z) > 80.0f, 0)) o = __fdiv_rn(z, 1.0f + exp32(-z)) * n;
     return f2bf(o);
 }
 

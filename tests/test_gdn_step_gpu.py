@@ -86,7 +86,7 @@ def test_normalize_qk_and_compute_g_bit_exact(qt, dev):
         qt.gated_delta.normalize_qk(to_dev(q[..., :64], dev, BF16), to_dev(k[..., :64], dev, BF16), inv_scale=64 ** -0.5, eps=1e-6)
 
 
-@pytest.mark.parametrize("R", [1, 7, 64, 2048])
+@pytest.mark.parametrize("R", [1, 7, 64, 2048, 4099])
 def test_gated_norm_bit_exact(qt, dev, R):
     gen = torch.Generator().manual_seed(200 + R)
     cw, A_log, dtb, gw = layer_params(3)
