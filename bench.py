@@ -307,6 +307,8 @@ def profile_leg(torch, qt, dev, args):
         bench_attn(torch, qt, dev, 16, 4, 1024, 8192, 1004)
     elif leg == "attn_prefill":
         bench_attn_prefill(torch, qt, dev)
+    elif leg == "attn_prefill_long":
+        bench_attn_prefill(torch, qt, dev, 8192)
     else:
         raise SystemExit(f"unknown leg {leg}")
     torch.cuda.synchronize()
@@ -335,7 +337,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the B sweep and the single-pool run")
     ap.add_argument("--only", default="", help="profile helper: run only one leg a few times and exit "
-                                               "(decode | copy | prefill | verify | attn_decode | attn_verify | attn_prefill)")
+                                               "(decode | copy | prefill | verify | attn_decode | attn_verify | attn_prefill | attn_prefill_long)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every work item of the path is an independent (slot, head) pair; "

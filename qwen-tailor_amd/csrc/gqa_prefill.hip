@@ -11,8 +11,11 @@
 //     O[rows x 256]   += P . V            A = two exponentiated S^T accumulators packed to bf16 (they ARE the A operand
 //                                         when a 32-key block is enumerated as 16 (j >> 2) + 4 g + (j & 3)),
 //                                         B = V through the transposing LDS load (4 consecutive keys of one column)
-// The next tile travels global -> registers while the current one is consumed; two barriers per tile.  A wavefront runs
-// at one per SIMD and keeps about 400 registers (Q^T of two heads, two 16 x 256 accumulators, the tile in flight).
+// K / V tiles travel HBM -> LDS directly (global_load_lds_dwordx4: 64 lanes x 16 bytes land as one contiguous KiB, no
+// registers in between) into double-buffered tiles, so the next tile's loads are in flight during the whole of the current
+// tile's arithmetic and a tile costs one workgroup barrier.  The LDS rows are unpadded (a direct load cannot pad); instead the
+// 16-byte chunks of row r are stored XOR-swizzled by r & 15 (the loading lane picks the matching global chunk), which keeps
+// the fragment reads of 16 rows on distinct banks.
 #include "qt_common.h"
 
 using namespace qt;
@@ -25,11 +28,10 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr float SCALE = 0.0625f;       // 256^-0.5
+constexpr float SCALE_LOG2E = 0.0625f * 1.4426950408889634f;   // 256^-0.5 log2 e: scores are exponentiated in base 2
 constexpr float NEG = -3.0e38f;
 constexpr int KT = 64;                 // keys per tile
-constexpr int KS_LD = AD + 8;          // LDS row strides (elements): 528 / 544 bytes spread the rows over the banks
-constexpr int VS_LD = AD + 16;
+constexpr int TILE = KT * AD;          // elements of one K or V tile in LDS (32 KiB), rows unpadded, chunks swizzled
 
 // AP_MARK(i): per-tile phase time stamps for profiling builds (QT_ATTN_PREFILL_PROF defines ap_prof_buf[workgroup][wave][8],
 // accumulated shader-clock ticks per phase); compiles to nothing otherwise
@@ -43,7 +45,7 @@ __device__ long long* ap_prof_buf;
     } while (0)
 #define AP_INIT() long long ap_last_ = clock64()
 #else
-#define AP_MARK(i)
+#define AP_MARK(i) __builtin_amdgcn_sched_barrier(0)     /* the phases of a tile are scheduled separately */
 #define AP_INIT()
 #endif
 
@@ -56,11 +58,11 @@ __device__ __forceinline__ void wave_lds_sync() {
 // NH = heads per wavefront: 2 (32 query rows per workgroup, as described above) for long sequences; 1 (16 rows per workgroup,
 // one head per wavefront: twice the workgroups, LDS-bound) when the launch would otherwise leave CUs idle.
 template <int NH>
-__global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
+__global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
                                                            const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
                                                            int q_pos0, long q_head_stride, long kv_head_stride) {
-    __shared__ __align__(16) bf16_t k_s[KT * KS_LD];
-    __shared__ __align__(16) bf16_t v_s[KT * VS_LD];
+    __shared__ __align__(1024) bf16_t k_s[2][TILE];
+    __shared__ __align__(1024) bf16_t v_s[2][TILE];
     __shared__ __align__(16) float c_s[4][2][16];
     constexpr int RB = 16 * NH;
     const int rb = gridDim.x - 1 - blockIdx.x;                   // long rows first
@@ -87,20 +89,31 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
             bq[hh][kb] = __builtin_bit_cast(bf16x8, v);
         }
     }
-    // tile loader: thread (tid >> 5, tid & 31) moves 16 bytes of the rows tid >> 5 + 8 i, i = 0..7, of K and of V
-    const int lr = tid >> 5, lc = tid & 31;
-    const bf16_t* kg = K + (size_t)kvh * kv_head_stride + 8 * lc;
-    const bf16_t* vg = V + (size_t)kvh * kv_head_stride + 8 * lc;
-    u32x4 kr[8], vr[8];
-    auto load_tile = [&](int t) {
+    // tile loader: wavefront w issues direct-to-LDS loads i = 0..7 of K and of V; load 8 w + i fills rows 2 (8 w + i) and
+    // + 1 (one KiB): lane l lands at chunk position l & 31 of row 2 (8 w + i) + (l >> 5) and fetches chunk (l & 31) ^ (row & 15).
+    // The per-lane byte offsets within a tile do not change from tile to tile; only the last tile of a sequence clamps rows.
+    const char* kg = reinterpret_cast<const char*>(K + (size_t)kvh * kv_head_stride);
+    const char* vg = reinterpret_cast<const char*>(V + (size_t)kvh * kv_head_stride);
+    // byte offset of load 0 within a tile; load i differs by XOR with 1056 i (row bits 10..12, chunk bits 5..7)
+    const unsigned ld_off0 = (unsigned)(16 * w + (lane >> 5)) * (AD * 2) + ((unsigned)((lane & 31) ^ (lane >> 5)) << 4);
+    auto load_tile = [&](int t, int buf) {
+        const bool whole = t * KT + KT <= L;                     // else: rows past the end repeat the last key; they are masked
+        const char* kt_g = kg + (size_t)t * (KT * AD * 2);
+        const char* vt_g = vg + (size_t)t * (KT * AD * 2);
+        unsigned off0 = ld_off0;
+        asm volatile("" : "+v"(off0));                           // recompute the eight offsets per tile (one XOR each) rather than
+                                                                 // keeping them in registers the accumulators need
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const int key = min(t * KT + lr + 8 * i, L - 1);     // rows past the end repeat the last key; they are masked
-            kr[i] = *reinterpret_cast<const u32x4*>(kg + (size_t)key * AD);
-            vr[i] = *reinterpret_cast<const u32x4*>(vg + (size_t)key * AD);
+            unsigned off = off0 ^ (1056u * i);
+            if (!whole) off = (unsigned)min((int)(off >> 9), L - 1 - t * KT) * (AD * 2) + (off & 511u);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kt_g + off),
+                                             (__attribute__((address_space(3))) void*)(&k_s[buf][(8 * w + i) * 512]), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vt_g + off),
+                                             (__attribute__((address_space(3))) void*)(&v_s[buf][(8 * w + i) * 512]), 16, 0, 0);
         }
     };
-    load_tile(0);
+    load_tile(0, 0);
 
     float m_run[NH], l_run[NH];
     f32x4 O[NH][16];
@@ -110,67 +123,84 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
         for (int j = 0; j < 16; j++) O[hh][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int hh = 0; hh < NH; hh++) m_run[hh] = NEG, l_run[hh] = 0.f;
-    const bf16_t* ka = k_s + n * KS_LD + 8 * g;                  // A operand of the scores: row 16 kt + n, columns 32 kb + 8 g
+    // A operand of the scores: row 16 kt + n of the tile, chunk (4 kb + g) ^ n
+    const int ka_row = n * AD;
     // transposing load: within 16 lanes, lane 4q + i receives element i of the 8-byte chunks addressed by lanes q, q+4,
     // q+8, q+12; lane n of group g points at key 4g + n/4, columns 4 (n%4).. of the block and receives keys 4g..4g+3 of column n
-    const bf16_t* va = v_s + (4 * g + (n >> 2)) * VS_LD + 4 * (n & 3);
+    const int vrow = 4 * g + (n >> 2);                           // row within a 16-key block = its swizzle
+    const int va_row = vrow * AD + 4 * (n & 1), vc0 = (n & 3) >> 1;
 
     AP_INIT();
     for (int t = 0; t < ntiles; t++) {
+        const int buf = t & 1;
         AP_MARK(0);
-        __syncthreads();                                         // everyone is done reading the previous tile
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wavefront's part of tile t has landed in LDS
         AP_MARK(1);
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            *reinterpret_cast<u32x4*>(k_s + (lr + 8 * i) * KS_LD + 8 * lc) = kr[i];
-            *reinterpret_cast<u32x4*>(v_s + (lr + 8 * i) * VS_LD + 8 * lc) = vr[i];
-        }
-        if (t + 1 < ntiles) load_tile(t + 1);
-        __syncthreads();
+        __syncthreads();                                         // ... and everyone's; everyone is done with tile t - 1
+        if (t + 1 < ntiles) load_tile(t + 1, buf ^ 1);           // in flight during the whole of this tile's arithmetic
         AP_MARK(2);
+        const bf16_t* ka = &k_s[buf][ka_row];
+        const bf16_t* va = &v_s[buf][va_row];
         if (t >= ntiles_w) continue;                             // wavefront-uniform: the upper row block may see one tile more
 
         // scores: each K fragment multiplies the Q^T of both heads (the compiler overlaps the next sub-tile's LDS reads with
         // these MFMAs as registers allow)
         f32x4 acc[NH][4];
-        bf16x8 Af[8];
+        bf16x8 Af[2][8];
+#pragma unroll
+        for (int kb = 0; kb < 8; kb++) Af[0][kb] = *reinterpret_cast<const bf16x8*>(ka + (((4 * kb + g) ^ n) << 3));
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (kt < 3) {
 #pragma unroll
-            for (int kb = 0; kb < 8; kb++) Af[kb] = *reinterpret_cast<const bf16x8*>(ka + 16 * kt * KS_LD + 32 * kb);
+                for (int kb = 0; kb < 8; kb++)
+                    Af[(kt + 1) & 1][kb] = *reinterpret_cast<const bf16x8*>(ka + 16 * (kt + 1) * AD + (((4 * kb + g) ^ n) << 3));
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int hh = 0; hh < NH; hh++) acc[hh][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kb = 0; kb < 8; kb++)
 #pragma unroll
                 for (int hh = 0; hh < NH; hh++)
-                    acc[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kb], bq[hh][kb], acc[hh][kt], 0, 0, 0);
+                    acc[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kt & 1][kb], bq[hh][kb], acc[hh][kt], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
         AP_MARK(3);
+        // softmax in base 2 on the raw products: p = 2^(c s - m), c = 256^-0.5 log2 e; only tiles that touch the diagonal or
+        // the end of the sequence need the mask (wavefront-uniform); every row sees key 0, so its maximum is finite from the
+        // first tile on and masked entries come out as 2^-huge = 0
+        if (t * KT + KT - 1 > q_pos0 + r0 || t * KT + KT > L) {
+#pragma unroll
+            for (int hh = 0; hh < NH; hh++)
+#pragma unroll
+                for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int key = t * KT + 16 * kt + 4 * g + i;
+                        if (!(key <= my_last && key < L)) acc[hh][kt][i] = NEG;
+                    }
+        }
         s16x8 P[NH][2];
         bool rescale = false;
 #pragma unroll
         for (int hh = 0; hh < NH; hh++) {
-            float sc[4][4], mx = NEG;
+            float mx = NEG;
 #pragma unroll
             for (int kt = 0; kt < 4; kt++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int key = t * KT + 16 * kt + 4 * g + i;
-                    sc[kt][i] = (key <= my_last && key < L) ? acc[hh][kt][i] * SCALE : NEG;
-                    mx = fmaxf(mx, sc[kt][i]);
-                }
+                for (int i = 0; i < 4; i++) mx = fmaxf(mx, acc[hh][kt][i]);
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run[hh], mx);
-            const float corr = __expf(m_run[hh] - m_new);        // m_run = NEG initially: exp(-huge) = 0
+            const float m_new = fmaxf(m_run[hh], mx * SCALE_LOG2E);
+            const float corr = __builtin_amdgcn_exp2f(m_run[hh] - m_new);      // m_run = NEG initially: 2^-huge = 0
             float ps = 0.f;
 #pragma unroll
             for (int kt = 0; kt < 4; kt++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const float pv = sc[kt][i] > 0.5f * NEG ? __expf(sc[kt][i] - m_new) : 0.f;
+                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt][i], SCALE_LOG2E, -m_new));
                     ps += pv;
                     P[hh][kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(pv);
                 }
@@ -194,7 +224,7 @@ __global__ __launch_bounds__(256, (NH == 1 ? 2 : 1)) void attn_prefill_kernel(co
         // both heads
         auto v_frag = [&](int j, int q4) {
             return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * VS_LD + 16 * j)));
+                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * AD + (((2 * j + vc0) ^ vrow) << 3))));
         };
         s16x4 Bf[3][4];
 #pragma unroll
