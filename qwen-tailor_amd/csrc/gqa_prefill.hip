@@ -55,6 +55,11 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// The output accumulators live in the accumulation half of the register file, which MFMA reads and writes in place; only the
+// rare rescale moves them through VALU registers.  The empty asm ties that move to the inside of the rescale branch (otherwise
+// it is hoisted to the top of every tile and holds 128 VALU registers through the score phase).
+#define PIN_ACC(x) asm volatile("" : "+a"(x))
+
 // NH = heads per wavefront: 2 (32 query rows per workgroup, as described above) for long sequences; 1 (16 rows per workgroup,
 // one head per wavefront: twice the workgroups, LDS-bound) when the launch would otherwise leave CUs idle.
 template <int NH>
@@ -216,7 +221,10 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             for (int hh = 0; hh < NH; hh++) {
                 const f32x4 c4 = *reinterpret_cast<const f32x4*>(&c_s[w][hh][4 * g]);
 #pragma unroll
-                for (int j = 0; j < 16; j++) O[hh][j] *= c4;
+                for (int j = 0; j < 16; j++) {
+                    PIN_ACC(O[hh][j]);
+                    O[hh][j] *= c4;
+                }
             }
         }
         AP_MARK(5);
