@@ -18,6 +18,8 @@
 // the fragment reads of 16 rows on distinct banks.
 #include "qt_common.h"
 
+#include <type_traits>
+
 using namespace qt;
 
 namespace {
@@ -55,6 +57,17 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// max over the four lanes n, n + 16, n + 32, n + 48 with the VALU lane swaps of gfx950 (v_permlane32_swap exchanges the upper half
+// of one register with the lower half of the other, v_permlane16_swap the odd 16-lane rows of one with the even rows of the
+// other), which keeps the softmax free of LDS traffic
+__device__ __forceinline__ float max_over_groups(float x) {
+    const unsigned xi = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    const unsigned mi = __float_as_uint(fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])));
+    const auto b = __builtin_amdgcn_permlane16_swap(mi, mi, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
 // The output accumulators live in the accumulation half of the register file, which MFMA reads and writes in place; only the
 // rare rescale moves them through VALU registers.  The empty asm ties that move to the inside of the rescale branch (otherwise
 // it is hoisted to the top of every tile and holds 128 VALU registers through the score phase).
@@ -66,8 +79,12 @@ template <int NH>
 __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
                                                            const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
                                                            int q_pos0, long q_head_stride, long kv_head_stride) {
-    __shared__ __align__(1024) bf16_t k_s[2][TILE];
-    __shared__ __align__(1024) bf16_t v_s[2][TILE];
+    // four separate arrays, not [2][TILE]: the compiler tracks outstanding direct-to-LDS loads per LDS variable, so a read of
+    // one buffer does not wait for the loads in flight to the others
+    __shared__ __align__(1024) bf16_t k_s0[TILE];
+    __shared__ __align__(1024) bf16_t k_s1[TILE];
+    __shared__ __align__(1024) bf16_t v_s0[TILE];
+    __shared__ __align__(1024) bf16_t v_s1[TILE];
     __shared__ __align__(16) float c_s[4][2][16];
     constexpr int RB = 16 * NH;
     const int rb = gridDim.x - 1 - blockIdx.x;                   // long rows first
@@ -101,24 +118,26 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     const char* vg = reinterpret_cast<const char*>(V + (size_t)kvh * kv_head_stride);
     // byte offset of load 0 within a tile; load i differs by XOR with 1056 i (row bits 10..12, chunk bits 5..7)
     const unsigned ld_off0 = (unsigned)(16 * w + (lane >> 5)) * (AD * 2) + ((unsigned)((lane & 31) ^ (lane >> 5)) << 4);
-    auto load_tile = [&](int t, int buf) {
-        const bool whole = t * KT + KT <= L;                     // else: rows past the end repeat the last key; they are masked
-        const char* kt_g = kg + (size_t)t * (KT * AD * 2);
-        const char* vt_g = vg + (size_t)t * (KT * AD * 2);
+    auto load_rows = [&](const char* src, bf16_t* dst, int t) {  // one K or V tile: this wavefront's eight direct loads
+        const char* tg = src + (size_t)t * (KT * AD * 2);
         unsigned off0 = ld_off0;
         asm volatile("" : "+v"(off0));                           // recompute the eight offsets per tile (one XOR each) rather than
                                                                  // keeping them in registers the accumulators need
+        if (t * KT + KT <= L) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            unsigned off = off0 ^ (1056u * i);
-            if (!whole) off = (unsigned)min((int)(off >> 9), L - 1 - t * KT) * (AD * 2) + (off & 511u);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kt_g + off),
-                                             (__attribute__((address_space(3))) void*)(&k_s[buf][(8 * w + i) * 512]), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vt_g + off),
-                                             (__attribute__((address_space(3))) void*)(&v_s[buf][(8 * w + i) * 512]), 16, 0, 0);
+            for (int i = 0; i < 8; i++)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(tg + (off0 ^ (1056u * i))),
+                                                 (__attribute__((address_space(3))) void*)(dst + (8 * w + i) * 512), 16, 0, 0);
+        } else {                                                 // rows past the end repeat the last key; they are masked
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const unsigned o = off0 ^ (1056u * i);
+                const unsigned off = (unsigned)min((int)(o >> 9), L - 1 - t * KT) * (AD * 2) + (o & 511u);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(tg + off),
+                                                 (__attribute__((address_space(3))) void*)(dst + (8 * w + i) * 512), 16, 0, 0);
+            }
         }
     };
-    load_tile(0, 0);
 
     float m_run[NH], l_run[NH];
     f32x4 O[NH][16];
@@ -135,32 +154,22 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     const int vrow = 4 * g + (n >> 2);                           // row within a 16-key block = its swizzle
     const int va_row = vrow * AD + 4 * (n & 1), vc0 = (n & 3) >> 1;
 
-    AP_INIT();
-    for (int t = 0; t < ntiles; t++) {
-        const int buf = t & 1;
-        AP_MARK(0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wavefront's part of tile t has landed in LDS
-        AP_MARK(1);
-        __syncthreads();                                         // ... and everyone's; everyone is done with tile t - 1
-        if (t + 1 < ntiles) load_tile(t + 1, buf ^ 1);           // in flight during the whole of this tile's arithmetic
-        AP_MARK(2);
-        const bf16_t* ka = &k_s[buf][ka_row];
-        const bf16_t* va = &v_s[buf][va_row];
-        if (t >= ntiles_w) continue;                             // wavefront-uniform: the upper row block may see one tile more
-
-        // scores: each K fragment multiplies the Q^T of both heads (the compiler overlaps the next sub-tile's LDS reads with
-        // these MFMAs as registers allow)
-        f32x4 acc[NH][4];
+    // K fragment kb of sub-tile kt
+    auto k_frag = [&](const bf16_t* ka, int kt, int kb) {
+        return *reinterpret_cast<const bf16x8*>(ka + 16 * kt * AD + (((4 * kb + g) ^ n) << 3));
+    };
+    // scores of tile 0, S^T = K_tile . Q^T: each K fragment multiplies the Q^T of both heads; the fragments of the next
+    // 16-key sub-tile are read while the MFMAs of the current one run
+    auto scores_first = [&](const bf16_t* ka, f32x4 (&acc)[NH][4]) {
         bf16x8 Af[2][8];
 #pragma unroll
-        for (int kb = 0; kb < 8; kb++) Af[0][kb] = *reinterpret_cast<const bf16x8*>(ka + (((4 * kb + g) ^ n) << 3));
+        for (int kb = 0; kb < 8; kb++) Af[0][kb] = k_frag(ka, 0, kb);
 #pragma unroll
         for (int kt = 0; kt < 4; kt++) {
             __builtin_amdgcn_sched_barrier(0);
             if (kt < 3) {
 #pragma unroll
-                for (int kb = 0; kb < 8; kb++)
-                    Af[(kt + 1) & 1][kb] = *reinterpret_cast<const bf16x8*>(ka + 16 * (kt + 1) * AD + (((4 * kb + g) ^ n) << 3));
+                for (int kb = 0; kb < 8; kb++) Af[(kt + 1) & 1][kb] = k_frag(ka, kt + 1, kb);
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -172,10 +181,35 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                     acc[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kt & 1][kb], bq[hh][kb], acc[hh][kt], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        AP_MARK(3);
-        // softmax in base 2 on the raw products: p = 2^(c s - m), c = 256^-0.5 log2 e; only tiles that touch the diagonal or
-        // the end of the sequence need the mask (wavefront-uniform); every row sees key 0, so its maximum is finite from the
-        // first tile on and masked entries come out as 2^-huge = 0
+    };
+
+    f32x4 accs[2][NH][4];                                        // scores of tile t live in accs[t & 1]
+    AP_INIT();
+    // One tile, software-pipelined around ONE workgroup barrier X(t):
+    //     before X(t): the scores of tile t are in registers (computed during tile t - 1), P.V of tile t - 1 is done
+    //     at X(t):     K(t + 1) and V(t) have landed; K(t)'s buffer takes K(t + 2), V(t - 1)'s buffer takes V(t + 1)
+    //     after X(t):  the score MFMAs of tile t + 1 are interleaved, step by step, with the softmax VALU work of tile t
+    //                  (online softmax in base 2 on the raw products: p = 2^(c s - m), c = 256^-0.5 log2 e; every row sees
+    //                  key 0, so its maximum is finite from the first tile on and masked entries come out as 2^-huge = 0);
+    //                  then P.V(t)
+    // PAR = t & 1 picks the buffers at compile time.
+    auto tile = [&](const int t, auto par) {
+        constexpr int PAR = decltype(par)::value;
+        f32x4 (&acc)[NH][4] = accs[PAR];
+        f32x4 (&acc_next)[NH][4] = accs[PAR ^ 1];
+        bf16_t* const k_cur = PAR ? k_s1 : k_s0;                 // K(t): consumed already, refilled with K(t + 2)
+        const bf16_t* const k_nxt = PAR ? k_s0 : k_s1;           // K(t + 1)
+        const bf16_t* const v_cur = PAR ? v_s1 : v_s0;           // V(t)
+        bf16_t* const v_nxt = PAR ? v_s0 : v_s1;                 // V(t - 1): consumed, refilled with V(t + 1)
+        AP_MARK(0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wavefront's loads of K(t + 1), V(t) have landed in LDS
+        AP_MARK(1);
+        __syncthreads();                                         // X(t)
+        if (t + 2 < ntiles) load_rows(kg, k_cur, t + 2);
+        if (t + 1 < ntiles) load_rows(vg, v_nxt, t + 1);
+        AP_MARK(2);
+        if (t >= ntiles_w) return;                               // wavefront-uniform: the upper row block may see one tile more
+        // only tiles that touch the diagonal or the end of the sequence need the mask (wavefront-uniform)
         if (t * KT + KT - 1 > q_pos0 + r0 || t * KT + KT > L) {
 #pragma unroll
             for (int hh = 0; hh < NH; hh++)
@@ -187,33 +221,86 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                         if (!(key <= my_last && key < L)) acc[hh][kt][i] = NEG;
                     }
         }
+        const bf16_t* ka = k_nxt + ka_row;
+        const bf16_t* va = v_cur + va_row;
+        auto v_frag = [&](int j, int q4) {
+            return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * AD + (((2 * j + vc0) ^ vrow) << 3))));
+        };
+        const bool more = t + 1 < ntiles_w;                      // wavefront-uniform
         s16x8 P[NH][2];
+        s16x4 Bf[3][4];
         bool rescale = false;
+        auto body = [&](auto with_scores) {
+            constexpr bool SC = decltype(with_scores)::value;
+            bf16x8 Af[2][8];
+            if (SC) {
 #pragma unroll
-        for (int hh = 0; hh < NH; hh++) {
-            float mx = NEG;
+                for (int kb = 0; kb < 8; kb++) Af[0][kb] = k_frag(ka, 0, kb);
+            }
+            float m_new[NH], ps[NH];
 #pragma unroll
-            for (int kt = 0; kt < 4; kt++)
+            for (int hh = 0; hh < NH; hh++) {
+                float mx = NEG;
 #pragma unroll
-                for (int i = 0; i < 4; i++) mx = fmaxf(mx, acc[hh][kt][i]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run[hh], mx * SCALE_LOG2E);
-            const float corr = __builtin_amdgcn_exp2f(m_run[hh] - m_new);      // m_run = NEG initially: 2^-huge = 0
-            float ps = 0.f;
+                for (int kt = 0; kt < 4; kt++)
 #pragma unroll
-            for (int kt = 0; kt < 4; kt++)
+                    for (int i = 0; i < 4; i++) mx = fmaxf(mx, acc[hh][kt][i]);
+                mx = max_over_groups(mx);
+                m_new[hh] = fmaxf(m_run[hh], mx * SCALE_LOG2E);
+                const float corr = __builtin_amdgcn_exp2f(m_run[hh] - m_new[hh]);   // m_run = NEG initially: 2^-huge = 0
+                l_run[hh] *= corr;                               // this lane's share; summed over g at the end
+                m_run[hh] = m_new[hh];
+                c_s[w][hh][n] = corr;                            // all four groups store the same value: no divergent branch
+                rescale |= corr != 1.0f;
+                ps[hh] = 0.f;
+            }
+            // 32 steps: two score MFMAs of tile t + 1 (one K fragment x both heads) and one softmax element of tile t
+            float pv_prev = 0.f;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt][i], SCALE_LOG2E, -m_new));
-                    ps += pv;
-                    P[hh][kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(pv);
+            for (int st = 0; st < 32; st++) {
+                const int kt = st >> 3, kb = st & 7;
+                __builtin_amdgcn_sched_barrier(0);
+                if (SC) {
+                    if (kt < 3) Af[(kt + 1) & 1][kb] = k_frag(ka, kt + 1, kb);
+                    if (st >= 30) {                              // the first V fragments of P.V ride along with the last steps
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; q4++) Bf[st - 30][q4] = v_frag(st - 30, q4);
+                    }
+#pragma unroll
+                    for (int hh = 0; hh < NH; hh++)
+                        acc_next[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            Af[kt & 1][kb], bq[hh][kb], kb == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc_next[hh][kt], 0, 0, 0);
                 }
-            l_run[hh] = l_run[hh] * corr + ps;                   // this lane's share; summed over g at the end
-            m_run[hh] = m_new;
-            if (g == 0) c_s[w][hh][n] = corr;
-            rescale |= corr != 1.0f;
-        }
+                // softmax elements: NH * 16 of them over the 32 steps
+#pragma unroll
+                for (int e = (NH * 16 * st) / 32; e < (NH * 16 * (st + 1)) / 32; e++) {
+                    const int hh = e >> 4, kt2 = (e >> 2) & 3, i = e & 3;
+                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_new[hh]));
+                    ps[hh] += pv;
+                    if (i & 1) {
+                        const uint32_t pk = pack_bf(pv_prev, pv);
+                        P[hh][kt2 >> 1][(kt2 & 1) * 4 + i - 1] = (short)(pk & 0xffff);
+                        P[hh][kt2 >> 1][(kt2 & 1) * 4 + i] = (short)(pk >> 16);
+                    }
+                    pv_prev = pv;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int hh = 0; hh < NH; hh++) l_run[hh] += ps[hh];
+            if (!SC) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    Bf[0][q4] = v_frag(0, q4);
+                    Bf[1][q4] = v_frag(1, q4);
+                }
+            }
+        };
+        if (more)
+            body(std::true_type{});
+        else
+            body(std::false_type{});
         wave_lds_sync();
         AP_MARK(4);
         if (__any(rescale)) {                                    // wavefront-uniform: most tiles leave every row's max alone
@@ -230,16 +317,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         AP_MARK(5);
         // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs and serve
         // both heads
-        auto v_frag = [&](int j, int q4) {
-            return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * AD + (((2 * j + vc0) ^ vrow) << 3))));
-        };
-        s16x4 Bf[3][4];
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) {
-            Bf[0][q4] = v_frag(0, q4);
-            Bf[1][q4] = v_frag(1, q4);
-        }
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             __builtin_amdgcn_sched_barrier(0);
@@ -260,6 +337,17 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         __builtin_amdgcn_sched_barrier(0);
         AP_MARK(6);
         wave_lds_sync();                                         // c_s is rewritten by the next tile
+    };
+
+    load_rows(kg, k_s0, 0);
+    load_rows(vg, v_s0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (ntiles > 1) load_rows(kg, k_s1, 1);
+    if (ntiles_w > 0) scores_first(k_s0 + ka_row, accs[0]);
+    for (int t = 0; t < ntiles; t += 2) {
+        tile(t, std::integral_constant<int, 0>{});
+        if (t + 1 < ntiles) tile(t + 1, std::integral_constant<int, 1>{});
     }
     // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n
 #pragma unroll
