@@ -32,6 +32,7 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr float SCALE_LOG2E = 0.0625f * 1.4426950408889634f;   // 256^-0.5 log2 e: scores are exponentiated in base 2
 constexpr float NEG = -3.0e38f;
+constexpr float LAZY = 8.0f;            // log2 of the growth of a row maximum that is tolerated before the row is rescaled
 constexpr int KT = 64;                 // keys per tile
 constexpr int TILE = KT * AD;          // elements of one K or V tile in LDS (32 KiB), rows unpadded, chunks swizzled
 
@@ -113,40 +114,46 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     }
     // tile loader: wavefront w issues direct-to-LDS loads i = 0..7 of K and of V; load 8 w + i fills rows 2 (8 w + i) and
     // + 1 (one KiB): lane l lands at chunk position l & 31 of row 2 (8 w + i) + (l >> 5) and fetches chunk (l & 31) ^ (row & 15).
-    // The per-lane byte offsets within a tile do not change from tile to tile; only the last tile of a sequence clamps rows.
+    // The per-lane byte offsets within a tile do not change from tile to tile.  A tile that would run past the end of the
+    // sequence is shifted back to end at L (tile_row0): its first rows repeat keys of the tile before and are masked.  Only a
+    // sequence shorter than one tile repeats its last key instead (slow path, first tile only).
     const char* kg = reinterpret_cast<const char*>(K + (size_t)kvh * kv_head_stride);
     const char* vg = reinterpret_cast<const char*>(V + (size_t)kvh * kv_head_stride);
     // byte offset of load 0 within a tile; load i differs by XOR with 1056 i (row bits 10..12, chunk bits 5..7)
     const unsigned ld_off0 = (unsigned)(16 * w + (lane >> 5)) * (AD * 2) + ((unsigned)((lane & 31) ^ (lane >> 5)) << 4);
-    auto load_rows = [&](const char* src, bf16_t* dst, int t) {  // one K or V tile: this wavefront's eight direct loads
-        const char* tg = src + (size_t)t * (KT * AD * 2);
+    auto tile_row0 = [&](int t) { return max(0, min(t * KT, L - KT)); };
+    auto load_one = [&](const char* src, bf16_t* dst, int t, int i) {        // load i of tile t (L >= KT)
         unsigned off0 = ld_off0;
-        asm volatile("" : "+v"(off0));                           // recompute the eight offsets per tile (one XOR each) rather than
-                                                                 // keeping them in registers the accumulators need
-        if (t * KT + KT <= L) {
+        asm volatile("" : "+v"(off0));                           // recompute the offset (one XOR) rather than keeping eight of
+                                                                 // them in registers the accumulators need
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(src + (size_t)tile_row0(t) * (AD * 2) + (off0 ^ (1056u * i))),
+            (__attribute__((address_space(3))) void*)(dst + (8 * w + i) * 512), 16, 0, 0);
+    };
+    auto load_rows = [&](const char* src, bf16_t* dst, int t) {  // one K or V tile: this wavefront's eight direct loads
+        if (L >= KT) {
 #pragma unroll
-            for (int i = 0; i < 8; i++)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(tg + (off0 ^ (1056u * i))),
-                                                 (__attribute__((address_space(3))) void*)(dst + (8 * w + i) * 512), 16, 0, 0);
-        } else {                                                 // rows past the end repeat the last key; they are masked
+            for (int i = 0; i < 8; i++) load_one(src, dst, t, i);
+        } else {                                                 // t = 0: rows past the end repeat the last key; they are masked
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const unsigned o = off0 ^ (1056u * i);
-                const unsigned off = (unsigned)min((int)(o >> 9), L - 1 - t * KT) * (AD * 2) + (o & 511u);
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(tg + off),
+                const unsigned o = ld_off0 ^ (1056u * i);
+                const unsigned off = (unsigned)min((int)(o >> 9), L - 1) * (AD * 2) + (o & 511u);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + off),
                                                  (__attribute__((address_space(3))) void*)(dst + (8 * w + i) * 512), 16, 0, 0);
             }
         }
     };
 
-    float m_run[NH], l_run[NH];
+    float m_run[NH];
+    f32x4 Lsum[NH];                                              // row sums of P, accumulated by MFMA against a block of ones
     f32x4 O[NH][16];
 #pragma unroll
     for (int hh = 0; hh < NH; hh++)
 #pragma unroll
         for (int j = 0; j < 16; j++) O[hh][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int hh = 0; hh < NH; hh++) m_run[hh] = NEG, l_run[hh] = 0.f;
+    for (int hh = 0; hh < NH; hh++) m_run[hh] = NEG, Lsum[hh] = f32x4{0.f, 0.f, 0.f, 0.f};
     // A operand of the scores: row 16 kt + n of the tile, chunk (4 kb + g) ^ n
     const int ka_row = n * AD;
     // transposing load: within 16 lanes, lane 4q + i receives element i of the 8-byte chunks addressed by lanes q, q+4,
@@ -205,8 +212,15 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wavefront's loads of K(t + 1), V(t) have landed in LDS
         AP_MARK(1);
         __syncthreads();                                         // X(t)
-        if (t + 2 < ntiles) load_rows(kg, k_cur, t + 2);
-        if (t + 1 < ntiles) load_rows(vg, v_nxt, t + 1);
+        // While scores of a further tile are due (then L > KT), this wavefront's 16 loads of K(t + 2) and V(t + 1) are spread
+        // over the steps below: a burst would stall on the memory pipeline's queue.  There a tile index past the end loads the
+        // last tile again, harmlessly: nothing reads that buffer any more.
+        const bool more = t + 1 < ntiles_w;                      // wavefront-uniform
+        const int tk = min(t + 2, ntiles - 1), tv = min(t + 1, ntiles - 1);
+        if (!more) {
+            if (t + 2 < ntiles) load_rows(kg, k_cur, t + 2);
+            if (t + 1 < ntiles) load_rows(vg, v_nxt, t + 1);
+        }
         AP_MARK(2);
         if (t >= ntiles_w) return;                               // wavefront-uniform: the upper row block may see one tile more
         // only tiles that touch the diagonal or the end of the sequence need the mask (wavefront-uniform)
@@ -217,8 +231,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 for (int kt = 0; kt < 4; kt++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const int key = t * KT + 16 * kt + 4 * g + i;
-                        if (!(key <= my_last && key < L)) acc[hh][kt][i] = NEG;
+                        const int key = tile_row0(t) + 16 * kt + 4 * g + i;     // a shifted tile repeats keys below t * KT
+                        if (!(key >= t * KT && key <= my_last && key < L)) acc[hh][kt][i] = NEG;
                     }
         }
         const bf16_t* ka = k_nxt + ka_row;
@@ -227,7 +241,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                 (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * AD + (((2 * j + vc0) ^ vrow) << 3))));
         };
-        const bool more = t + 1 < ntiles_w;                      // wavefront-uniform
         s16x8 P[NH][2];
         s16x4 Bf[3][4];
         bool rescale = false;
@@ -238,7 +251,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
 #pragma unroll
                 for (int kb = 0; kb < 8; kb++) Af[0][kb] = k_frag(ka, 0, kb);
             }
-            float m_new[NH], ps[NH];
+            float m_new[NH];
 #pragma unroll
             for (int hh = 0; hh < NH; hh++) {
                 float mx = NEG;
@@ -247,13 +260,14 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
 #pragma unroll
                     for (int i = 0; i < 4; i++) mx = fmaxf(mx, acc[hh][kt][i]);
                 mx = max_over_groups(mx);
-                m_new[hh] = fmaxf(m_run[hh], mx * SCALE_LOG2E);
+                // the reference point of a row only moves when its maximum has grown by more than 2^LAZY: until then p stays
+                // below 2^LAZY, which bf16 and the f32 sums hold as well as values below 1, and the accumulators are left alone
+                mx *= SCALE_LOG2E;
+                m_new[hh] = mx > m_run[hh] + LAZY ? mx : m_run[hh];
                 const float corr = __builtin_amdgcn_exp2f(m_run[hh] - m_new[hh]);   // m_run = NEG initially: 2^-huge = 0
-                l_run[hh] *= corr;                               // this lane's share; summed over g at the end
                 m_run[hh] = m_new[hh];
                 c_s[w][hh][n] = corr;                            // all four groups store the same value: no divergent branch
                 rescale |= corr != 1.0f;
-                ps[hh] = 0.f;
             }
             // 32 steps: two score MFMAs of tile t + 1 (one K fragment x both heads) and one softmax element of tile t
             float pv_prev = 0.f;
@@ -261,6 +275,12 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             for (int st = 0; st < 32; st++) {
                 const int kt = st >> 3, kb = st & 7;
                 __builtin_amdgcn_sched_barrier(0);
+                if (SC && (st & 1) == 0) {
+                    if (st < 16)
+                        load_one(kg, k_cur, tk, st >> 1);
+                    else
+                        load_one(vg, v_nxt, tv, (st >> 1) - 8);
+                }
                 if (SC) {
                     if (kt < 3) Af[(kt + 1) & 1][kb] = k_frag(ka, kt + 1, kb);
                     if (st >= 30) {                              // the first V fragments of P.V ride along with the last steps
@@ -277,7 +297,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 for (int e = (NH * 16 * st) / 32; e < (NH * 16 * (st + 1)) / 32; e++) {
                     const int hh = e >> 4, kt2 = (e >> 2) & 3, i = e & 3;
                     const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_new[hh]));
-                    ps[hh] += pv;
                     if (i & 1) {
                         const uint32_t pk = pack_bf(pv_prev, pv);
                         P[hh][kt2 >> 1][(kt2 & 1) * 4 + i - 1] = (short)(pk & 0xffff);
@@ -287,8 +306,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int hh = 0; hh < NH; hh++) l_run[hh] += ps[hh];
             if (!SC) {
 #pragma unroll
                 for (int q4 = 0; q4 < 4; q4++) {
@@ -312,11 +329,24 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                     PIN_ACC(O[hh][j]);
                     O[hh][j] *= c4;
                 }
+                PIN_ACC(Lsum[hh]);
+                Lsum[hh] *= c4;
             }
         }
         AP_MARK(5);
         // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs and serve
-        // both heads
+        // both heads; the row sums are one more column block, P . 1 (the sum of exactly the rounded values that multiply V)
+        {
+            s16x8 ones;
+#pragma unroll
+            for (int e = 0; e < 8; e++) ones[e] = (short)0x3f80;
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++)
+#pragma unroll
+                for (int hh = 0; hh < NH; hh++)
+                    Lsum[hh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[hh][pp]),
+                                                                      __builtin_bit_cast(bf16x8, ones), Lsum[hh], 0, 0, 0);
+        }
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             __builtin_amdgcn_sched_barrier(0);
@@ -349,23 +379,14 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         tile(t, std::integral_constant<int, 0>{});
         if (t + 1 < ntiles) tile(t + 1, std::integral_constant<int, 1>{});
     }
-    // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n
+    // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n, and of the row sums (any column)
 #pragma unroll
     for (int hh = 0; hh < NH; hh++) {
-        float l = l_run[hh];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
-        if (g == 0) c_s[w][hh][n] = l;
-    }
-    wave_lds_sync();
-#pragma unroll
-    for (int hh = 0; hh < NH; hh++) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&c_s[w][hh][4 * g]);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int orow = r0 + 4 * g + r;
             if (orow < S) {
-                const float inv = 1.0f / l4[r];
+                const float inv = 1.0f / Lsum[hh][r];
                 bf16_t* dst = out + (size_t)(h0 + hh) * q_head_stride + (size_t)orow * AD + n;
 #pragma unroll
                 for (int j = 0; j < 16; j++) dst[16 * j] = f2bf(O[hh][j][r] * inv);
