@@ -36,20 +36,29 @@ constexpr float LAZY = 8.0f;            // log2 of the growth of a row maximum t
 constexpr int KT = 64;                 // keys per tile
 constexpr int TILE = KT * AD;          // elements of one K or V tile in LDS (32 KiB), rows unpadded, chunks swizzled
 
-// AP_MARK(i): per-tile phase time stamps for profiling builds (QT_ATTN_PREFILL_PROF defines ap_prof_buf[workgroup][wave][8],
-// accumulated shader-clock ticks per phase); compiles to nothing otherwise
+// AP_MARK(i): phase time stamps for profiling builds (QT_ATTN_PREFILL_PROF defines ap_prof_buf[workgroup][wave][8]: shader-clock
+// ticks per phase, summed over the tiles in scalar registers and stored once at the end); otherwise only a scheduling fence
 #ifdef QT_ATTN_PREFILL_PROF
 __device__ long long* ap_prof_buf;
-#define AP_MARK(i)                                                                                              \
-    do {                                                                                                        \
-        const long long now_ = clock64();                                                                       \
-        if ((threadIdx.x & 63) == 0) ap_prof_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6)) * 8 + (i)] += now_ - ap_last_; \
-        ap_last_ = now_;                                                                                        \
+#define AP_MARK(i)                                  \
+    do {                                            \
+        const long long now_ = clock64();           \
+        ap_acc_[i] += now_ - ap_last_;              \
+        ap_last_ = now_;                            \
     } while (0)
-#define AP_INIT() long long ap_last_ = clock64()
+#define AP_INIT()                                   \
+    long long ap_acc_[8] = {0, 0, 0, 0, 0, 0, 0, 0}; \
+    long long ap_last_ = clock64()
+#define AP_STORE()                                                                                              \
+    do {                                                                                                        \
+        if ((threadIdx.x & 63) == 0)                                                                            \
+            for (int i_ = 0; i_ < 8; i_++)                                                                      \
+                ap_prof_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6)) * 8 + i_] = ap_acc_[i_]; \
+    } while (0)
 #else
 #define AP_MARK(i) __builtin_amdgcn_sched_barrier(0)     /* the phases of a tile are scheduled separately */
 #define AP_INIT()
+#define AP_STORE()
 #endif
 
 __device__ __forceinline__ void wave_lds_sync() {
@@ -269,6 +278,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 c_s[w][hh][n] = corr;                            // all four groups store the same value: no divergent branch
                 rescale |= corr != 1.0f;
             }
+            AP_MARK(3);
             // 32 steps: two score MFMAs of tile t + 1 (one K fragment x both heads) and one softmax element of tile t
             float pv_prev = 0.f;
 #pragma unroll
@@ -379,6 +389,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         tile(t, std::integral_constant<int, 0>{});
         if (t + 1 < ntiles) tile(t + 1, std::integral_constant<int, 1>{});
     }
+    AP_STORE();
     // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n, and of the row sums (any column)
 #pragma unroll
     for (int hh = 0; hh < NH; hh++) {
