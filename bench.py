@@ -253,6 +253,35 @@ def bench_attn_glue(torch, qt, dev, R=2048, seed=5):
     return {"rows": R, "qkv_prep_us": t1 * 1e6, "qkv_prep_GBps": b1 / t1 / 1e9, "out_gate_us": t2 * 1e6, "out_gate_GBps": b2 / t2 / 1e9}
 
 
+def bench_projections(torch, qt, dev, B=64, seed=9):
+    """The projections either side of the GDN core at a decode step of B rows (hidden 1024): rms_rows + in_proj [8224 x 1024],
+    and out_proj [1024 x 2048] with the residual (qwen35/batch.py:496-501); eight copies of each weight rotate so that no copy
+    stays in the last-level cache between uses less than the layer count apart."""
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    Wi = [(torch.randn((PW, 1024), generator=g) / 32).to(bf).to(dev) for _ in range(8)]
+    Wo = [(torch.randn((1024, 2048), generator=g) / 45).to(bf).to(dev) for _ in range(8)]
+    x = torch.randn((B, 1024), generator=g).to(bf).to(dev)
+    ln = torch.ones(1024, dtype=bf, device=dev)
+    yn = torch.randn((B, 2048), generator=g).to(bf).to(dev)
+    it = [0]
+
+    def in_proj():
+        qt.kernels.fused_gemv(Wi[it[0] % 8], qt.batch.rms_rows(x, ln))
+        it[0] += 1
+
+    def out_proj():
+        qt.kernels.fused_gemv(Wo[it[0] % 8], yn, res=x)
+        it[0] += 1
+    t0 = time_graph(torch, lambda: qt.batch.rms_rows(x, ln), reps=40, inner=8)
+    t1 = time_graph(torch, in_proj, reps=40, inner=8)
+    t2 = time_graph(torch, out_proj, reps=40, inner=8)
+    b1 = PW * 1024 * 2 + B * (1024 * 2 * 3 + PW * 2)
+    b2 = 1024 * 2048 * 2 + B * (2048 * 2 + 1024 * 2 * 2)
+    return {"B": B, "rms_rows_us": t0 * 1e6, "rms_in_proj_us": t1 * 1e6, "rms_in_proj_GBps": b1 / t1 / 1e9,
+            "out_proj_add_us": t2 * 1e6, "out_proj_add_GBps": b2 / t2 / 1e9}
+
+
 def cpu_baseline(B, budget_s=12.0):
     """The C restatement of the decode step (float accumulation) timed on this host's cores: a reported baseline only."""
     import numpy as np
@@ -307,6 +336,8 @@ def profile_leg(torch, qt, dev, args):
         bench_attn(torch, qt, dev, 16, 4, 1024, 8192, 1004)
     elif leg == "attn_prefill":
         bench_attn_prefill(torch, qt, dev)
+    elif leg == "projections":
+        bench_projections(torch, qt, dev)
     elif leg == "attn_prefill_long":
         bench_attn_prefill(torch, qt, dev, 8192)
     else:
@@ -337,7 +368,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the B sweep and the single-pool run")
     ap.add_argument("--only", default="", help="profile helper: run only one leg a few times and exit "
-                                               "(decode | copy | prefill | verify | attn_decode | attn_verify | attn_prefill | attn_prefill_long)")
+                                               "(decode | copy | prefill | verify | attn_decode | attn_verify | attn_prefill | attn_prefill_long | projections)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every work item of the path is an independent (slot, head) pair; "
@@ -404,6 +435,7 @@ def main():
         extras["attn_prefill_causal"] = [bench_attn_prefill(torch, qt, dev, S) for S in (2048, 8192)]
         extras["state_admission"] = bench_state_admission(torch, qt, dev)
         extras["attn_glue"] = bench_attn_glue(torch, qt, dev)
+        extras["gdn_layer_projections"] = bench_projections(torch, qt, dev)
 
     out = {
         "metric": "GDN decode steps/s @B=64 (% HBM peak); GDN prefill tok/s @2048 (% MFMA)",

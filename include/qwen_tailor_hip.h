@@ -136,6 +136,17 @@ int qt_attn_qkv_prep(const void* qkv, const void* q_norm, const void* k_norm, co
                      int M, float eps, qt_stream_t stream);
 int qt_attn_out_gate(const void* o, const void* qkv, void* out, long R, qt_stream_t stream);
 
+/* The projections either side of the core at decode / verify time: the reference's fused_gemv (qwen35/kernels.py:80-319) on
+ * plain bf16 weights and its stand-alone prologue rms_rows (qwen35/batch.py:249-301).
+ * qt_rms_rows: y [M,K] bf16 = BF(nw * (x * rsqrt(mean(x^2) + eps))), x [M,K] bf16, nw [K] bf16; K a multiple of 8.
+ * qt_fused_gemv: s = x [M,K] . W [N,K]^T accumulated in fp32 (bf16 MFMA), then epilogue
+ *     0: y [M,N] = bf16(s)        1: y [M,N] = bf16(BF(s) + res [M,N])
+ *     2: y [M,N/2], y[m][p] = bf16(silu_bf16(BF(s[m][2p])) * BF(s[m][2p+1]))   (interleaved gate / up rows, N even)
+ * K a multiple of 256.  The gated-norm prologue of the reference is qt_gated_rmsnorm applied to x first; the rms prologue is
+ * qt_rms_rows: both round to bf16 before the product, exactly as the fused forms do. */
+int qt_rms_rows(const void* x, const void* nw, void* y, int M, int K, float eps, qt_stream_t stream);
+int qt_fused_gemv(const void* W, const void* x, const void* res, void* y, int M, int N, int K, int epilogue, qt_stream_t stream);
+
 /* batch.blit (qwen35/batch.py:365-372), the in-place strided copy behind Pools.load / read (batch.py:431-462) and the
  * scheduler's plain <-> speculative state moves (qwen35/serve.py:310-348):
  *     dst.flat[d0 + y*dstride + i] = src.flat[s0 + y*sstride + i]   for i < n, y < ny   (offsets and strides in elements)

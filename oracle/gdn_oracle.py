@@ -436,3 +436,33 @@ def attn_out_gate(o, qkv):
     o = np.asarray(o, np.float32).reshape(-1, 8, 256)
     gate = np.asarray(qkv, np.float32)[:, :4096].reshape(-1, 8, 512)[:, :, 256:]
     return BF((o * sigmoid_bf16(gate)).astype(np.float32)).reshape(-1, 2048)
+
+
+# ------------------------------------------------------------------------------------------------
+# the projections either side of the core (kernels.py:80-319, batch.py:249-301)
+# ------------------------------------------------------------------------------------------------
+def rms_rows(x, nw, eps=1e-6):
+    """The `rms` prologue of fused_gemv / rms_rows (kernels.py:106-131, batch.py:249-294): inv = rsqrt(sum(x^2) / K + eps) with the
+    sum of squares exact, then BF(nw * (x * inv)), each product rounded to float32."""
+    x = np.asarray(x, np.float32)
+    ss = (x.astype(np.float64) ** 2).sum(-1, keepdims=True).astype(np.float32)
+    inv = rsqrt32((ss / F32(x.shape[-1]) + F32(eps)).astype(np.float32))
+    return BF((np.asarray(nw, np.float32) * (x * inv).astype(np.float32)).astype(np.float32))
+
+
+def fused_gemv(W, x, nw=None, eps=1e-6, res=None, swiglu=False, gnorm=None):
+    """y = W @ f(x) (kernels.py:291-319): W [N,K], x [M,K] (bf16 values); prologue rms (nw) or gated norm (gnorm = (proj, gw));
+    the products are accumulated in float64 here (the reference and the kernels accumulate in float32, in different orders);
+    epilogue none: BF(s); add: BF(BF(s) + res) (kernels.py:161-169); swiglu: BF(silu_bf16(BF(s[2p])) * BF(s[2p+1]))
+    (kernels.py:170-182)."""
+    x = np.asarray(x, np.float32)
+    if nw is not None:
+        x = rms_rows(x, nw, eps)
+    if gnorm is not None:
+        x = gated_norm(x, gnorm[0], gnorm[1], eps)
+    s = BF((x.astype(np.float64) @ np.asarray(W, np.float32).astype(np.float64).T).astype(np.float32))
+    if res is not None:
+        return BF((s + np.asarray(res, np.float32)).astype(np.float32))
+    if swiglu:
+        return BF((silu_bf16(s[:, 0::2]) * s[:, 1::2]).astype(np.float32))
+    return s

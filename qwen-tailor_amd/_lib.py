@@ -37,6 +37,8 @@ _SIGS = {
     "qt_attn_qkv_prep": [_vp] * 7 + [_l, _i, _f, _vp],
     "qt_attn_out_gate": [_vp, _vp, _vp, _l, _vp],
     "qt_blit_batch": [_vp, _vp, _vp, _i, _vp],
+    "qt_rms_rows": [_vp, _vp, _vp, _i, _i, _f, _vp],
+    "qt_fused_gemv": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
 }
 
 

@@ -108,6 +108,12 @@ def gnorm_rows(y, proj, gw, eps=1e-6):
     return out
 
 
+def rms_rows(x, nw, eps=1e-6, T=128, f32=False):
+    """qwen35/batch.py:295-301; see kernels.rms_rows."""
+    from .kernels import rms_rows as _rms_rows
+    return _rms_rows(x, nw, eps, T, f32)
+
+
 def blit(dst, src, n, d0, s0, ny=1, dstride=0, sstride=0):
     """dst.flat[d0 + y*dstride + i] = src.flat[s0 + y*sstride + i] for i < n, y < ny, in place (qwen35/batch.py:365-372).
     dst and src are contiguous device tensors of the same dtype (bf16 or float32); returns dst."""

@@ -42,6 +42,10 @@ def test_host_rejects_bad_arguments_without_a_gpu():
         qt.prefill.conv_prep(x, x, x)
     with pytest.raises(TypeError):
         qt.batch.attn_b(x, x, x, x, x, x, x)
+    with pytest.raises(TypeError):
+        qt.kernels.fused_gemv(x, x)
+    with pytest.raises(TypeError):
+        qt.batch.rms_rows(x, x[0])
 
 
 def test_null_and_dimension_errors_from_the_c_abi():
@@ -64,6 +68,14 @@ def test_null_and_dimension_errors_from_the_c_abi():
     assert lib.qt_gdn_phase_a_conv(p16, p16, p16, p16, p16, p16, p16, z, z, z, p16, p16, p16, 64, z) == -3   # q without k, v
     assert lib.qt_gdn_phase_a_conv(p16, p16, p16, p16, p16, p16, z, z, z, p16, p16, p16, p16, 64, z) == -4   # conv_out aliases conv_state
     assert lib.qt_gqa_attn_decode(p16, p16, p16, p16, p16, p16, p16, p16, p16, 1 << 40, 2000, 1, 64, 1, 128, z) == -4   # B * 2 > 2048 segments
+    assert lib.qt_rms_rows(p16, z, p16, 4, 1024, 1e-6, z) == -3
+    assert lib.qt_rms_rows(p16, p16, p16, 4, 1020, 1e-6, z) == -1                    # K must be a multiple of 8
+    assert lib.qt_rms_rows(p16, p16, p16, 0, 1024, 1e-6, z) == 0
+    assert lib.qt_fused_gemv(p16, p16, z, p16, 4, 64, 1024, 1, z) == -3              # the add epilogue needs res
+    assert lib.qt_fused_gemv(p16, p16, z, p16, 4, 64, 1000, 0, z) == -1              # K must be a multiple of 256
+    assert lib.qt_fused_gemv(p16, p16, z, p16, 4, 63, 1024, 2, z) == -1              # swiglu pairs rows
+    assert lib.qt_fused_gemv(p16, p16, z, p16, 4, 64, 1024, 3, z) == -4
+    assert lib.qt_fused_gemv(ctypes.c_void_p(8), p16, z, p16, 4, 64, 1024, 0, z) == -2
 
 
 def test_product_does_not_import_the_oracle():

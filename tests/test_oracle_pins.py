@@ -530,3 +530,57 @@ def test_blit_is_a_strided_copy():
         for i in range(10):
             want[7 + y * 100 + i] = src[3 + y * 50 + i]
     assert np.array_equal(dst, want)
+
+
+# ------------------------------------------------------------------------------------------------
+# the projections either side of the core
+# ------------------------------------------------------------------------------------------------
+def test_rms_rows_vs_torch_and_constant_row():
+    """the rms prologue reduces to torch's rms_norm in float64 up to its single bf16 rounding; a constant row maps to the weight"""
+    rng = np.random.default_rng(5)
+    x = bf(rng.standard_normal((7, 1024)) * 2)
+    w = bf(1 + 0.3 * rng.standard_normal(1024))
+    got = O.rms_rows(x, w, 1e-6)
+    ref = torch.nn.functional.rms_norm(torch.from_numpy(x).double(), (1024,), torch.from_numpy(w).double(), 1e-6).numpy()
+    assert np.all(np.abs(got - ref) <= 0.502 * ulp_bf16(ref) + 1e-30)           # one rounding (plus float32 products)
+    assert np.array_equal(O.rms_rows(np.full((1, 512), -4.0, np.float32), w[:512], 0.0), -w[None, :512])
+
+
+def test_fused_gemv_bruteforce_and_epilogues():
+    """the product by plain loops on a tiny case with small-integer data (every partial sum exact, so no accumulation order
+    matters); the epilogues by their closed forms; the prologues compose with the product"""
+    rng = np.random.default_rng(6)
+    M, N, K = 3, 6, 16
+    W = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    x = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    want = np.zeros((M, N), np.float32)
+    for m in range(M):
+        for n in range(N):
+            s = 0.0
+            for k in range(K):
+                s += float(W[n, k]) * float(x[m, k])
+            want[m, n] = s
+    assert np.array_equal(O.fused_gemv(W, x), want)                              # |s| <= 192: every sum is a bf16 value
+    res = bf(rng.standard_normal((M, N)))
+    assert np.array_equal(O.fused_gemv(W, x, res=res), bf(bf(want) + res))
+    sw = O.fused_gemv(W, x, swiglu=True)
+    g, u = bf(want[:, 0::2]), bf(want[:, 1::2])
+    assert sw.shape == (M, N // 2) and np.array_equal(sw, bf(O.silu_bf16(g) * u))
+    # linearity in W where every value stays exactly representable
+    assert np.array_equal(O.fused_gemv(2 * W, x), 2 * O.fused_gemv(W, x))
+    # the rms prologue is applied to x before the product
+    nw = bf(1 + 0.1 * rng.standard_normal(K))
+    xr = bf(rng.standard_normal((M, K)))
+    assert np.array_equal(O.fused_gemv(W, xr, nw=nw), O.fused_gemv(W, O.rms_rows(xr, nw)))
+    # rounding: a product that needs more than 8 bits rounds to nearest even
+    assert O.fused_gemv(np.array([[257.0]], np.float32), np.array([[1.0]], np.float32))[0, 0] == 256.0
+    assert O.fused_gemv(np.array([[259.0]], np.float32), np.array([[1.0]], np.float32))[0, 0] == 260.0
+
+
+def test_fused_gemv_gnorm_prologue_is_gated_norm():
+    rng = np.random.default_rng(8)
+    y = bf(rng.standard_normal((2, 2048)))
+    proj = bf(rng.standard_normal((2, O.PW)))
+    gw = (1 + 0.1 * rng.standard_normal(128)).astype(np.float32)
+    W = bf(rng.standard_normal((8, 2048)) * 0.05)
+    assert np.array_equal(O.fused_gemv(W, y, gnorm=(proj, gw)), O.fused_gemv(W, O.gated_norm(y, proj, gw)))
