@@ -282,6 +282,28 @@ def bench_projections(torch, qt, dev, B=64, seed=9):
             "out_proj_add_us": t2 * 1e6, "out_proj_add_GBps": b2 / t2 / 1e9}
 
 
+def bench_prefix_cache(torch, qt, dev, pos=2048, max_len=4096):
+    """A prefix-cache checkpoint of a prefilled sequence (qwen35/prefix_cache.py:157-188: 12 K / V segments of `pos` rows + 18
+    recurrent states, one launch) and its restore into fresh max_len buffers (prefix_cache.py:139-154)."""
+    import numpy as np
+    cfg = qt.model.Cfg()
+    nl = sum(cfg.is_linear(i) for i in range(cfg.layers))
+    na = cfg.layers - nl
+    bf = torch.bfloat16
+    st = {"kv": [(torch.zeros((1, cfg.n_kv, max_len, cfg.head_dim), dtype=bf, device=dev),
+                  torch.zeros((1, cfg.n_kv, max_len, cfg.head_dim), dtype=bf, device=dev)) for _ in range(na)],
+          "conv": [torch.zeros((1, 3, CD), dtype=bf, device=dev) for _ in range(nl)],
+          "ssm": [torch.zeros((1, HV, DV, DK), device=dev) for _ in range(nl)]}
+    pc = qt.prefix_cache.PrefixCache(budget_mb=4096)
+    node = pc.insert(None, np.arange(pos, dtype=np.int32), pos, st)
+    t1 = time_graph(torch, lambda: pc._snapshot(st, 0, pos), reps=40, inner=4)
+    t2 = time_graph(torch, lambda: pc.restore(node, max_len), reps=40, inner=4)
+    moved = na * 2 * cfg.n_kv * pos * cfg.head_dim * 2 + nl * (HV * DV * DK * 4 + 3 * CD * 2)
+    pad = na * 2 * cfg.n_kv * (max_len - pos) * cfg.head_dim * 2
+    return {"pos": pos, "max_len": max_len, "checkpoint_us": t1 * 1e6, "checkpoint_GBps": 2 * moved / t1 / 1e9,
+            "restore_us": t2 * 1e6, "restore_GBps": (2 * moved + pad) / t2 / 1e9, "node_bytes": node.nbytes}
+
+
 def cpu_baseline(B, budget_s=12.0):
     """The C restatement of the decode step (float accumulation) timed on this host's cores: a reported baseline only."""
     import numpy as np
@@ -436,6 +458,7 @@ def main():
         extras["state_admission"] = bench_state_admission(torch, qt, dev)
         extras["attn_glue"] = bench_attn_glue(torch, qt, dev)
         extras["gdn_layer_projections"] = bench_projections(torch, qt, dev)
+        extras["prefix_cache"] = bench_prefix_cache(torch, qt, dev)
 
     out = {
         "metric": "GDN decode steps/s @B=64 (% HBM peak); GDN prefill tok/s @2048 (% MFMA)",

@@ -466,3 +466,42 @@ def fused_gemv(W, x, nw=None, eps=1e-6, res=None, swiglu=False, gnorm=None):
     if swiglu:
         return BF((silu_bf16(s[:, 0::2]) * s[:, 1::2]).astype(np.float32))
     return s
+
+
+# ------------------------------------------------------------------------------------------------
+# prefix-cache checkpoints (prefix_cache.py:90-188): the segment format and the lookup rule
+# ------------------------------------------------------------------------------------------------
+def pc_segment(kv_pairs, a, pos):
+    """The K / V segment of a checkpoint (prefix_cache.py:185): rows [a, pos) of every buffer, K and V of a layer interleaved,
+    stacked to [2 * layers, 1, n_kv, pos - a, D]."""
+    return np.stack([np.asarray(x)[:, :, a:pos] for k, v in kv_pairs for x in (k, v)])
+
+
+def pc_restore(segments, max_len):
+    """Fresh K / V buffers from a chain of segments (prefix_cache.py:139-154): buffer j = the chain's rows end to end, zero rows
+    up to max_len.  Returns [(K, V)] per layer, each [1, n_kv, max_len, D]."""
+    nb = segments[0].shape[0]
+    bufs = []
+    for j in range(nb):
+        rows = np.concatenate([s[j] for s in segments], axis=2)
+        pad = np.zeros(rows.shape[:2] + (max_len - rows.shape[2], rows.shape[3]), rows.dtype)
+        bufs.append(np.concatenate([rows, pad], axis=2))
+    return [(bufs[2 * i], bufs[2 * i + 1]) for i in range(nb // 2)]
+
+
+def pc_lookup(nodes, ids, min_split=32, min_gain=32):
+    """The lookup rule (prefix_cache.py:90-125) by plain loops.  nodes: [(toks, has_last)] with pos = len(toks).  Returns (index of
+    the deepest checkpoint that is a prefix of ids or None, split position or 0)."""
+    S = len(ids)
+    best, part = None, 0
+    for i, (toks, has_last) in enumerate(nodes):
+        lcp = 0
+        while lcp < min(len(toks), S) and toks[lcp] == ids[lcp]:
+            lcp += 1
+        if lcp == len(toks):
+            if (len(toks) < S or has_last) and (best is None or len(toks) > len(nodes[best][0])):
+                best = i
+        elif lcp < S:
+            part = max(part, lcp)
+    base = len(nodes[best][0]) if best is not None else 0
+    return best, (part if part >= min_split and part - base >= min_gain else 0)
