@@ -4,18 +4,18 @@
 //
 // One workgroup = 32 query rows x the 4 query heads that share a KV head: wavefront w owns the 16 rows of block w >> 1 for
 // the two heads 2 (w & 1), 2 (w & 1) + 1, so a K / V tile of 64 keys is fetched from HBM once and staged in LDS for all of
-// them, and every K or V fragment a wavefront reads from LDS feeds two MFMAs (one per head): the kernel is bound by MFMA
-// issue and LDS bandwidth in equal parts instead of by LDS bandwidth alone.  Per tile and wavefront:
+// them, and every K or V fragment a wavefront reads from LDS feeds two MFMAs (one per head).  Per tile and wavefront:
 //     S^T[keys x rows] = K_tile . Q^T     A = K rows from LDS, B = Q^T resident in registers (16x16x32 bf16 MFMA)
 //     online softmax in the accumulator layout: lane (row n, group g) holds keys 4g..4g+3 of each 16-key sub-tile
 //     O[rows x 256]   += P . V            A = two exponentiated S^T accumulators packed to bf16 (they ARE the A operand
 //                                         when a 32-key block is enumerated as 16 (j >> 2) + 4 g + (j & 3)),
-//                                         B = V through the transposing LDS load (4 consecutive keys of one column)
+//                                         B = V through the transposing LDS load (4 consecutive keys of one column);
+//                                         the row sums are one more column block, P . 1
 // K / V tiles travel HBM -> LDS directly (global_load_lds_dwordx4: 64 lanes x 16 bytes land as one contiguous KiB, no
-// registers in between) into double-buffered tiles, so the next tile's loads are in flight during the whole of the current
-// tile's arithmetic and a tile costs one workgroup barrier.  The LDS rows are unpadded (a direct load cannot pad); instead the
+// registers in between) into double-buffered tiles.  The LDS rows are unpadded (a direct load cannot pad); instead the
 // 16-byte chunks of row r are stored XOR-swizzled by r & 15 (the loading lane picks the matching global chunk), which keeps
-// the fragment reads of 16 rows on distinct banks.
+// the fragment reads of 16 rows on distinct banks.  The tile loop is software-pipelined around one workgroup barrier per tile:
+// the score MFMAs of tile t + 1 are interleaved step by step with the softmax of tile t (see `tile` below).
 #include "qt_common.h"
 
 #include <type_traits>

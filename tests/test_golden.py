@@ -64,6 +64,12 @@ def test_oracle_reproduces_fixtures():
     check_equal("glue k", k, unbits(z["k"]))
     check_equal("glue v", v, unbits(z["v"]))
     check_equal("glue gate", O.attn_out_gate(unbits(z["o"]), unbits(z["qkv"])), unbits(z["gated"]))
+    z = np.load(os.path.join(G, "projections.npz"))
+    x, nw, W1, Wg = (unbits(z[n]) for n in ("x", "nw", "W1", "Wg"))
+    check_equal("rms_rows", O.rms_rows(x, nw), unbits(z["xn"]))
+    check_equal("gemv rms", O.fused_gemv(W1, x, nw=nw), unbits(z["y_rms"]))
+    check_equal("gemv add", O.fused_gemv(W1, x, res=unbits(z["res"])), unbits(z["y_add"]))
+    check_equal("gemv swiglu", O.fused_gemv(Wg, x, swiglu=True), unbits(z["y_swiglu"]))
 
 
 @pytest.fixture(scope="module")
@@ -123,3 +129,20 @@ def test_attention_glue_matches_fixture(qt, dev):
     check_equal("k", to_np(k), unbits(z["k"]))
     check_equal("v", to_np(v), unbits(z["v"]))
     check_equal("gated output", to_np(qt.attention.out_gate(d("o"), d("qkv"))), unbits(z["gated"]))
+
+
+@pytest.mark.gpu
+def test_projections_match_fixture(qt, dev):
+    """rms_rows bit for bit; the products within one bf16 rounding step (two after the second rounding of add / swiglu) plus the
+    float32 accumulation error of sums that nearly cancel"""
+    z = np.load(os.path.join(G, "projections.npz"))
+    d = lambda name: to_dev(unbits(z[name]), dev, BF16)
+    check_equal("rms_rows", to_np(qt.batch.rms_rows(d("x"), d("nw"))), unbits(z["xn"]))
+
+    def close(name, got, want, ulps):
+        got, want = to_np(got).astype(np.float64), unbits(z[want]).astype(np.float64)
+        bad = np.abs(got - want) > ulps * ulp_bf16(np.maximum(np.abs(got), np.abs(want))) + 2e-5 * np.abs(want).max()
+        assert not bad.any(), f"{name}: {int(bad.sum())} outputs off"
+    close("rms + product", qt.kernels.fused_gemv(d("W1"), d("x"), nw=d("nw")), "y_rms", 1)
+    close("add", qt.kernels.fused_gemv(d("W1"), d("x"), res=d("res")), "y_add", 2)
+    close("swiglu", qt.kernels.fused_gemv(d("Wg"), d("x"), swiglu=True), "y_swiglu", 2)
