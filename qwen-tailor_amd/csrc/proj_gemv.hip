@@ -264,9 +264,9 @@ extern "C" {
 
 // y [M, K] bf16 = rms prologue of x [M, K] bf16 with weight nw [K] bf16.  K a multiple of 8.
 int qt_rms_rows(const void* x, const void* nw, void* y, int M, int K, float eps, hipStream_t stream) {
-    if (!x || !nw || !y) return QT_ERR_NULL;
     if (M < 0 || K < 8 || (K & 7)) return QT_ERR_DIM;
-    if (M == 0) return QT_OK;
+    if (M == 0) return QT_OK;                                     // nothing to do: empty buffers may be null
+    if (!x || !nw || !y) return QT_ERR_NULL;
     for (const void* p : {x, nw, (const void*)y})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     hipLaunchKernelGGL(rms_rows_kernel, dim3((M + 3) / 4), dim3(256), 0, stream, (const bf16_t*)x, (const bf16_t*)nw, (bf16_t*)y, M, K, eps);
@@ -277,10 +277,10 @@ int qt_rms_rows(const void* x, const void* nw, void* y, int M, int K, float eps,
 // y = epilogue(W [N, K] . x [M, K]^T): epilogue 0 none (y [M, N]), 1 add (res [M, N], y [M, N]), 2 swiglu (y [M, N / 2], N even).
 // K a multiple of 256.
 int qt_fused_gemv(const void* W, const void* x, const void* res, void* y, int M, int N, int K, int epilogue, hipStream_t stream) {
-    if (!W || !x || !y || (epilogue == EPI_ADD && !res)) return QT_ERR_NULL;
     if (epilogue < 0 || epilogue > 2) return QT_ERR_UNSUPPORTED;
     if (M < 0 || N < 1 || K < 256 || (K % 256) || (epilogue == EPI_SWIGLU && (N & 1))) return QT_ERR_DIM;
-    if (M == 0) return QT_OK;
+    if (M == 0) return QT_OK;                                     // nothing to do: empty buffers may be null
+    if (!W || !x || !y || (epilogue == EPI_ADD && !res)) return QT_ERR_NULL;
     for (const void* p : {W, x})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     // wavefronts per workgroup: 4 when the output is wide enough to fill the chip with workgroups; 16 or 8 (as K divides) for

@@ -75,6 +75,7 @@ def test_null_and_dimension_errors_from_the_c_abi():
     assert lib.qt_fused_gemv(p16, p16, z, p16, 4, 64, 1000, 0, z) == -1              # K must be a multiple of 256
     assert lib.qt_fused_gemv(p16, p16, z, p16, 4, 63, 1024, 2, z) == -1              # swiglu pairs rows
     assert lib.qt_fused_gemv(p16, p16, z, p16, 4, 64, 1024, 3, z) == -4
+    assert lib.qt_fused_gemv(p16, z, z, z, 0, 64, 1024, 1, z) == 0                   # no rows: nothing is dereferenced
     assert lib.qt_fused_gemv(ctypes.c_void_p(8), p16, z, p16, 4, 64, 1024, 0, z) == -2
 
 

@@ -123,7 +123,8 @@ def test_attn_b_config4_verify_mix(qt, dev):
 
 
 # ------------------------------------------------------------------------------------- causal prefill attention
-@pytest.mark.parametrize("S,L", [(1, 1), (5, 5), (64, 64), (100, 100), (37, 200), (300, 300), (128, 1000)])
+@pytest.mark.parametrize("S,L", [(1, 1), (5, 5), (64, 64), (100, 100), (37, 200), (300, 300), (128, 1000),
+                                 (63, 63), (65, 65), (129, 129), (1, 64), (2, 65), (70, 135), (64, 128), (17, 1025)])
 def test_prefill_causal_vs_oracle(qt, dev, S, L):
     """softmax(Q K^T / 16 + causal) V, GQA 8/2, D=256 (model.py:160-167); with L > S the queries are the last S positions"""
     rng = np.random.default_rng(S * 1000 + L)
@@ -170,6 +171,39 @@ def test_prefill_causal_8192_two_heads_per_wavefront(qt, dev):
         ref = O.sdpa_causal(qn[:, r:r + 1], Kn[:, :r + 1], Vn[:, :r + 1])            # the row at position r sees keys 0..r
         check_attn(f"S=8192 row {r}", o[:, r:r + 1], ref)
     check_equal("row 0 == v[0]", o[:, 0], np.repeat(Vn[:, 0], 4, axis=0))
+
+
+def test_prefill_causal_long_ragged_continuation(qt, dev):
+    """two heads per wavefront with nothing aligned: S = 8170 query rows continue a prefix of 37 keys (L = 8207: the last tile is
+    shifted back, the last row blocks are partial, some wavefronts have one tile less than their workgroup)"""
+    rng = np.random.default_rng(8170)
+    S, P0 = 8170, 37
+    L = S + P0
+    g = torch.Generator().manual_seed(8170)
+    q = torch.randn((8, S, 256), generator=g).bfloat16()
+    K = torch.randn((2, L, 256), generator=g).bfloat16()
+    V = torch.randn((2, L, 256), generator=g).bfloat16()
+    o = to_np(qt.attention.scaled_dot_product_attention(q.to(dev)[None], K.to(dev)[None], V.to(dev)[None], scale=256 ** -0.5,
+                                                        mask="causal"))[0]
+    rows = sorted(set([0, 1, 15, 16, 26, 27, 31, 32, 8127, 8128, 8159, 8160, 8161, 8168, 8169] + [int(r) for r in rng.integers(0, S, 30)]))
+    qn, Kn, Vn = q.float().numpy(), K.float().numpy(), V.float().numpy()
+    for r in rows:
+        ref = O.sdpa_causal(qn[:, r:r + 1], Kn[:, :P0 + r + 1], Vn[:, :P0 + r + 1])   # the row at position P0 + r sees keys 0..P0 + r
+        check_attn(f"continuation row {r}", o[:, r:r + 1], ref)
+
+
+@pytest.mark.parametrize("qscale", [0.05, 6.0, 40.0])
+def test_prefill_causal_score_ranges(qt, dev, qscale):
+    """flat scores (no row is ever rescaled after the first tile), scores whose maxima keep jumping by more than the rescale
+    threshold, and near one-hot softmax rows"""
+    rng = np.random.default_rng(int(qscale * 100))
+    S = 400
+    q = bf(rng.standard_normal((8, S, 256)) * qscale)
+    K = bf(rng.standard_normal((2, S, 256)))
+    V = bf(rng.standard_normal((2, S, 256)))
+    o = qt.attention.scaled_dot_product_attention(to_dev(q, dev, BF16)[None], to_dev(K, dev, BF16)[None], to_dev(V, dev, BF16)[None],
+                                                  scale=256 ** -0.5, mask="causal")
+    check_attn(f"q scale {qscale}", to_np(o)[0], O.sdpa_causal(q, K, V))
 
 
 # ------------------------------------------------------------------------------------- glue either side of the attention kernels

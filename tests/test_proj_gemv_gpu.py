@@ -87,6 +87,13 @@ def test_fused_gemv_prologues_and_leading_dims(qt, dev):
     _close("gnorm + add", to_np(c), O.fused_gemv(to_np(Wo), to_np(y), gnorm=(to_np(proj), to_np(gw)), res=to_np(res)), 2)
 
 
+def test_no_rows_is_not_an_error(qt, dev):
+    W = torch.zeros((64, 1024), dtype=BF16, device=dev)
+    x = torch.zeros((0, 1024), dtype=BF16, device=dev)
+    assert tuple(qt.kernels.fused_gemv(W, x).shape) == (0, 64)
+    assert tuple(qt.batch.rms_rows(x, torch.ones(1024, dtype=BF16, device=dev)).shape) == (0, 1024)
+
+
 def test_fused_gemv_rejects_bad_arguments(qt, dev):
     W = torch.zeros((64, 1024), dtype=BF16, device=dev)
     x = torch.zeros((2, 1024), dtype=BF16, device=dev)
