@@ -360,6 +360,12 @@ def profile_leg(torch, qt, dev, args):
         bench_attn_prefill(torch, qt, dev)
     elif leg == "projections":
         bench_projections(torch, qt, dev)
+    elif leg == "state_admission":
+        bench_state_admission(torch, qt, dev)
+    elif leg == "prefix_cache":
+        bench_prefix_cache(torch, qt, dev)
+    elif leg == "attn_glue":
+        bench_attn_glue(torch, qt, dev)
     elif leg == "attn_prefill_long":
         bench_attn_prefill(torch, qt, dev, 8192)
     else:
@@ -390,7 +396,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the B sweep and the single-pool run")
     ap.add_argument("--only", default="", help="profile helper: run only one leg a few times and exit "
-                                               "(decode | copy | prefill | verify | attn_decode | attn_verify | attn_prefill | attn_prefill_long | projections)")
+                                               "(decode | copy | prefill | verify | attn_decode | attn_verify | attn_prefill | attn_prefill_long | "
+                                               "projections | state_admission | prefix_cache | attn_glue)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every work item of the path is an independent (slot, head) pair; "
