@@ -55,22 +55,22 @@ __global__ __launch_bounds__(256) void rms_rows_kernel(const bf16_t* __restrict_
 }
 
 constexpr int EPI_NONE = 0, EPI_ADD = 1, EPI_SWIGLU = 2;
-constexpr int MT = 64;                 // rows per pass
+constexpr int MT = 64;                 // most rows a workgroup takes
 constexpr int G = 2;                   // k chunks (of 32) per register batch
 
-// One workgroup = 16 output features x 64 rows; its NWV wavefronts split K.  grid = (ceil(N / 16), ceil(M / 64)).
+// One workgroup = 16 output features x 16 MS rows; its NWV wavefronts split K.  grid = (ceil(N / 16), ceil(M / 16 MS)).
 // K / 32 is a multiple of G NWV: every wavefront gets a whole number of batches of G chunks.  At most 128 registers, so that
 // four workgroups of four wavefronts (or one of sixteen) share a CU: 514 workgroups of the widest projection (N = 8224) are
 // resident at once, and the narrow ones (N = 1024: 64 workgroups) get short K chains from sixteen wavefronts each.
-// MS = 16-row blocks that are computed (1, 2 or 4; rows past M repeat the last row and are dropped): a compile-time count keeps
-// the MFMA sequence free of branches.
+// MS = 16-row blocks per workgroup (1, 2 or 4; rows past M repeat the last row and are dropped): a compile-time count keeps
+// the MFMA sequence free of branches, and a small one spreads a narrow output over more workgroups.
 template <int NWV, int MS, int EPI>
 __global__ __launch_bounds__(64 * NWV, 16 / NWV) void skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ x,
                                                                          const bf16_t* __restrict__ res, bf16_t* __restrict__ y, int M, int N,
                                                                          int K) {
-    __shared__ float red[NWV][16][MT + 1];
+    __shared__ float red[NWV][16][16 * MS + 1];
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * 16, m0 = blockIdx.y * MT;
+    const int n0 = blockIdx.x * 16, m0 = blockIdx.y * (16 * MS);
     const int kc_w = K / 32 / NWV;                                // chunks of this wavefront
     const int k_base = w * kc_w * 32 + 8 * g;
     // lane (n, g) loads feature n0 + n and row m0 + 16 ms + n, elements k + 8 g .. + 8; rows past the end repeat the last
@@ -241,7 +241,7 @@ void launch_wide(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, b
 
 template <int NWV, int MS>
 void launch_gemm_ms(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, bf16_t* y, int M, int N, int K, hipStream_t stream) {
-    const dim3 grid((N + 15) / 16, (M + MT - 1) / MT), block(64 * NWV);
+    const dim3 grid((N + 15) / 16, (M + 16 * MS - 1) / (16 * MS)), block(64 * NWV);
     if (epi == EPI_NONE)
         hipLaunchKernelGGL((skinny_gemm_kernel<NWV, MS, EPI_NONE>), grid, block, 0, stream, W, x, res, y, M, N, K);
     else if (epi == EPI_ADD)
@@ -249,9 +249,13 @@ void launch_gemm_ms(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res
     else
         hipLaunchKernelGGL((skinny_gemm_kernel<NWV, MS, EPI_SWIGLU>), grid, block, 0, stream, W, x, res, y, M, N, K);
 }
+// narrow: the output has few feature blocks, so fewer rows per workgroup (more workgroups) pay for re-reading W from L2
 template <int NWV>
-void launch_gemm(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, bf16_t* y, int M, int N, int K, hipStream_t stream) {
-    switch (row_blocks(M)) {
+void launch_gemm(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, bf16_t* y, int M, int N, int K, hipStream_t stream,
+                 bool narrow) {
+    int ms = row_blocks(M);
+    while (narrow && ms > 1 && (long)((N + 15) / 16) * ((M + 16 * ms - 1) / (16 * ms)) < 256) ms /= 2;
+    switch (ms) {
         case 1: launch_gemm_ms<NWV, 1>(epi, W, x, res, y, M, N, K, stream); break;
         case 2: launch_gemm_ms<NWV, 2>(epi, W, x, res, y, M, N, K, stream); break;
         default: launch_gemm_ms<NWV, 4>(epi, W, x, res, y, M, N, K, stream);
@@ -293,11 +297,11 @@ int qt_fused_gemv(const void* W, const void* x, const void* res, void* y, int M,
     }
     const bool wide = (long)((N + 15) / 16) * ((M + MT - 1) / MT) >= 512;
     if (!wide && kc % (2 * 16) == 0)
-        launch_gemm<16>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, K, stream);
+        launch_gemm<16>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, K, stream, true);
     else if (!wide && kc % (2 * 8) == 0)
-        launch_gemm<8>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, K, stream);
+        launch_gemm<8>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, K, stream, true);
     else
-        launch_gemm<4>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, K, stream);
+        launch_gemm<4>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, K, stream, !wide);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }
