@@ -442,6 +442,25 @@ def main():
         t1 = time_graph(torch, one, reps=N_LAYERS * 20, inner=N_LAYERS)
         extras["decode_plus_gated_norm"] = {"two_launches_us": t2 * 1e6, "fused_us": t1 * 1e6,
                                             "fused_GBps": (decode_bytes(B) + B * 2048 * 2) / t1 / 1e9}
+        # the whole GatedDeltaNet half of a layer at a decode step (qwen35/batch.py:496-501): rms_rows, in_proj, the step with
+        # the gated norm, out_proj with the residual: four launches
+        g = torch.Generator().manual_seed(3)
+        bf = torch.bfloat16
+        Wi = [(torch.randn((PW, 1024), generator=g) / 32).to(bf).to(dev) for _ in range(8)]
+        Wo = [(torch.randn((1024, 2048), generator=g) / 45).to(bf).to(dev) for _ in range(8)]
+        xh = torch.randn((B, 1024), generator=g).to(bf).to(dev)
+        ln = torch.ones(1024, dtype=bf, device=dev)
+
+        def layer():
+            l = it[0] % N_LAYERS
+            it[0] += 1
+            proj = qt.kernels.fused_gemv(Wi[l & 7], qt.batch.rms_rows(xh, ln))
+            yn = qt.batch.deltanet_b_gnorm(proj, st["conv"][l], st["cw"][l], st["A_log"][l], st["dtb"][l], st["ssm"][l], st["slots"],
+                                           st["pos"][0], gw)
+            qt.kernels.fused_gemv(Wo[l & 7], yn, res=xh)
+        t3 = time_graph(torch, layer, reps=N_LAYERS * 10, inner=N_LAYERS)
+        extras["gdn_layer_half_decode"] = {"B": B, "launches": 4, "us": t3 * 1e6}
+        del Wi, Wo
         w1, d1 = time_decode(torch, qt, st, B, 1, args.steps, args.warmup, use_graph=not args.no_graph)
         extras["single_pool_cache_resident"] = {"steps_per_s": args.steps / w1, "GBps": decode_bytes(B) / (d1 / args.steps) / 1e9}
         if not args.no_graph:
