@@ -135,9 +135,17 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         unsigned off0 = ld_off0;
         asm volatile("" : "+v"(off0));                           // recompute the offset (one XOR) rather than keeping eight of
                                                                  // them in registers the accumulators need
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(src + (size_t)tile_row0(t) * (AD * 2) + (off0 ^ (1056u * i))),
-            (__attribute__((address_space(3))) void*)(dst + (8 * w + i) * 512), 16, 0, 0);
+        // the row part of load i (2 i rows = 1024 i bytes) goes into the instruction's immediate offset, which moves the global
+        // address and the LDS destination alike (at most 4095: the upper four loads start 4 KiB further in both)
+        const auto gp = (const __attribute__((address_space(1))) void*)(src + (size_t)tile_row0(t) * (AD * 2) + 4096 * (i >> 2) +
+                                                                        (off0 ^ (32u * i)));
+        const auto lp = (__attribute__((address_space(3))) void*)(dst + (8 * w + 4 * (i >> 2)) * 512);
+        switch (i & 3) {                                         // the immediate has to be a literal
+            case 0: __builtin_amdgcn_global_load_lds(gp, lp, 16, 0, 0); break;
+            case 1: __builtin_amdgcn_global_load_lds(gp, lp, 16, 1024, 0); break;
+            case 2: __builtin_amdgcn_global_load_lds(gp, lp, 16, 2048, 0); break;
+            default: __builtin_amdgcn_global_load_lds(gp, lp, 16, 3072, 0);
+        }
     };
     auto load_rows = [&](const char* src, bf16_t* dst, int t) {  // one K or V tile: this wavefront's eight direct loads
         if (L >= KT) {
