@@ -131,10 +131,14 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     // byte offset of load 0 within a tile; load i differs by XOR with 1056 i (row bits 10..12, chunk bits 5..7)
     const unsigned ld_off0 = (unsigned)(16 * w + (lane >> 5)) * (AD * 2) + ((unsigned)((lane & 31) ^ (lane >> 5)) << 4);
     auto tile_row0 = [&](int t) { return max(0, min(t * KT, L - KT)); };
-    auto load_one = [&](const char* src, bf16_t* dst, int t, int i) {        // load i of tile t (L >= KT)
+    // a copy of ld_off0 the compiler cannot see through: the offsets of the eight loads are then recomputed where they are
+    // used (one XOR each) instead of living in registers the accumulators need
+    auto opaque_off0 = [&]() {
         unsigned off0 = ld_off0;
-        asm volatile("" : "+v"(off0));                           // recompute the offset (one XOR) rather than keeping eight of
-                                                                 // them in registers the accumulators need
+        asm volatile("" : "+v"(off0));
+        return off0;
+    };
+    auto load_one = [&](const char* src, bf16_t* dst, int t, int i, unsigned off0) {   // load i of tile t (L >= KT)
         // the row part of load i (2 i rows = 1024 i bytes) goes into the instruction's immediate offset, which moves the global
         // address and the LDS destination alike (at most 4095: the upper four loads start 4 KiB further in both)
         const auto gp = (const __attribute__((address_space(1))) void*)(src + (size_t)tile_row0(t) * (AD * 2) + 4096 * (i >> 2) +
@@ -150,7 +154,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     auto load_rows = [&](const char* src, bf16_t* dst, int t) {  // one K or V tile: this wavefront's eight direct loads
         if (L >= KT) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) load_one(src, dst, t, i);
+            for (int i = 0; i < 8; i++) load_one(src, dst, t, i, ld_off0);
         } else {                                                 // t = 0: rows past the end repeat the last key; they are masked
 #pragma unroll
             for (int i = 0; i < 8; i++) {
@@ -180,7 +184,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
 
     // K fragment kb of sub-tile kt
     auto k_frag = [&](const bf16_t* ka, int kt, int kb) {
-        return *reinterpret_cast<const bf16x8*>(ka + 16 * kt * AD + (((4 * kb + g) ^ n) << 3));
+        // chunk (4 kb + g) ^ n; n < 16 leaves bit 4 alone, so fragments kb and kb + 4 share an address register
+        return *reinterpret_cast<const bf16x8*>(ka + 16 * kt * AD + (((4 * (kb & 3) + g) ^ n) << 3) + 128 * (kb >> 2));
     };
     // scores of tile 0, S^T = K_tile . Q^T: each K fragment multiplies the Q^T of both heads; the fragments of the next
     // 16-key sub-tile are read while the MFMAs of the current one run
@@ -256,7 +261,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         const bf16_t* va = v_cur + va_row;
         auto v_frag = [&](int j, int q4) {
             return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * AD + (((2 * j + vc0) ^ vrow) << 3))));
+                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * AD + (((2 * (j & 7) + vc0) ^ vrow) << 3) +
+                                                                             128 * (j >> 3))));   // the swizzle (< 16) leaves bit 4 alone
         };
         s16x8 P[NH][2];
         s16x4 Bf[3][4];
@@ -287,6 +293,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 rescale |= corr != 1.0f;
             }
             AP_MARK(3);
+            const unsigned step_off0 = SC ? opaque_off0() : 0u;
             // 32 steps: two score MFMAs of tile t + 1 (one K fragment x both heads) and one softmax element of tile t
             float pv_prev = 0.f;
 #pragma unroll
@@ -295,9 +302,9 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 __builtin_amdgcn_sched_barrier(0);
                 if (SC && (st & 1) == 0) {
                     if (st < 16)
-                        load_one(kg, k_cur, tk, st >> 1);
+                        load_one(kg, k_cur, tk, st >> 1, step_off0);
                     else
-                        load_one(vg, v_nxt, tv, (st >> 1) - 8);
+                        load_one(vg, v_nxt, tv, (st >> 1) - 8, step_off0);
                 }
                 if (SC) {
                     if (kt < 3) Af[(kt + 1) & 1][kb] = k_frag(ka, kt + 1, kb);
