@@ -56,6 +56,7 @@ def lib():
         for name in ("qt_gdn_chunk_ops_bytes", "qt_gdn_chunk_u_bytes", "qt_gdn_chunk_gc_bytes", "qt_gdn_chunk_snap_bytes",
                      "qt_gqa_prefill_workspace_bytes"):
             getattr(L, name).argtypes, getattr(L, name).restype = [_i], ctypes.c_long
+        L.qt_gqa_prefill_workspace_bytes_for.argtypes, L.qt_gqa_prefill_workspace_bytes_for.restype = [_i] * 3, ctypes.c_long
         _lib = L
     return _lib
 

@@ -18,6 +18,7 @@
 // the score MFMAs of tile t + 1 are interleaved step by step with the softmax of tile t (see `tile` below).
 #include "qt_common.h"
 
+#include <algorithm>
 #include <type_traits>
 
 using namespace qt;
@@ -83,12 +84,27 @@ __device__ __forceinline__ float max_over_groups(float x) {
 // it is hoisted to the top of every tile and holds 128 VALU registers through the score phase).
 #define PIN_ACC(x) asm volatile("" : "+a"(x))
 
+// Key split (NH = 1 launches only).  A causal launch with about one workgroup per CU is as slow as its longest row block, twice
+// the average.  With tmax > 0 the tiles of a 16-row block are cut into parts of tmax tiles, one workgroup per part; a block
+// with more than one part leaves unnormalised partial results (O, reference point m, row sums l) in the workspace and
+// attn_prefill_merge_kernel combines them.  Block i counts ceil((p + i + 1) / c) parts, p = ceil(q_pos0 / 16), c = 4 tmax (16
+// rows advance the visible keys by a quarter tile), which is never fewer than its tiles need (a part may be empty); the
+// parts of blocks 0 .. r-1 are then parts_upto(p + r, c) - parts_upto(p, c), and a workgroup inverts that sum to find its part.
+__host__ __device__ inline long parts_upto(long n, long c) {      // sum over j = 1 .. n of ceil(j / c)
+    const long k = n / c;
+    return c * (k * (k + 1) / 2) + (n - k * c) * (k + 1);
+}
+constexpr int PART_O = 4 * 16 * AD;    // floats of one part's O: [4 heads][16 rows][256]
+constexpr int PART_ML = 4 * 2 * 16;    // ... and of its m, l: [4 heads][m | l][16 rows]
+
 // NH = heads per wavefront: 2 (32 query rows per workgroup, as described above) for long sequences; 1 (16 rows per workgroup,
 // one head per wavefront: twice the workgroups, LDS-bound) when the launch would otherwise leave CUs idle.
+// grid = (row blocks, or parts when tmax > 0; KV heads)
 template <int NH>
 __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
                                                            const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
-                                                           int q_pos0, long q_head_stride, long kv_head_stride) {
+                                                           int q_pos0, long q_head_stride, long kv_head_stride, int tmax,
+                                                           float* __restrict__ part_o, float* __restrict__ part_ml) {
     // four separate arrays, not [2][TILE]: the compiler tracks outstanding direct-to-LDS loads per LDS variable, so a read of
     // one buffer does not wait for the loads in flight to the others
     __shared__ __align__(1024) bf16_t k_s0[TILE];
@@ -97,7 +113,19 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     __shared__ __align__(1024) bf16_t v_s1[TILE];
     __shared__ __align__(16) float c_s[4][2][16];
     constexpr int RB = 16 * NH;
-    const int rb = gridDim.x - 1 - blockIdx.x;                   // long rows first
+    int rb = gridDim.x - 1 - blockIdx.x;                         // long rows first
+    int part = 0, nparts = 1;
+    if (NH == 1 && tmax > 0) {                                   // blockIdx.x counts parts, again from the long end
+        const int c = 4 * tmax, p = (q_pos0 + 15) >> 4;
+        const long y = (long)rb + parts_upto(p, c);              // parts_upto(nn) <= y < parts_upto(nn + 1), nn = p + row block
+        int k = 0;
+        while ((long)c * ((k + 1) * (k + 2) / 2) <= y) k++;
+        const int nn = k * c + (int)((y - (long)c * (k * (k + 1) / 2)) / (k + 1));
+        part = (int)(y - parts_upto(nn, c));
+        nparts = k + 1;
+        rb = nn - p;
+    }
+    const size_t slot = (size_t)blockIdx.y * gridDim.x + (gridDim.x - 1 - blockIdx.x);   // parts of a block: consecutive slots
     const int kvh = blockIdx.y;
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int h0 = kvh * (AH / AKV) + (NH == 2 ? 2 * (w & 1) : w);       // this wavefront's heads: h0 (, h0 + 1)
@@ -108,6 +136,9 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     const int ntiles = (kend + KT - 1) / KT;
     const int kend_w = r0 < S ? min(L, q_pos0 + min(r0 + 15, S - 1) + 1) : 0;  // keys any row of this wavefront sees
     const int ntiles_w = (kend_w + KT - 1) / KT;
+    // this workgroup's tiles [ta, tb); tw: where this wavefront's rows end
+    const int ta = part * (NH == 1 && tmax > 0 ? tmax : 0), tb = NH == 1 && tmax > 0 ? min(ntiles, ta + tmax) : ntiles;
+    const int tw = min(ntiles_w, tb);
 
     // Q^T as the B operand of the score MFMA: lane (row n, group g) holds q[row][32 kb + 8 g .. + 8], for both heads
     bf16x8 bq[NH][8];
@@ -237,14 +268,14 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         // While scores of a further tile are due (then L > KT), this wavefront's 16 loads of K(t + 2) and V(t + 1) are spread
         // over the steps below: a burst would stall on the memory pipeline's queue.  There a tile index past the end loads the
         // last tile again, harmlessly: nothing reads that buffer any more.
-        const bool more = t + 1 < ntiles_w;                      // wavefront-uniform
-        const int tk = min(t + 2, ntiles - 1), tv = min(t + 1, ntiles - 1);
+        const bool more = t + 1 < tw;                            // wavefront-uniform
+        const int tk = min(t + 2, tb - 1), tv = min(t + 1, tb - 1);
         if (!more) {
-            if (t + 2 < ntiles) load_rows(kg, k_cur, t + 2);
-            if (t + 1 < ntiles) load_rows(vg, v_nxt, t + 1);
+            if (t + 2 < tb) load_rows(kg, k_cur, t + 2);
+            if (t + 1 < tb) load_rows(vg, v_nxt, t + 1);
         }
         AP_MARK(2);
-        if (t >= ntiles_w) return;                               // wavefront-uniform: the upper row block may see one tile more
+        if (t >= tw) return;                               // wavefront-uniform: the upper row block may see one tile more
         // only tiles that touch the diagonal or the end of the sequence need the mask (wavefront-uniform)
         if (t * KT + KT - 1 > q_pos0 + r0 || t * KT + KT > L) {
 #pragma unroll
@@ -394,17 +425,37 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         wave_lds_sync();                                         // c_s is rewritten by the next tile
     };
 
-    load_rows(kg, k_s0, 0);
-    load_rows(vg, v_s0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (ntiles > 1) load_rows(kg, k_s1, 1);
-    if (ntiles_w > 0) scores_first(k_s0 + ka_row, accs[0]);
-    for (int t = 0; t < ntiles; t += 2) {
-        tile(t, std::integral_constant<int, 0>{});
-        if (t + 1 < ntiles) tile(t + 1, std::integral_constant<int, 1>{});
+    if (ta < tb) {                                               // (a part past the block's last tile is empty)
+        load_rows(kg, k_s0, ta);
+        load_rows(vg, v_s0, ta);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tb - ta > 1) load_rows(kg, k_s1, ta + 1);
+        if (tw > ta) scores_first(k_s0 + ka_row, accs[0]);
+        for (int t = ta; t < tb; t += 2) {
+            tile(t, std::integral_constant<int, 0>{});
+            if (t + 1 < tb) tile(t + 1, std::integral_constant<int, 1>{});
+        }
     }
     AP_STORE();
+    if (NH == 1 && nparts > 1) {
+        // One part of several: leave O, m, l of this wavefront's head as they are.  A row that sees no key of this part (its
+        // last key lies before the part's first) has exponentiated masked scores against a masked maximum: it is written as
+        // the neutral element (m = NEG, l = 0, O = 0).
+        const int first_key = ta * KT;
+        float* po = part_o + (slot * 4 + w) * (16 * AD);
+        float* pml = part_ml + (slot * 4 + w) * 32;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int lr = 4 * g + r;
+            const bool seen = q_pos0 + r0 + lr >= first_key;
+#pragma unroll
+            for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n] = seen ? O[0][j][r] : 0.f;
+            if (n == 0) pml[16 + lr] = seen ? Lsum[0][r] : 0.f;
+        }
+        if (g == 0) pml[n] = my_last >= first_key ? m_run[0] : NEG;
+        return;
+    }
     // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n, and of the row sums (any column)
 #pragma unroll
     for (int hh = 0; hh < NH; hh++) {
@@ -421,33 +472,149 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     }
 }
 
+// Combines the parts of the row blocks that were split: grid = (split blocks, KV heads, 4 heads of the group); thread (row,
+// 16-column group) of the 16 x 256 block.  out = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p, parts in order; a thread's
+// loads of O do not depend on the factors, so all parts are in flight together.
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                                 bf16_t* __restrict__ out, int S, int q_pos0, int tmax, long slots_per_kv,
+                                                                 long q_head_stride) {
+    const int c = 4 * tmax, p = (q_pos0 + 15) >> 4;
+    const int rb = max(0, c - p) + blockIdx.x;                   // the first block with two parts is c - p
+    const int np = (p + rb) / c + 1;
+    const size_t slot0 = (size_t)blockIdx.y * slots_per_kv + (size_t)(parts_upto(p + rb, c) - parts_upto(p, c));
+    const int hq = blockIdx.z, lr = threadIdx.x >> 4, cg = threadIdx.x & 15;
+    if (rb * 16 + lr >= S) return;
+    const float* po = part_o + (slot0 * 4 + hq) * (16 * AD) + lr * AD + cg * 16;
+    const float* pml = part_ml + (slot0 * 4 + hq) * 32 + lr;
+    float m = NEG;
+    for (int pp = 0; pp < np; pp++) m = fmaxf(m, pml[(size_t)pp * PART_ML]);
+    float l = 0.f;
+    f32x4 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+    for (int pp = 0; pp < np; pp++) {
+        f32x4 o[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = reinterpret_cast<const f32x4*>(po + (size_t)pp * PART_O)[i];
+        const float f = __builtin_amdgcn_exp2f(pml[(size_t)pp * PART_ML] - m);
+        l += f * pml[(size_t)pp * PART_ML + 16];
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[i] += f * o[i];
+    }
+    const float inv = 1.0f / l;
+    uint32_t pk[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        pk[2 * i] = pack_bf(acc[i][0] * inv, acc[i][1] * inv);
+        pk[2 * i + 1] = pack_bf(acc[i][2] * inv, acc[i][3] * inv);
+    }
+    u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)(blockIdx.y * (AH / AKV) + hq) * q_head_stride + (size_t)(rb * 16 + lr) * AD + cg * 16);
+    dst[0] = u32x4{pk[0], pk[1], pk[2], pk[3]};
+    dst[1] = u32x4{pk[4], pk[5], pk[6], pk[7]};
+}
+
+}  // namespace
+
+namespace {
+
+int cu_count() {                       // CUs of the current device (256 if the query fails)
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+        n = 256;
+    return n;
+}
+inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 304; }
+
+// The key split of a launch: tmax = 0 (none) or the tiles per part, parts = grid width, split_blocks = blocks with several parts.
+// Only launches that leave at least half of the CUs without a workgroup are split (up to 1024 query rows: a short continuation
+// of a long prefix, a short prompt); a part then holds at least the launch's average tiles per CU, and at least 8.  A workgroup costs
+// about 6 us beyond its tiles (dispatch, Q and first-tile latency, the output stores): measured at S = 2048 (256 workgroups,
+// 57 us unsplit) every part size from 4 to 32 tiles came out between 53 and 61 us before the parts were even merged.
+struct KeySplit {
+    int tmax = 0;
+    long parts = 0;
+    int split_blocks = 0;
+};
+KeySplit plan_split(int S, int L, int q_pos0) {
+    KeySplit ks;
+    if (S < 1 || two_heads_per_wave(S)) return ks;
+    const int nb = (S + 15) / 16, cus = cu_count();
+    if (nb * AKV > cus / 2) return ks;
+    long total = 0;
+    int longest = 0;
+    for (int i = 0; i < nb; i++) {
+        const int kend = std::min(L, q_pos0 + std::min(16 * i + 15, S - 1) + 1), nt = (kend + KT - 1) / KT;
+        total += nt;
+        longest = std::max(longest, nt);
+    }
+    // the smallest part size (from the average per CU, at least 8 tiles) whose parts are all resident at once: a CU that has
+    // to run a second part pays the per-workgroup cost twice
+    const long p = (q_pos0 + 15) >> 4;
+    int tmax = (int)std::max(8L, (total * AKV + cus - 1) / cus);
+    while (tmax < longest && (parts_upto(p + nb, 4L * tmax) - parts_upto(p, 4L * tmax)) * AKV > cus) tmax++;
+    if (tmax >= longest) return ks;
+    const long c = 4L * tmax;
+    ks.tmax = tmax;
+    ks.parts = parts_upto(p + nb, c) - parts_upto(p, c);
+    ks.split_blocks = nb - (int)std::max(0L, c - p);
+    return ks;
+}
+
 }  // namespace
 
 extern "C" {
 
-// no workspace is needed any more; the entry point keeps its argument (may be null) so that callers do not change
-long qt_gqa_prefill_workspace_bytes(int L) { return L < 0 ? -1 : 0; }
+// Bytes of workspace the key split of this launch uses (0: the launch is not split).  Without that much workspace
+// qt_gqa_prefill_causal runs the same launch unsplit, with the same results up to rounding.
+long qt_gqa_prefill_workspace_bytes_for(int S, int L, int q_pos0) {
+    if (S < 0 || L < 1 || q_pos0 < 0) return -1;
+    const KeySplit ks = plan_split(S, L, q_pos0);
+    return ks.tmax ? ks.parts * AKV * (long)(PART_O + PART_ML) * 4 : 0;
+}
+// An upper bound of the above over every launch with at most L keys (S <= L, q_pos0 = L - S or smaller): a part holds at least
+// total / CUs tiles, so there are at most CUs / 2 + 2 * blocks parts per KV head, and a split launch has at most CUs / 4 blocks.
+long qt_gqa_prefill_workspace_bytes(int L) {
+    if (L < 0) return -1;
+    const long cus = cu_count(), nb = std::min((long)(L + 15) / 16, cus / (2 * AKV));
+    return (cus + AKV * (2 * nb + 2)) * (long)(PART_O + PART_ML) * 4;
+}
 
 // q, out [8][S][256] bf16 (head stride q_head_stride elements), K, V [2][>=L][256] bf16 (head stride kv_head_stride):
-// query i sits at absolute position q_pos0 + i and sees keys 0 .. q_pos0 + i (< L).
+// query i sits at absolute position q_pos0 + i and sees keys 0 .. q_pos0 + i (< L).  workspace: see above; may be null.
 int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out, void* workspace, long workspace_bytes, int S,
                           int L, int q_pos0, long q_head_stride, long kv_head_stride, hipStream_t stream) {
-    (void)workspace;
-    (void)workspace_bytes;
     if (!q || !K || !V || !out) return QT_ERR_NULL;
-    if (S < 0 || L < 1 || q_pos0 < 0 || q_head_stride < (long)S * AD || kv_head_stride < (long)L * AD) return QT_ERR_DIM;
+    if (S < 0 || L < 1 || q_pos0 < 0 || (long)q_pos0 + S > L || q_head_stride < (long)S * AD || kv_head_stride < (long)L * AD)
+        return QT_ERR_DIM;
     if (S == 0) return QT_OK;
-    for (const void* p : {q, K, V, (const void*)out})
+    for (const void* p : {q, K, V, (const void*)out, (const void*)workspace})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if ((q_head_stride | kv_head_stride) & 7) return QT_ERR_ALIGN;
     // two heads per wavefront from about 4800 query rows on (measured: one head per wavefront 140 us at S = 4096 and 296 us at
     // S = 6144, two heads 156 us and 237 us); below that, 16-row blocks give twice the workgroups
-    if ((S + 31) / 32 * AKV >= 304)
+    if (two_heads_per_wave(S)) {
         hipLaunchKernelGGL(attn_prefill_kernel<2>, dim3((S + 31) / 32, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
-                           (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride);
-    else
+                           (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, 0, (float*)nullptr,
+                           (float*)nullptr);
+        QT_CHECK_LAUNCH();
+        return QT_OK;
+    }
+    KeySplit ks = plan_split(S, L, q_pos0);
+    if (ks.tmax && (!workspace || workspace_bytes < ks.parts * AKV * (long)(PART_O + PART_ML) * 4)) ks = KeySplit();
+    if (!ks.tmax) {
         hipLaunchKernelGGL(attn_prefill_kernel<1>, dim3((S + 15) / 16, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
-                           (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride);
+                           (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, 0, (float*)nullptr,
+                           (float*)nullptr);
+        QT_CHECK_LAUNCH();
+        return QT_OK;
+    }
+    float* part_o = (float*)workspace;
+    float* part_ml = part_o + (size_t)ks.parts * AKV * PART_O;
+    hipLaunchKernelGGL(attn_prefill_kernel<1>, dim3((unsigned)ks.parts, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
+                       (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
+    hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)ks.split_blocks, AKV, AH / AKV), dim3(256), 0, stream, part_o,
+                       part_ml, (bf16_t*)out, S, q_pos0, ks.tmax, ks.parts, q_head_stride);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

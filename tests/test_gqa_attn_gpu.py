@@ -206,6 +206,44 @@ def test_prefill_causal_score_ranges(qt, dev, qscale):
     check_attn(f"q scale {qscale}", to_np(o)[0], O.sdpa_causal(q, K, V))
 
 
+@pytest.mark.parametrize("S,P0,qscale", [(1024, 0, 1.0), (1000, 23, 1.0), (100, 1007, 1.0), (64, 8000, 1.0), (300, 4001, 1.0),
+                                         (1024, 3000, 1.0), (16, 5000, 1.0), (1, 4095, 1.0), (1000, 9, 40.0), (130, 2000, 0.05)])
+def test_prefill_causal_key_split(qt, dev, S, P0, qscale):
+    """Launches that leave half of the CUs idle are split along the keys (parts of a row block meet in a workspace and a second
+    kernel combines them): prompts of up to 1024 rows and short continuations of a long prefix, positions that are no
+    multiple of 16 (some rows of a block then see no key of the block's last part), rescaled and flat score ranges.  Checked
+    against the float64 oracle on a sample of rows, and against the same launch without a workspace (unsplit)."""
+    from qwen_tailor_amd import _lib as QL
+    rng = np.random.default_rng(S * 7 + P0)
+    L = S + P0
+    g = torch.Generator().manual_seed(S * 7 + P0)
+    q = (torch.randn((8, S, 256), generator=g) * qscale).bfloat16()
+    K = torch.randn((2, L, 256), generator=g).bfloat16()
+    V = torch.randn((2, L, 256), generator=g).bfloat16()
+    assert QL.lib().qt_gqa_prefill_workspace_bytes_for(S, L, P0) > 0, "this case is meant to be split"
+    assert QL.lib().qt_gqa_prefill_workspace_bytes_for(S, L, P0) <= QL.lib().qt_gqa_prefill_workspace_bytes(L)
+    dq, dK, dV = q.to(dev)[None], K.to(dev)[None], V.to(dev)[None]
+    o = qt.attention.scaled_dot_product_attention(dq, dK, dV, scale=256 ** -0.5, mask="causal")
+    plain = torch.full_like(o, float("nan"))
+    QL.call("qt_gqa_prefill_causal", QL.ptr(dq), QL.ptr(dK), QL.ptr(dV), QL.ptr(plain), None, 0, S, L, P0, S * 256, L * 256, QL.stream())
+    o, plain = to_np(o)[0], to_np(plain)[0]
+    assert np.isfinite(o).all() and np.isfinite(plain).all()
+    check_attn("split against unsplit", o, plain)
+    rows = sorted(set([0, 1, 15, 16, 17, S // 2, S - 17, S - 16, S - 2, S - 1] + [int(r) for r in rng.integers(0, S, 24)]) & set(range(S)))
+    qn, Kn, Vn = q.float().numpy(), K.float().numpy(), V.float().numpy()
+    for r in rows:
+        ref = O.sdpa_causal(qn[:, r:r + 1], Kn[:, :P0 + r + 1], Vn[:, :P0 + r + 1])
+        check_attn(f"S={S} P0={P0} row {r}", o[:, r:r + 1], ref)
+
+
+def test_prefill_causal_rejects_queries_past_the_keys(qt, dev):
+    from qwen_tailor_amd import _lib as QL
+    t = torch.zeros((1, 8, 32, 256), dtype=BF16, device=dev)
+    kv = torch.zeros((1, 2, 40, 256), dtype=BF16, device=dev)
+    with pytest.raises(RuntimeError):
+        QL.call("qt_gqa_prefill_causal", QL.ptr(t), QL.ptr(kv), QL.ptr(kv), QL.ptr(t), None, 0, 32, 40, 9, 32 * 256, 40 * 256, QL.stream())
+
+
 # ------------------------------------------------------------------------------------- glue either side of the attention kernels
 @pytest.mark.parametrize("R,M", [(1, 1), (5, 1), (8, 4), (64, 1)])
 def test_qkv_prep_and_out_gate_bit_exact(qt, dev, R, M):
