@@ -6,10 +6,12 @@
 //     epilogue  none:   y = bf16(s)                                                                     (kernels.py:153-160)
 //               add:    y = bf16(BF(s) + res)                                                           (kernels.py:161-169)
 //               swiglu: y[m][p] = bf16(silu_bf16(BF(s[m][2p])) * BF(s[m][2p+1]))   interleaved rows     (kernels.py:170-182)
-// The batch is small, so the product is bound by streaming W once from HBM: one workgroup owns 16 output features and all
-// rows (64 per pass); its wavefronts split K, each feeding 16x16x32 bf16 MFMAs straight from global memory (a W
-// fragment is 16 features x 32 k, an x fragment 16 rows x 32 k: both are 16-byte row-contiguous loads per lane), and the
-// partial sums meet in LDS.  Arithmetic contract of rms_rows: sum of squares exact, rounded to float once; inv = correctly
+// The batch is small, so the product is bound by streaming W once from HBM.  General form: one workgroup owns 16 output
+// features and all rows (64 per pass); its wavefronts split K, each feeding 16x16x32 bf16 MFMAs straight from global memory (a
+// W fragment is 16 features x 32 k, an x fragment 16 rows x 32 k: both are 16-byte row-contiguous loads per lane), and the
+// partial sums meet in LDS.  The wide projections of a decode batch (K = 1024, 4 to 64 rows) keep the rows in LDS instead and
+// give every wavefront a feature block with all of its K (xlds_gemm_kernel): what bounds such a launch is the bytes one CU
+// has to pull in, its share of W plus ALL of x.  Arithmetic contract of rms_rows: sum of squares exact, rounded to float once; inv = correctly
 // rounded 1/sqrt(ss / K + eps); t = x * inv and w * t rounded to float separately, then to bf16.
 #include "qt_common.h"
 
@@ -218,6 +220,123 @@ __global__ __launch_bounds__(64 * NWV) void wide_gemm_kernel(const bf16_t* __res
     }
 }
 
+// K = 1024, wide outputs: the rows live in LDS, shared by the whole workgroup, and a wavefront owns a feature block with all
+// of its K, so nothing is summed across wavefronts.  x [16 MS rows][1024] goes HBM / L2 -> LDS directly (global_load_lds: one
+// instruction lands half a row, 1 KiB, contiguously), its 16-byte chunks XOR-swizzled by the row number (the loading lane
+// fetches the chunk that belongs at its position) so that the fragment reads of 16 rows fall on distinct banks.  The
+// wavefront's W block [16 features][1024] is 32 loads, all issued up front (128 registers); every W fragment then meets MS
+// x fragments read from LDS.  Accumulator element i of lane (n, g) is feature 4 g + i of row 16 ms + n: four adjacent
+// features, stored as 8 bytes.  grid = ceil(N / (16 WPB)), block = 64 WPB.
+constexpr int XK = 1024;
+// XL_MARK(i): time stamps of the constant-rate clock for profiling builds (QT_XLDS_PROF defines xl_prof_buf[workgroup][8])
+#ifdef QT_XLDS_PROF
+__device__ long long* xl_prof_buf;
+#define XL_MARK(i)                                                                              \
+    do {                                                                                        \
+        if (threadIdx.x == 0) xl_prof_buf[(size_t)blockIdx.x * 8 + (i)] = wall_clock64();       \
+    } while (0)
+#else
+#define XL_MARK(i)
+#endif
+template <int MS, int WPB, int EPI>
+__global__ __launch_bounds__(64 * WPB) void xlds_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ x,
+                                                        const bf16_t* __restrict__ res, bf16_t* __restrict__ y, int M, int N) {
+    __shared__ __align__(1024) bf16_t x_s[16 * MS * XK];
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    const int n0 = (blockIdx.x * WPB + w) * 16;                   // this wavefront's feature block (may lie past N)
+    XL_MARK(0);
+    // W first (it comes from HBM): the wavefront's block is 32 loads, all in flight at once
+    u32x4 a[XK / 32];
+    {
+        const bf16_t* wp = W + (size_t)min(n0 + n, N - 1) * XK + 8 * g;
+#pragma unroll
+        for (int c = 0; c < XK / 32; c++) a[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + 32 * c));
+    }
+    // x -> LDS: half-row h (of 2 * 16 MS) by wavefront h % WPB; lane l lands at chunk position 64 (h & 1) + l of row h >> 1
+    // (every workgroup reads the same rows at the same time; starting each at another half-row changed nothing)
+    for (int h = w; h < 32 * MS; h += WPB) {
+        const int r = h >> 1, cp = 64 * (h & 1) + lane;
+        const bf16_t* src = x + (size_t)min(r, M - 1) * XK + 8 * (cp ^ (r & 15));
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)(x_s + h * 512), 16, 0, 0);
+    }
+    XL_MARK(1);
+    // (a direct-to-LDS load in flight makes the compiler wait for every outstanding load before the first use of any, so the
+    // products cannot start under the tail of the W stream; both streams are drained here)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    XL_MARK(2);
+    __syncthreads();
+    XL_MARK(3);
+    f32x4 acc[MS];
+#pragma unroll
+    for (int ms = 0; ms < MS; ms++) acc[ms] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // x fragments are read two chunks ahead of their MFMAs (a ring of three), the scheduler pinned
+    auto x_frag = [&](int c, int ms) {
+        return *reinterpret_cast<const u32x4*>(x_s + (16 * ms + n) * XK + 8 * ((4 * c + g) ^ n));
+    };
+    u32x4 b[3][MS];
+#pragma unroll
+    for (int ms = 0; ms < MS; ms++) b[0][ms] = x_frag(0, ms), b[1][ms] = x_frag(1, ms);
+#pragma unroll
+    for (int c = 0; c < XK / 32; c++) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (c + 2 < XK / 32) {
+#pragma unroll
+            for (int ms = 0; ms < MS; ms++) b[(c + 2) % 3][ms] = x_frag(c + 2, ms);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ms = 0; ms < MS; ms++)
+            acc[ms] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[c]), __builtin_bit_cast(bf16x8, b[c % 3][ms]),
+                                                             acc[ms], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    XL_MARK(4);
+    const int f0 = n0 + 4 * g;                                    // first of this lane's four features (N is a multiple of 4)
+    if (f0 >= N) return;                                          // (also a wavefront whose whole block lies past N)
+#pragma unroll
+    for (int ms = 0; ms < MS; ms++) {
+        const int m = 16 * ms + n;
+        if (m >= M) continue;
+        if (EPI == EPI_SWIGLU) {
+            const float g0 = BF(acc[ms][0]), u0 = BF(acc[ms][1]), g1 = BF(acc[ms][2]), u1 = BF(acc[ms][3]);
+            *reinterpret_cast<uint32_t*>(y + (size_t)m * (N / 2) + f0 / 2) = pack_bf(silu_bf16(g0) * u0, silu_bf16(g1) * u1);
+        } else {
+            const size_t o = (size_t)m * N + f0;
+            float v[4] = {acc[ms][0], acc[ms][1], acc[ms][2], acc[ms][3]};
+            if (EPI == EPI_ADD) {
+                const uint2 rr = *reinterpret_cast<const uint2*>(res + o);
+                v[0] = BF(v[0]) + lo_bf(rr.x), v[1] = BF(v[1]) + hi_bf(rr.x), v[2] = BF(v[2]) + lo_bf(rr.y), v[3] = BF(v[3]) + hi_bf(rr.y);
+            }
+            *reinterpret_cast<uint2*>(y + o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
+        }
+    }
+    XL_MARK(5);
+}
+
+template <int MS, int WPB>
+void launch_xlds_wpb(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, bf16_t* y, int M, int N, hipStream_t stream) {
+    const int blocks = (N + 15) / 16;
+    const dim3 grid((blocks + WPB - 1) / WPB), block(64 * WPB);
+    if (epi == EPI_NONE)
+        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_NONE>), grid, block, 0, stream, W, x, res, y, M, N);
+    else if (epi == EPI_ADD)
+        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_ADD>), grid, block, 0, stream, W, x, res, y, M, N);
+    else
+        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_SWIGLU>), grid, block, 0, stream, W, x, res, y, M, N);
+}
+template <int MS>
+void launch_xlds_ms(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, bf16_t* y, int M, int N, hipStream_t stream, int cus) {
+    // as few wavefronts per workgroup as keep the launch within one workgroup per CU (the rows take most of a CU's LDS)
+    const int blocks = (N + 15) / 16, wpb = (blocks + cus - 1) / cus;
+    if (wpb <= 2)
+        launch_xlds_wpb<MS, 2>(epi, W, x, res, y, M, N, stream);
+    else if (wpb == 3)
+        launch_xlds_wpb<MS, 3>(epi, W, x, res, y, M, N, stream);
+    else
+        launch_xlds_wpb<MS, 4>(epi, W, x, res, y, M, N, stream);
+}
+
 // row blocks per pass: 1, 2 or 4 (3 rounds up)
 inline int row_blocks(int M) { return M <= 16 ? 1 : M <= 32 ? 2 : 4; }
 
@@ -262,6 +381,16 @@ void launch_gemm(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, b
     }
 }
 
+int cu_count() {                       // CUs of the current device (256 if the query fails), asked once
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        return n;
+    }();
+    return cus;
+}
+
 }  // namespace
 
 extern "C" {
@@ -290,7 +419,20 @@ int qt_fused_gemv(const void* W, const void* x, const void* res, void* y, int M,
     // wavefronts per workgroup: 4 when the output is wide enough to fill the chip with workgroups; 16 or 8 (as K divides) for
     // the narrow outputs, whose few workgroups would otherwise walk long K chains
     const int kc = K / 32;
-    if (K == 1024 && N >= 4096 && M > 16) {                       // the wide projections of a decode batch: x stays in registers
+    // the wide projections of a decode batch: rows in LDS.  From four rows on (in_proj, one row 6.6 us either way; 4 / 16 /
+    // 64 rows: 6.9 / 7.0 / 9.7 us against 7.0 / 8.4 / 11.9 us for the kernels below)
+    if (K == XK && N >= 4096 && (N & 3) == 0 && M >= 4 && M <= 64) {
+        const int cus = cu_count();
+        if (M <= 16)
+            launch_xlds_ms<1>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, stream, cus);
+        else if (M <= 32)
+            launch_xlds_ms<2>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, stream, cus);
+        else
+            launch_xlds_ms<4>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, stream, cus);
+        QT_CHECK_LAUNCH();
+        return QT_OK;
+    }
+    if (K == 1024 && N >= 4096 && M > 16) {                       // ... of more than 64 rows: x stays in registers
         // three feature blocks per workgroup (172 workgroups for 8224 features): four leave half the CUs without one, two
         // double what the workgroups pull of x from L2; measured 13.2 / 11.7 / 16.3 us for 4 / 3 / 2 at 64 rows
         launch_wide<8, 4, 3>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, K, stream);
