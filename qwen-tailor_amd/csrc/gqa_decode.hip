@@ -101,6 +101,21 @@ __device__ __forceinline__ void pv_tile(f32x4 (&O)[16], const float (&p)[4], con
 }
 
 constexpr int MAX_SEG = 2048;          // segments (2 per sequence) a launch can hold
+// A workgroup pays about 3 us for every segment it visits (the query rows, the first tiles' latency, the merge of its four
+// wavefronts, the partial result): as much as streaming ~5 tiles.  Every segment therefore starts with that many empty
+// positions in the flat tile space, so that a workgroup whose range crosses a segment border gets fewer tiles to stream.
+constexpr int VISIT_TILES = 5;
+
+// AD_MARK(i): time stamps of the constant-rate clock for profiling builds (QT_ATTN_DECODE_PROF defines ad_prof_buf[workgroup][8])
+#ifdef QT_ATTN_DECODE_PROF
+__device__ long long* ad_prof_buf;
+#define AD_MARK(i)                                                                              \
+    do {                                                                                        \
+        if (threadIdx.x == 0) ad_prof_buf[(size_t)blockIdx.x * 8 + (i)] = wall_clock64();       \
+    } while (0)
+#else
+#define AD_MARK(i)
+#endif
 
 // Exclusive prefix of the segments' tile counts -> seg_start[0 .. nseg] (LDS); returns the total.  Rows whose slot or position
 // is out of range own no tiles (they are skipped by both kernels).  Every thread of the workgroup must call it.
@@ -111,7 +126,7 @@ __device__ __forceinline__ int build_segments(int* seg_start, const int* __restr
     for (int sg = tid; sg < nseg; sg += 256) {
         const int b = sg / AKV, slot = slots[b], p0 = pos[b];
         const bool ok = (unsigned)slot < (unsigned)n_slots && p0 >= 0 && p0 + M <= Lmax;
-        seg_start[sg + 1] = ok ? max(1, (p0 + 15) >> 4) : 0;
+        seg_start[sg + 1] = ok ? max(1, (p0 + 15) >> 4) + VISIT_TILES : 0;
     }
     if (tid == 0) seg_start[0] = 0;
     __syncthreads();
@@ -145,13 +160,15 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
                                                            int Lmax, int min_tiles, int n_slots) {
     constexpr int R = 4 * M;
     __shared__ int seg_start[MAX_SEG + 1];
-    __shared__ __align__(16) bf16_t v_s[4][16 * VL_LD];          // one V tile per wavefront; reused for the merged O below
-    __shared__ __align__(16) bf16_t k_s[4][16 * KL_LD];          // one K tile per wavefront
+    // one V tile and one K tile per wavefront, in one array: at the end the same memory holds the four wavefronts' scaled O
+    // ([4][R rows][256] f32) for the merge
+    __shared__ __align__(16) bf16_t tile_s[4 * 16 * (VL_LD + KL_LD)];
     __shared__ __align__(16) float c_s[4][16];
     __shared__ float m_s[4][16], l_s[4][16];
-    static_assert(sizeof(bf16_t) * 4 * 16 * VL_LD >= sizeof(float) * 16 * AD, "the merged O tile must fit into the V tiles");
-    float (*o_s)[AD] = reinterpret_cast<float (*)[AD]>(&v_s[0][0]);
+    static_assert(sizeof(bf16_t) * 4 * 16 * (VL_LD + KL_LD) >= sizeof(float) * 4 * 16 * AD, "the four O tiles must fit into the K / V tiles");
+    float* const mo = reinterpret_cast<float*>(tile_s);
 
+    AD_MARK(0);
     const int nseg = B * AKV;
     const int total = build_segments<M>(seg_start, slots, pos, nseg, Lmax, n_slots);
     const int per = tiles_per_wg(total, gridDim.x, min_tiles);
@@ -166,13 +183,14 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int hw = lane >> 5, cl = lane & 31;
 
+    AD_MARK(1);
   for (int sg = sg0; sg < nseg && seg_start[sg] < wt1; sg++) {
     const int ss = seg_start[sg], se = seg_start[sg + 1];
     if (se == ss) continue;                                      // a skipped row
     const int kvh = sg % AKV, b = sg / AKV;
     const int slot = slots[b], p0 = pos[b];
     const bool first = wt0 <= ss;                                // this workgroup holds the segment's first tile
-    const int lo = (max(wt0, ss) - ss) * 16, hi = min((min(wt1, se) - ss) * 16, p0);
+    const int lo = max(0, max(wt0, ss) - ss - VISIT_TILES) * 16, hi = min(max(0, min(wt1, se) - ss - VISIT_TILES) * 16, p0);
     const size_t pslot = (size_t)blockIdx.x + sg;
 
     // Q^T as the MFMA B operand: lane (row n, group g) holds q[row n][32 kb + 8 g .. + 8]; row n = token (n / 4), head n % 4
@@ -195,8 +213,8 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     const size_t pbase = ((size_t)slot * AKV + kvh) * Lmax * AD;
     const bf16_t* kbase = Kp + pbase;
     const bf16_t* vbase = Vp + pbase;
-    bf16_t* vl = v_s[w];
-    bf16_t* kl = k_s[w];
+    bf16_t* vl = tile_s + w * (16 * VL_LD);
+    bf16_t* kl = tile_s + 4 * (16 * VL_LD) + w * (16 * KL_LD);
     const int ntiles = hi > lo ? (hi - lo + 15) / 16 : 0;
     if (w < ntiles) {
         // Row addresses of a tile: key 2i (lower half wavefront) / 2i + 1 (upper half), 8 columns per lane, so one load covers
@@ -212,6 +230,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
 #pragma unroll
         for (int i = 0; i < 8; i++) vv[i] = __builtin_nontemporal_load(row_ptr(vbase, w, i));
         __builtin_amdgcn_sched_barrier(0);
+        AD_MARK(2);
         for (int t = w; t < ntiles; t += 4) {
             const int tn = t + 4 < ntiles ? t + 4 : t;           // the last step re-reads its own tile
             const int nvalid = min(16, hi - (lo + t * 16));
@@ -242,6 +261,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
             wave_lds_sync();
         }
     }
+    AD_MARK(3);
     if (first && w == 3) {
         // The M new keys of this sequence, straight from the inputs (batch.py:143-145), with the causal rule among them:
         // key i is visible to query token j only if i <= j.  Not pipelined: it runs once per sequence.
@@ -280,6 +300,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
         }
     }
 
+    AD_MARK(4);
     // ---- merge the 4 wavefronts (deterministic order); lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
@@ -295,21 +316,22 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
         const float mm = fmaxf(fmaxf(m_s[0][row], m_s[1][row]), fmaxf(m_s[2][row], m_s[3][row]));
         f[r] = __expf(m_s[w][row] - mm);
     }
-    for (int ww = 0; ww < 4; ww++) {
-        if (w == ww && 4 * g < R) {
+    // every wavefront leaves its scaled O in its own part of LDS; then each thread adds the four for R / 4 groups of four
+    // columns, in a fixed order, and writes the partial result
+    if (4 * g < R) {
 #pragma unroll
-            for (int j = 0; j < 16; j++)
+        for (int j = 0; j < 16; j++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    float* dst = &o_s[4 * g + r][16 * j + n];
-                    *dst = (ww == 0 ? 0.f : *dst) + O[j][r] * f[r];
-                }
-        }
-        __syncthreads();
+            for (int r = 0; r < 4; r++) mo[(w * R + 4 * g + r) * AD + 16 * j + n] = O[j][r] * f[r];
     }
+    __syncthreads();
+    AD_MARK(5);
     float* po = part_o + pslot * R * AD;
-    for (int i = tid; i < R * AD / 4; i += 256)
-        reinterpret_cast<f32x4*>(po)[i] = reinterpret_cast<const f32x4*>(&o_s[0][0])[i];
+#pragma unroll
+    for (int i = tid; i < R * AD / 4; i += 256) {
+        const f32x4* src = reinterpret_cast<const f32x4*>(mo) + i;
+        reinterpret_cast<f32x4*>(po)[i] = (src[0] + src[R * AD / 4]) + (src[2 * (R * AD / 4)] + src[3 * (R * AD / 4)]);
+    }
     if (tid < R) {
         const float mm = fmaxf(fmaxf(m_s[0][tid], m_s[1][tid]), fmaxf(m_s[2][tid], m_s[3][tid]));
         float ll = 0.f;
@@ -318,6 +340,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
         part_ml[(pslot * R + tid) * 2 + 1] = ll;
     }
     __syncthreads();                                             // the LDS tiles are reused by the next segment
+    AD_MARK(6);
   }
 }
 
