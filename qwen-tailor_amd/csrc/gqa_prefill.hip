@@ -527,8 +527,10 @@ int cu_count() {                       // CUs of the current device (256 if the 
 inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 304; }
 
 // The key split of a launch: tmax = 0 (none) or the tiles per part, parts = grid width, split_blocks = blocks with several parts.
-// Only launches that leave at least half of the CUs without a workgroup are split (up to 1024 query rows: a short continuation
-// of a long prefix, a short prompt); a part then holds at least the launch's average tiles per CU, and at least 8.  A workgroup costs
+// Only launches that leave CUs without a workgroup are split (fewer than 2048 query rows: a short continuation of a long
+// prefix, a short prompt), and only as far as the idle CUs go: a part holds the smallest number of tiles (from the launch's
+// average per CU, at least 8) with which all parts are resident at once, and the split must shorten the longest workgroup
+// by six tiles or more to pay for the merge launch.  A workgroup costs
 // about 6 us beyond its tiles (dispatch, Q and first-tile latency, the output stores): measured at S = 2048 (256 workgroups,
 // 57 us unsplit) every part size from 4 to 32 tiles came out between 53 and 61 us before the parts were even merged.
 struct KeySplit {
@@ -540,7 +542,7 @@ KeySplit plan_split(int S, int L, int q_pos0) {
     KeySplit ks;
     if (S < 1 || two_heads_per_wave(S)) return ks;
     const int nb = (S + 15) / 16, cus = cu_count();
-    if (nb * AKV > cus / 2) return ks;
+    if (nb * AKV >= cus) return ks;
     long total = 0;
     int longest = 0;
     for (int i = 0; i < nb; i++) {
@@ -553,7 +555,7 @@ KeySplit plan_split(int S, int L, int q_pos0) {
     const long p = (q_pos0 + 15) >> 4;
     int tmax = (int)std::max(8L, (total * AKV + cus - 1) / cus);
     while (tmax < longest && (parts_upto(p + nb, 4L * tmax) - parts_upto(p, 4L * tmax)) * AKV > cus) tmax++;
-    if (tmax >= longest) return ks;
+    if (longest - tmax < 6) return ks;                           // the merge launch costs about as much as six tiles
     const long c = 4L * tmax;
     ks.tmax = tmax;
     ks.parts = parts_upto(p + nb, c) - parts_upto(p, c);
@@ -573,10 +575,10 @@ long qt_gqa_prefill_workspace_bytes_for(int S, int L, int q_pos0) {
     return ks.tmax ? ks.parts * AKV * (long)(PART_O + PART_ML) * 4 : 0;
 }
 // An upper bound of the above over every launch with at most L keys (S <= L, q_pos0 = L - S or smaller): a part holds at least
-// total / CUs tiles, so there are at most CUs / 2 + 2 * blocks parts per KV head, and a split launch has at most CUs / 4 blocks.
+// total / CUs tiles, so there are at most CUs / 2 + 2 * blocks parts per KV head, and a split launch has fewer than CUs / 2 blocks.
 long qt_gqa_prefill_workspace_bytes(int L) {
     if (L < 0) return -1;
-    const long cus = cu_count(), nb = std::min((long)(L + 15) / 16, cus / (2 * AKV));
+    const long cus = cu_count(), nb = std::min((long)(L + 15) / 16, cus / AKV);
     return (cus + AKV * (2 * nb + 2)) * (long)(PART_O + PART_ML) * 4;
 }
 
