@@ -79,6 +79,27 @@ def test_null_and_dimension_errors_from_the_c_abi():
     assert lib.qt_fused_gemv(ctypes.c_void_p(8), p16, z, p16, 4, 64, 1024, 0, z) == -2
 
 
+def test_prefill_attention_split_plan_on_the_host():
+    """The key split of the causal prefill attention is planned on the host (no GPU call computes anything here): which launches
+    are split, how much workspace they use, and that the bound for a key count covers every launch below it."""
+    import qwen_tailor_amd as qt
+    lib = qt._lib.lib()
+    need, bound = lib.qt_gqa_prefill_workspace_bytes_for, lib.qt_gqa_prefill_workspace_bytes
+    z, p16 = ctypes.c_void_p(0), ctypes.c_void_p(16)
+    assert need(-1, 8, 0) == -1 and need(8, 0, 0) == -1 and bound(-1) == -1
+    assert need(2048, 2048, 0) == 0 and need(8192, 8192, 0) == 0          # a workgroup per CU or more: not split
+    assert need(0, 64, 64) == 0 and need(5, 5, 0) == 0                    # nothing to split
+    part = 4 * (16 * 256 + 2 * 16) * 4                                    # bytes of one part: O, m, l of 16 rows x 4 heads
+    for S, P0 in ((64, 8000), (16, 32000), (1024, 0), (1536, 1000), (300, 4001), (1, 4095)):
+        n = need(S, S + P0, P0)
+        assert n > 0 and n % (2 * part) == 0, (S, P0, n)                  # whole parts, the same number for both KV heads
+        assert n // part <= 256 + 1, (S, P0, n)                           # all parts resident at once (at most one per CU; 256 CUs assumed without a GPU)
+        assert n <= bound(S + P0), (S, P0)
+    # queries past the keys are refused before anything is launched
+    assert lib.qt_gqa_prefill_causal(p16, p16, p16, p16, z, 0, 32, 40, 9, 32 * 256, 40 * 256, z) == -1
+    assert lib.qt_gqa_prefill_causal(p16, p16, p16, p16, ctypes.c_void_p(8), 0, 32, 40, 8, 32 * 256, 40 * 256, z) == -2
+
+
 def test_product_does_not_import_the_oracle():
     pkg = os.path.join(ROOT, "qwen-tailor_amd")
     for dirpath, _, files in os.walk(pkg):
