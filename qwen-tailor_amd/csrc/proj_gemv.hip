@@ -421,7 +421,9 @@ int qt_fused_gemv(const void* W, const void* x, const void* res, void* y, int M,
     const int kc = K / 32;
     // the wide projections of a decode batch: rows in LDS.  From four rows on (in_proj, one row 6.6 us either way; 4 / 16 /
     // 64 rows: 6.9 / 7.0 / 9.7 us against 7.0 / 8.4 / 11.9 us for the kernels below)
-    if (K == XK && N >= 4096 && (N & 3) == 0 && M >= 4 && M <= 64) {
+    // (its 8-byte stores and residual loads want y and res aligned to 8 bytes; anything else takes the general kernels)
+    if (K == XK && N >= 4096 && (N & 3) == 0 && M >= 4 && M <= 64 &&
+        ((reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(res)) & 7u) == 0) {
         const int cus = cu_count();
         if (M <= 16)
             launch_xlds_ms<1>(epilogue, (const bf16_t*)W, (const bf16_t*)x, (const bf16_t*)res, (bf16_t*)y, M, N, stream, cus);

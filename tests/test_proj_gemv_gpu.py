@@ -3,6 +3,8 @@ rms_rows) against the numpy restatement.  rms_rows is bit exact.  The product ac
 float32 on the matrix cores (the reference accumulates them in float32 in another order, the restatement in float64), so its
 bf16 outputs may differ by one rounding step: the tolerance is 1 bf16 ulp (2 after the add / swiglu epilogues, which round a
 second time) plus 2e-5 of the largest output for sums that nearly cancel, and 2e-3 relative in the l2 norm."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -73,6 +75,35 @@ def test_fused_gemv_exact_on_small_integers(qt, dev):
     x = torch.randint(-2, 3, (M, K), generator=g).float().numpy()
     got = qt.kernels.fused_gemv(to_dev(W, dev, BF16), to_dev(x, dev, BF16))
     check_equal("integer product", to_np(got), O.fused_gemv(W, x))
+
+
+@pytest.mark.parametrize("M,N,epi", [(33, 4112, 0), (64, 8224, 1), (16, 4096, 2), (5, 5120, 0)])
+def test_wide_projection_exact_and_any_output_alignment(qt, dev, M, N, epi):
+    """The kernel for wide outputs at K = 1024 (rows in LDS) on small-integer data, where every order of summation gives the
+    same bits; and the same call through the C ABI with y and res 2 bytes off an 8-byte boundary (the general kernels take
+    over) must give the same bits."""
+    from qwen_tailor_amd import _lib as QL
+    g = torch.Generator().manual_seed(M + N + epi)
+    K = 1024
+    W = torch.randint(-3, 4, (N, K), generator=g).float().numpy()
+    x = torch.randint(-2, 3, (M, K), generator=g).float().numpy()
+    res = torch.randint(-9, 10, (M, N), generator=g).float().numpy() if epi == 1 else None
+    dW, dx = to_dev(W, dev, BF16), to_dev(x, dev, BF16)
+    dres = None if res is None else to_dev(res, dev, BF16)
+    got = qt.kernels.fused_gemv(dW, dx, res=dres, swiglu=epi == 2)
+    want = O.fused_gemv(W, x, res=res, swiglu=epi == 2)
+    if epi == 2:
+        _close("integer swiglu", to_np(got), want, 1)            # silu of an integer is not an integer: within one rounding
+    else:
+        check_equal("integer product", to_np(got), want)
+    NO = N // 2 if epi == 2 else N
+    ybuf = torch.zeros(M * NO + 8, dtype=BF16, device=dev)
+    rbuf = torch.zeros(M * N + 8, dtype=BF16, device=dev)
+    if dres is not None:
+        rbuf[1:1 + M * N] = dres.reshape(-1)
+    QL.call("qt_fused_gemv", QL.ptr(dW), QL.ptr(dx), ctypes.c_void_p(rbuf.data_ptr() + 2) if dres is not None else None,
+            ctypes.c_void_p(ybuf.data_ptr() + 2), M, N, K, epi, QL.stream())
+    assert torch.equal(ybuf[1:1 + M * NO].reshape(M, NO), got), "outputs off an 8-byte boundary differ"
 
 
 def test_fused_gemv_prologues_and_leading_dims(qt, dev):
