@@ -121,8 +121,8 @@ int qt_gdn_phase_b_norm(const void* ops, const float* U, const float* gC, void* 
 /* Causal prefill attention: the mx.fast.scaled_dot_product_attention(..., mask="causal") call of the full-attention layers
  * (qwen35/model.py:160-167, qwen35/prefill.py:468).  q, out [8][S][256] bf16 with head stride q_head_stride (elements);
  * K, V [2][>=L][256] bf16 with head stride kv_head_stride; query i sits at position q_pos0 + i and sees keys 0..q_pos0+i.
- * Launches that would leave CUs idle (fewer than 2048 query rows: a short prompt, or a short continuation of a long
- * prefix) are split along the keys; the parts meet in `workspace` and a second kernel combines them.  qt_gqa_prefill_workspace_bytes_for gives the bytes this launch uses (0: not split),
+ * Launches that would leave CUs idle (a prompt of up to about 2800 rows, or rows continuing a long prefix) are split along
+ * the keys; the parts meet in `workspace` and a second kernel combines them.  qt_gqa_prefill_workspace_bytes_for gives the bytes this launch uses (0: not split),
  * qt_gqa_prefill_workspace_bytes an upper bound for every launch with at most L keys.  With a null or smaller workspace the
  * launch runs unsplit: same results up to rounding, slower.  Requires q_pos0 + S <= L. */
 long qt_gqa_prefill_workspace_bytes(int L);

@@ -84,18 +84,20 @@ __device__ __forceinline__ float max_over_groups(float x) {
 // it is hoisted to the top of every tile and holds 128 VALU registers through the score phase).
 #define PIN_ACC(x) asm volatile("" : "+a"(x))
 
-// Key split (NH = 1 launches only).  A causal launch with about one workgroup per CU is as slow as its longest row block, twice
-// the average.  With tmax > 0 the tiles of a 16-row block are cut into parts of tmax tiles, one workgroup per part; a block
-// with more than one part leaves unnormalised partial results (O, reference point m, row sums l) in the workspace and
-// attn_prefill_merge_kernel combines them.  Block i counts ceil((p + i + 1) / c) parts, p = ceil(q_pos0 / 16), c = 4 tmax (16
-// rows advance the visible keys by a quarter tile), which is never fewer than its tiles need (a part may be empty); the
-// parts of blocks 0 .. r-1 are then parts_upto(p + r, c) - parts_upto(p, c), and a workgroup inverts that sum to find its part.
+// Key split.  A causal launch with few workgroups is as slow as its longest row block, twice the average.  With tmax > 0 the
+// tiles of a row block (RB = 16 or 32 rows) are cut into parts of tmax tiles, one workgroup per part; a block with more than
+// one part leaves unnormalised partial results (O, reference point m, row sums l) in the workspace and
+// attn_prefill_merge_kernel combines them.  Block i counts ceil((p + i + 1) / c) parts, p = ceil(q_pos0 / RB),
+// c = (64 / RB) tmax (RB rows advance the visible keys by RB / 64 of a tile), which is never fewer than its tiles need (a part
+// may be empty); the parts of blocks 0 .. r-1 are then parts_upto(p + r, c) - parts_upto(p, c), and a workgroup inverts that
+// sum to find its part.
 __host__ __device__ inline long parts_upto(long n, long c) {      // sum over j = 1 .. n of ceil(j / c)
     const long k = n / c;
     return c * (k * (k + 1) / 2) + (n - k * c) * (k + 1);
 }
-constexpr int PART_O = 4 * 16 * AD;    // floats of one part's O: [4 heads][16 rows][256]
-constexpr int PART_ML = 4 * 2 * 16;    // ... and of its m, l: [4 heads][m | l][16 rows]
+// floats of one part's O, [4 heads][RB rows][256], and of its m, l, [4 heads][m | l][RB rows] (RB = rows of a block: 16 or 32)
+constexpr int part_o_floats(int RB) { return 4 * RB * AD; }
+constexpr int part_ml_floats(int RB) { return 4 * 2 * RB; }
 
 // NH = heads per wavefront: 2 (32 query rows per workgroup, as described above) for long sequences; 1 (16 rows per workgroup,
 // one head per wavefront: twice the workgroups, LDS-bound) when the launch would otherwise leave CUs idle.
@@ -115,8 +117,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     constexpr int RB = 16 * NH;
     int rb = gridDim.x - 1 - blockIdx.x;                         // long rows first
     int part = 0, nparts = 1;
-    if (NH == 1 && tmax > 0) {                                   // blockIdx.x counts parts, again from the long end
-        const int c = 4 * tmax, p = (q_pos0 + 15) >> 4;
+    if (tmax > 0) {                                              // blockIdx.x counts parts, again from the long end
+        const int c = (KT / RB) * tmax, p = (q_pos0 + RB - 1) / RB;
         const long y = (long)rb + parts_upto(p, c);              // parts_upto(nn) <= y < parts_upto(nn + 1), nn = p + row block
         int k = 0;
         while ((long)c * ((k + 1) * (k + 2) / 2) <= y) k++;
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     const int kend_w = r0 < S ? min(L, q_pos0 + min(r0 + 15, S - 1) + 1) : 0;  // keys any row of this wavefront sees
     const int ntiles_w = (kend_w + KT - 1) / KT;
     // this workgroup's tiles [ta, tb); tw: where this wavefront's rows end
-    const int ta = part * (NH == 1 && tmax > 0 ? tmax : 0), tb = NH == 1 && tmax > 0 ? min(ntiles, ta + tmax) : ntiles;
+    const int ta = part * tmax, tb = tmax > 0 ? min(ntiles, ta + tmax) : ntiles;
     const int tw = min(ntiles_w, tb);
 
     // Q^T as the B operand of the score MFMA: lane (row n, group g) holds q[row][32 kb + 8 g .. + 8], for both heads
@@ -438,22 +440,26 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         }
     }
     AP_STORE();
-    if (NH == 1 && nparts > 1) {
-        // One part of several: leave O, m, l of this wavefront's head as they are.  A row that sees no key of this part (its
+    if (nparts > 1) {
+        // One part of several: leave O, m, l of this wavefront's heads as they are.  A row that sees no key of this part (its
         // last key lies before the part's first) has exponentiated masked scores against a masked maximum: it is written as
         // the neutral element (m = NEG, l = 0, O = 0).
-        const int first_key = ta * KT;
-        float* po = part_o + (slot * 4 + w) * (16 * AD);
-        float* pml = part_ml + (slot * 4 + w) * 32;
+        const int first_key = ta * KT, lr0 = r0 - rb * RB;       // this wavefront's first row within the block
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int lr = 4 * g + r;
-            const bool seen = q_pos0 + r0 + lr >= first_key;
+        for (int hh = 0; hh < NH; hh++) {
+            const int hq = (NH == 2 ? 2 * (w & 1) : w) + hh;     // head within the KV group
+            float* po = part_o + (slot * 4 + hq) * (RB * AD);
+            float* pml = part_ml + (slot * 4 + hq) * (2 * RB);
 #pragma unroll
-            for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n] = seen ? O[0][j][r] : 0.f;
-            if (n == 0) pml[16 + lr] = seen ? Lsum[0][r] : 0.f;
+            for (int r = 0; r < 4; r++) {
+                const int lr = lr0 + 4 * g + r;
+                const bool seen = q_pos0 + rb * RB + lr >= first_key;
+#pragma unroll
+                for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n] = seen ? O[hh][j][r] : 0.f;
+                if (n == 0) pml[RB + lr] = seen ? Lsum[hh][r] : 0.f;
+            }
+            if (g == 0) pml[lr0 + n] = my_last >= first_key ? m_run[hh] : NEG;
         }
-        if (g == 0) pml[n] = my_last >= first_key ? m_run[0] : NEG;
         return;
     }
     // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n, and of the row sums (any column)
@@ -473,45 +479,50 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
 }
 
 // Combines the parts of the row blocks that were split: grid = (split blocks, KV heads, 4 heads of the group); thread (row,
-// 16-column group) of the 16 x 256 block.  out = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p, parts in order; a thread's
-// loads of O do not depend on the factors, so all parts are in flight together.
+// 16-column group) of 16 x 256 outputs at a time.  out = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p, parts in order; a
+// thread's loads of O do not depend on the factors, so all parts are in flight together.
+template <int RB>
 __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                                  bf16_t* __restrict__ out, int S, int q_pos0, int tmax, long slots_per_kv,
                                                                  long q_head_stride) {
-    const int c = 4 * tmax, p = (q_pos0 + 15) >> 4;
+    constexpr int PO = part_o_floats(RB), PML = part_ml_floats(RB);
+    const int c = (KT / RB) * tmax, p = (q_pos0 + RB - 1) / RB;
     const int rb = max(0, c - p) + blockIdx.x;                   // the first block with two parts is c - p
     const int np = (p + rb) / c + 1;
     const size_t slot0 = (size_t)blockIdx.y * slots_per_kv + (size_t)(parts_upto(p + rb, c) - parts_upto(p, c));
-    const int hq = blockIdx.z, lr = threadIdx.x >> 4, cg = threadIdx.x & 15;
-    if (rb * 16 + lr >= S) return;
-    const float* po = part_o + (slot0 * 4 + hq) * (16 * AD) + lr * AD + cg * 16;
-    const float* pml = part_ml + (slot0 * 4 + hq) * 32 + lr;
-    float m = NEG;
-    for (int pp = 0; pp < np; pp++) m = fmaxf(m, pml[(size_t)pp * PART_ML]);
-    float l = 0.f;
-    f32x4 acc[4];
+    const int hq = blockIdx.z, cg = threadIdx.x & 15;
 #pragma unroll
-    for (int i = 0; i < 4; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int lr = threadIdx.x >> 4; lr < RB; lr += 16) {
+        if (rb * RB + lr >= S) return;
+        const float* po = part_o + (slot0 * 4 + hq) * (RB * AD) + lr * AD + cg * 16;
+        const float* pml = part_ml + (slot0 * 4 + hq) * (2 * RB) + lr;
+        float m = NEG;
+        for (int pp = 0; pp < np; pp++) m = fmaxf(m, pml[(size_t)pp * PML]);
+        float l = 0.f;
+        f32x4 acc[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 2
-    for (int pp = 0; pp < np; pp++) {
-        f32x4 o[4];
+        for (int pp = 0; pp < np; pp++) {
+            f32x4 o[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) o[i] = reinterpret_cast<const f32x4*>(po + (size_t)pp * PART_O)[i];
-        const float f = __builtin_amdgcn_exp2f(pml[(size_t)pp * PART_ML] - m);
-        l += f * pml[(size_t)pp * PART_ML + 16];
+            for (int i = 0; i < 4; i++) o[i] = reinterpret_cast<const f32x4*>(po + (size_t)pp * PO)[i];
+            const float f = __builtin_amdgcn_exp2f(pml[(size_t)pp * PML] - m);
+            l += f * pml[(size_t)pp * PML + RB];
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[i] += f * o[i];
+            for (int i = 0; i < 4; i++) acc[i] += f * o[i];
+        }
+        const float inv = 1.0f / l;
+        uint32_t pk[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            pk[2 * i] = pack_bf(acc[i][0] * inv, acc[i][1] * inv);
+            pk[2 * i + 1] = pack_bf(acc[i][2] * inv, acc[i][3] * inv);
+        }
+        u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)(blockIdx.y * (AH / AKV) + hq) * q_head_stride + (size_t)(rb * RB + lr) * AD + cg * 16);
+        dst[0] = u32x4{pk[0], pk[1], pk[2], pk[3]};
+        dst[1] = u32x4{pk[4], pk[5], pk[6], pk[7]};
     }
-    const float inv = 1.0f / l;
-    uint32_t pk[8];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        pk[2 * i] = pack_bf(acc[i][0] * inv, acc[i][1] * inv);
-        pk[2 * i + 1] = pack_bf(acc[i][2] * inv, acc[i][3] * inv);
-    }
-    u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)(blockIdx.y * (AH / AKV) + hq) * q_head_stride + (size_t)(rb * 16 + lr) * AD + cg * 16);
-    dst[0] = u32x4{pk[0], pk[1], pk[2], pk[3]};
-    dst[1] = u32x4{pk[4], pk[5], pk[6], pk[7]};
 }
 
 }  // namespace
@@ -534,33 +545,55 @@ inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 304; }
 // about 6 us beyond its tiles (dispatch, Q and first-tile latency, the output stores): measured at S = 2048 (256 workgroups,
 // 57 us unsplit) every part size from 4 to 32 tiles came out between 53 and 61 us before the parts were even merged.
 struct KeySplit {
+    int nh = 1;            // heads per wavefront: row blocks of 16 nh rows
     int tmax = 0;
     long parts = 0;
     int split_blocks = 0;
+    long bytes() const { return parts * AKV * (long)(part_o_floats(16 * nh) + part_ml_floats(16 * nh)) * 4; }
 };
-KeySplit plan_split(int S, int L, int q_pos0) {
+KeySplit plan_split_nh(int S, int L, int q_pos0, int nh, int min_gain) {
     KeySplit ks;
-    if (S < 1 || two_heads_per_wave(S)) return ks;
-    const int nb = (S + 15) / 16, cus = cu_count();
-    if (nb * AKV >= cus) return ks;
+    ks.nh = nh;
+    const int RB = 16 * nh, nb = (S + RB - 1) / RB, cus = cu_count();
+    if (S < 1 || nb * AKV >= cus) return ks;
     long total = 0;
     int longest = 0;
     for (int i = 0; i < nb; i++) {
-        const int kend = std::min(L, q_pos0 + std::min(16 * i + 15, S - 1) + 1), nt = (kend + KT - 1) / KT;
+        const int kend = std::min(L, q_pos0 + std::min(RB * i + RB - 1, S - 1) + 1), nt = (kend + KT - 1) / KT;
         total += nt;
         longest = std::max(longest, nt);
     }
     // the smallest part size (from the average per CU, at least 8 tiles) whose parts are all resident at once: a CU that has
     // to run a second part pays the per-workgroup cost twice
-    const long p = (q_pos0 + 15) >> 4;
+    const long p = (q_pos0 + RB - 1) / RB, cpt = KT / RB;
     int tmax = (int)std::max(8L, (total * AKV + cus - 1) / cus);
-    while (tmax < longest && (parts_upto(p + nb, 4L * tmax) - parts_upto(p, 4L * tmax)) * AKV > cus) tmax++;
-    if (longest - tmax < 6) return ks;                           // the merge launch costs about as much as six tiles
-    const long c = 4L * tmax;
+    while (tmax < longest && (parts_upto(p + nb, cpt * tmax) - parts_upto(p, cpt * tmax)) * AKV > cus) tmax++;
+    if (longest - tmax < min_gain) return ks;                    // the merge launch has to be earned
+    const long c = cpt * tmax;
     ks.tmax = tmax;
     ks.parts = parts_upto(p + nb, c) - parts_upto(p, c);
     ks.split_blocks = nb - (int)std::max(0L, c - p);
     return ks;
+}
+// The form of a launch, by measurement (us at q_pos0 = 0, one head per wavefront in its best form / two heads with the split:
+// S = 1280 30.6 / 35.7, 1536 39.4 / 37.7, 2048 57.5 / 47.0, 2560 70.2 / 64.6, 3072 84.4 / 88.5, 4096 130 / 132; after a prefix
+// two heads win by more: 1536 rows after 1000 keys 63.4 / 52.8, 2048 after 6000 201 / 174):
+//   from about 4800 rows on     two heads per wavefront, unsplit (enough 32-row blocks to balance themselves);
+//   from about 1500 rows on     two heads per wavefront with the key split, where the launch leaves room for it and, for a
+//                               whole prompt, up to about 2800 rows (a tile of a 32-row block costs 2.4 us against 2 x 1.6 -
+//                               2 us for two 16-row blocks, but its parts are twice the size);
+//   everything else             one head per wavefront, split if CUs would idle.
+KeySplit plan_split(int S, int L, int q_pos0) {
+    if (two_heads_per_wave(S)) {
+        KeySplit ks;
+        ks.nh = 2;
+        return ks;
+    }
+    if (S >= 1472 && (q_pos0 > 0 || S <= 2816)) {
+        const KeySplit ks = plan_split_nh(S, L, q_pos0, 2, 4);
+        if (ks.tmax) return ks;
+    }
+    return plan_split_nh(S, L, q_pos0, 1, 6);
 }
 
 }  // namespace
@@ -572,14 +605,17 @@ extern "C" {
 long qt_gqa_prefill_workspace_bytes_for(int S, int L, int q_pos0) {
     if (S < 0 || L < 1 || q_pos0 < 0) return -1;
     const KeySplit ks = plan_split(S, L, q_pos0);
-    return ks.tmax ? ks.parts * AKV * (long)(PART_O + PART_ML) * 4 : 0;
+    return ks.tmax ? ks.bytes() : 0;
 }
 // An upper bound of the above over every launch with at most L keys (S <= L, q_pos0 = L - S or smaller): a part holds at least
-// total / CUs tiles, so there are at most CUs / 2 + 2 * blocks parts per KV head, and a split launch has fewer than CUs / 2 blocks.
+// total / CUs tiles, so there are at most CUs / 2 + 2 * blocks parts per KV head, a split launch has fewer than CUs / 2 blocks,
+// and a part of a 16-row block is half the size of one of a 32-row block.
 long qt_gqa_prefill_workspace_bytes(int L) {
     if (L < 0) return -1;
-    const long cus = cu_count(), nb = std::min((long)(L + 15) / 16, cus / AKV);
-    return (cus + AKV * (2 * nb + 2)) * (long)(PART_O + PART_ML) * 4;
+    const long cus = cu_count(), nb16 = std::min((long)(L + 15) / 16, cus / AKV), nb32 = std::min((long)(L + 31) / 32, cus / AKV);
+    const long b16 = (cus + AKV * (2 * nb16 + 2)) * (long)(part_o_floats(16) + part_ml_floats(16)) * 4;
+    const long b32 = (cus + AKV * (2 * nb32 + 2)) * (long)(part_o_floats(32) + part_ml_floats(32)) * 4;
+    return std::max(b16, b32);
 }
 
 // q, out [8][S][256] bf16 (head stride q_head_stride elements), K, V [2][>=L][256] bf16 (head stride kv_head_stride):
@@ -593,30 +629,30 @@ int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out
     for (const void* p : {q, K, V, (const void*)out, (const void*)workspace})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if ((q_head_stride | kv_head_stride) & 7) return QT_ERR_ALIGN;
-    // two heads per wavefront from about 4800 query rows on (measured: one head per wavefront 140 us at S = 4096 and 296 us at
-    // S = 6144, two heads 156 us and 237 us); below that, 16-row blocks give twice the workgroups
-    if (two_heads_per_wave(S)) {
-        hipLaunchKernelGGL(attn_prefill_kernel<2>, dim3((S + 31) / 32, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
-                           (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, 0, (float*)nullptr,
-                           (float*)nullptr);
-        QT_CHECK_LAUNCH();
-        return QT_OK;
-    }
     KeySplit ks = plan_split(S, L, q_pos0);
-    if (ks.tmax && (!workspace || workspace_bytes < ks.parts * AKV * (long)(PART_O + PART_ML) * 4)) ks = KeySplit();
-    if (!ks.tmax) {
-        hipLaunchKernelGGL(attn_prefill_kernel<1>, dim3((S + 15) / 16, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
-                           (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, 0, (float*)nullptr,
-                           (float*)nullptr);
-        QT_CHECK_LAUNCH();
-        return QT_OK;
+    if (ks.tmax && (!workspace || workspace_bytes < ks.bytes())) {          // no room for the parts: the unsplit form
+        ks = KeySplit();
+        ks.nh = two_heads_per_wave(S) ? 2 : 1;
     }
-    float* part_o = (float*)workspace;
-    float* part_ml = part_o + (size_t)ks.parts * AKV * PART_O;
-    hipLaunchKernelGGL(attn_prefill_kernel<1>, dim3((unsigned)ks.parts, AKV), dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K,
-                       (const bf16_t*)V, (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
-    hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)ks.split_blocks, AKV, AH / AKV), dim3(256), 0, stream, part_o,
-                       part_ml, (bf16_t*)out, S, q_pos0, ks.tmax, ks.parts, q_head_stride);
+    const int RB = 16 * ks.nh;
+    const dim3 grid(ks.tmax ? (unsigned)ks.parts : (unsigned)((S + RB - 1) / RB), AKV);
+    float* part_o = ks.tmax ? (float*)workspace : nullptr;
+    float* part_ml = ks.tmax ? part_o + (size_t)ks.parts * AKV * part_o_floats(RB) : nullptr;
+    if (ks.nh == 2)
+        hipLaunchKernelGGL(attn_prefill_kernel<2>, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
+                           (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
+    else
+        hipLaunchKernelGGL(attn_prefill_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
+                           (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
+    if (ks.tmax) {
+        const dim3 mgrid((unsigned)ks.split_blocks, AKV, AH / AKV);
+        if (ks.nh == 2)
+            hipLaunchKernelGGL(attn_prefill_merge_kernel<32>, mgrid, dim3(256), 0, stream, part_o, part_ml, (bf16_t*)out, S, q_pos0,
+                               ks.tmax, ks.parts, q_head_stride);
+        else
+            hipLaunchKernelGGL(attn_prefill_merge_kernel<16>, mgrid, dim3(256), 0, stream, part_o, part_ml, (bf16_t*)out, S, q_pos0,
+                               ks.tmax, ks.parts, q_head_stride);
+    }
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

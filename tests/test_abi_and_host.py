@@ -87,13 +87,14 @@ def test_prefill_attention_split_plan_on_the_host():
     need, bound = lib.qt_gqa_prefill_workspace_bytes_for, lib.qt_gqa_prefill_workspace_bytes
     z, p16 = ctypes.c_void_p(0), ctypes.c_void_p(16)
     assert need(-1, 8, 0) == -1 and need(8, 0, 0) == -1 and bound(-1) == -1
-    assert need(2048, 2048, 0) == 0 and need(8192, 8192, 0) == 0          # a workgroup per CU or more: not split
+    assert need(4096, 4096, 0) == 0 and need(8192, 8192, 0) == 0          # a workgroup per CU or more: not split
     assert need(0, 64, 64) == 0 and need(5, 5, 0) == 0                    # nothing to split
     part = 4 * (16 * 256 + 2 * 16) * 4                                    # bytes of one part: O, m, l of 16 rows x 4 heads
-    for S, P0 in ((64, 8000), (16, 32000), (1024, 0), (1536, 1000), (300, 4001), (1, 4095)):
+    for S, P0 in ((64, 8000), (16, 32000), (1024, 0), (1536, 1000), (300, 4001), (1, 4095), (2048, 0), (2048, 6000)):
         n = need(S, S + P0, P0)
-        assert n > 0 and n % (2 * part) == 0, (S, P0, n)                  # whole parts, the same number for both KV heads
-        assert n // part <= 256 + 1, (S, P0, n)                           # all parts resident at once (at most one per CU; 256 CUs assumed without a GPU)
+        size = part * (2 if S >= 1472 else 1)                             # from about 1500 rows on the row blocks are 32 rows
+        assert n > 0 and n % (2 * size) == 0, (S, P0, n)                  # whole parts, the same number for both KV heads
+        assert n // size <= 256 + 1, (S, P0, n)                           # all parts resident at once (at most one per CU; 256 CUs assumed without a GPU)
         assert n <= bound(S + P0), (S, P0)
     # queries past the keys are refused before anything is launched
     assert lib.qt_gqa_prefill_causal(p16, p16, p16, p16, z, 0, 32, 40, 9, 32 * 256, 40 * 256, z) == -1
