@@ -478,8 +478,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     }
 }
 
-// Combines the parts of the row blocks that were split: grid = (split blocks, KV heads, 4 heads of the group); thread (row,
-// 16-column group) of 16 x 256 outputs at a time.  out = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p, parts in order; a
+// Combines the parts of the row blocks that were split: grid = (split blocks, KV heads, 4 heads of the group x 16-row halves of
+// a block); thread (row, 16-column group) of 16 x 256 outputs.  out = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p, parts in order; a
 // thread's loads of O do not depend on the factors, so all parts are in flight together.
 template <int RB>
 __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
@@ -490,9 +490,9 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
     const int rb = max(0, c - p) + blockIdx.x;                   // the first block with two parts is c - p
     const int np = (p + rb) / c + 1;
     const size_t slot0 = (size_t)blockIdx.y * slots_per_kv + (size_t)(parts_upto(p + rb, c) - parts_upto(p, c));
-    const int hq = blockIdx.z, cg = threadIdx.x & 15;
-#pragma unroll
-    for (int lr = threadIdx.x >> 4; lr < RB; lr += 16) {
+    const int hq = blockIdx.z / (RB / 16), cg = threadIdx.x & 15;
+    {
+        const int lr = 16 * (blockIdx.z % (RB / 16)) + (threadIdx.x >> 4);
         if (rb * RB + lr >= S) return;
         const float* po = part_o + (slot0 * 4 + hq) * (RB * AD) + lr * AD + cg * 16;
         const float* pml = part_ml + (slot0 * 4 + hq) * (2 * RB) + lr;
@@ -645,7 +645,7 @@ int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out
         hipLaunchKernelGGL(attn_prefill_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
                            (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
     if (ks.tmax) {
-        const dim3 mgrid((unsigned)ks.split_blocks, AKV, AH / AKV);
+        const dim3 mgrid((unsigned)ks.split_blocks, AKV, (AH / AKV) * ks.nh);
         if (ks.nh == 2)
             hipLaunchKernelGGL(attn_prefill_merge_kernel<32>, mgrid, dim3(256), 0, stream, part_o, part_ml, (bf16_t*)out, S, q_pos0,
                                ks.tmax, ks.parts, q_head_stride);
