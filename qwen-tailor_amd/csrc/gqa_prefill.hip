@@ -54,7 +54,7 @@ __device__ long long* ap_prof_buf;
     do {                                                                                                        \
         if ((threadIdx.x & 63) == 0)                                                                            \
             for (int i_ = 0; i_ < 8; i_++)                                                                      \
-                ap_prof_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + (threadIdx.x >> 6)) * 8 + i_] = ap_acc_[i_]; \
+                ap_prof_buf[((size_t)((blockIdx.x % AKV) * (gridDim.x / AKV) + blockIdx.x / AKV) * 4 + (threadIdx.x >> 6)) * 8 + i_] = ap_acc_[i_]; \
     } while (0)
 #else
 #define AP_MARK(i) __builtin_amdgcn_sched_barrier(0)     /* the phases of a tile are scheduled separately */
@@ -101,7 +101,7 @@ constexpr int part_ml_floats(int RB) { return 4 * 2 * RB; }
 
 // NH = heads per wavefront: 2 (32 query rows per workgroup, as described above) for long sequences; 1 (16 rows per workgroup,
 // one head per wavefront: twice the workgroups, LDS-bound) when the launch would otherwise leave CUs idle.
-// grid = (row blocks, or parts when tmax > 0; KV heads)
+// grid = (row blocks, or parts when tmax > 0) x KV heads
 template <int NH>
 __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
                                                            const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
@@ -115,9 +115,12 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     __shared__ __align__(1024) bf16_t v_s1[TILE];
     __shared__ __align__(16) float c_s[4][2][16];
     constexpr int RB = 16 * NH;
-    int rb = gridDim.x - 1 - blockIdx.x;                         // long rows first
+    // grid = items x KV heads in one dimension, the KV head varying fastest: workgroups are dispatched in the order of their
+    // index, so both heads' long row blocks come first
+    const int nitems = gridDim.x / AKV, item = blockIdx.x / AKV;
+    int rb = nitems - 1 - item;                                  // long rows first
     int part = 0, nparts = 1;
-    if (tmax > 0) {                                              // blockIdx.x counts parts, again from the long end
+    if (tmax > 0) {                                              // items are parts, again from the long end
         const int c = (KT / RB) * tmax, p = (q_pos0 + RB - 1) / RB;
         const long y = (long)rb + parts_upto(p, c);              // parts_upto(nn) <= y < parts_upto(nn + 1), nn = p + row block
         int k = 0;
@@ -127,8 +130,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         nparts = k + 1;
         rb = nn - p;
     }
-    const size_t slot = (size_t)blockIdx.y * gridDim.x + (gridDim.x - 1 - blockIdx.x);   // parts of a block: consecutive slots
-    const int kvh = blockIdx.y;
+    const int kvh = blockIdx.x % AKV;
+    const size_t slot = (size_t)kvh * nitems + (nitems - 1 - item);     // parts of a block: consecutive slots
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int h0 = kvh * (AH / AKV) + (NH == 2 ? 2 * (w & 1) : w);       // this wavefront's heads: h0 (, h0 + 1)
     const int r0 = rb * RB + (NH == 2 ? 16 * (w >> 1) : 0), row = r0 + n;   // this wavefront's 16 rows
@@ -635,7 +638,7 @@ int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out
         ks.nh = two_heads_per_wave(S) ? 2 : 1;
     }
     const int RB = 16 * ks.nh;
-    const dim3 grid(ks.tmax ? (unsigned)ks.parts : (unsigned)((S + RB - 1) / RB), AKV);
+    const dim3 grid((ks.tmax ? (unsigned)ks.parts : (unsigned)((S + RB - 1) / RB)) * AKV);
     float* part_o = ks.tmax ? (float*)workspace : nullptr;
     float* part_ml = ks.tmax ? part_o + (size_t)ks.parts * AKV * part_o_floats(RB) : nullptr;
     if (ks.nh == 2)
