@@ -239,6 +239,28 @@ def test_prefill_causal_key_split(qt, dev, S, P0, qscale):
         check_attn(f"S={S} P0={P0} row {r}", o[:, r:r + 1], ref)
 
 
+@pytest.mark.parametrize("S,P0", [(1024, 0), (2048, 0), (300, 3000), (5000, 0)])
+def test_prefill_causal_head_strides(qt, dev, S, P0):
+    """q / out with a head stride beyond S rows and K / V inside a longer cache, through the C ABI, in every form of the launch
+    (16- and 32-row blocks, split and unsplit): same bits as the contiguous call, and nothing written between the heads"""
+    from qwen_tailor_amd import _lib as QL
+    L, pad = S + P0, 5
+    g = torch.Generator().manual_seed(S + P0)
+    q = torch.randn((8, S, 256), generator=g).bfloat16().to(dev)
+    K = torch.randn((2, L + 9, 256), generator=g).bfloat16().to(dev)
+    V = torch.randn((2, L + 9, 256), generator=g).bfloat16().to(dev)
+    want = qt.attention.scaled_dot_product_attention(q[None], K[None, :, :L], V[None, :, :L], scale=256 ** -0.5, mask="causal")[0]
+    qs = torch.zeros((8, S + pad, 256), dtype=BF16, device=dev)
+    qs[:, :S] = q
+    outs = torch.full((8, S + pad, 256), 7.0, dtype=BF16, device=dev)
+    nws = QL.lib().qt_gqa_prefill_workspace_bytes_for(S, L, P0)
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+    QL.call("qt_gqa_prefill_causal", QL.ptr(qs), QL.ptr(K), QL.ptr(V), QL.ptr(outs), QL.ptr(ws), nws, S, L, P0, (S + pad) * 256, (L + 9) * 256,
+            QL.stream())
+    assert torch.equal(outs[:, :S], want), "strided call differs from the contiguous one"
+    assert bool((outs[:, S:] == 7.0).all()), "rows between the heads were written"
+
+
 def test_prefill_causal_rejects_queries_past_the_keys(qt, dev):
     from qwen_tailor_amd import _lib as QL
     t = torch.zeros((1, 8, 32, 256), dtype=BF16, device=dev)
