@@ -74,12 +74,17 @@ __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const bf16_t* __rest
 #pragma unroll
         for (int e = 0; e < 4; e++) o4[e] = __shfl_xor(y[e], 8, 64);
         if (lane < 16) {
+            // The two products and their sum are rounded one by one.  Plain operators inside a contract(off) block: the
+            // __fmul_rn / __fadd_rn helpers are ordinary operators compiled elsewhere, which the compiler contracts into one
+            // fused multiply-add after inlining (a bf16 value in ~10^5 then rounds the other way).
+#pragma clang fp contract(off)
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int i = (lane & 7) * 4 + e;
                 const float c = cs_s[0][i], sn = cs_s[1][i];
-                y[e] = lane < 8 ? BF(__fsub_rn(__fmul_rn(y[e], c), __fmul_rn(o4[e], sn)))      // y1 c - y2 s
-                                : BF(__fadd_rn(__fmul_rn(o4[e], sn), __fmul_rn(y[e], c)));     // y1 s + y2 c
+                const float own = y[e] * c, other = o4[e] * sn;
+                y[e] = BF(lane < 8 ? own - other                 // y1 c - y2 s
+                                   : other + own);               // y1 s + y2 c
             }
         }
         bf16_t* dst = is_q ? q + (r * AH + part) * AD : k + (r * AKV + (part - 8)) * AD;

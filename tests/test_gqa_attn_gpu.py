@@ -270,7 +270,7 @@ def test_prefill_causal_rejects_queries_past_the_keys(qt, dev):
 
 
 # ------------------------------------------------------------------------------------- glue either side of the attention kernels
-@pytest.mark.parametrize("R,M", [(1, 1), (5, 1), (8, 4), (64, 1)])
+@pytest.mark.parametrize("R,M", [(1, 1), (5, 1), (8, 4), (64, 1), (259, 1), (2048, 4)])
 def test_qkv_prep_and_out_gate_bit_exact(qt, dev, R, M):
     """q / k RMSNorm + partial RoPE + v split, and o * sigmoid(gate) (batch.py:505-513): every bf16 value equals the oracle's"""
     rng = np.random.default_rng(100 * R + M)
@@ -285,6 +285,12 @@ def test_qkv_prep_and_out_gate_bit_exact(qt, dev, R, M):
     check_equal("k", to_np(k), ok)
     check_equal("v", to_np(v), ov)
     o = bf(rng.standard_normal((R, 8, 256)))
+    if R >= 256:                                                 # tiny, huge, zero and -0 gates among the ordinary ones
+        special = bf(np.array([1e-7, -3e-6, 200.0, -150.0, 0.0, -0.0, 127.5, -1e-30]))
+        for h in (0, 3, 6):
+            blk = qkv[::7, h * 512 + 256:(h + 1) * 512:5]        # a view: every 5th gate of head h in every 7th row
+            blk[...] = special[rng.integers(0, 8, blk.shape)]
+        dq = to_dev(qkv, dev, BF16)
     check_equal("gated output", to_np(qt.attention.out_gate(to_dev(o, dev, BF16), dq)), O.attn_out_gate(o, qkv))
 
 
