@@ -55,7 +55,7 @@ def test_silu_exhaustive_through_conv(qt, dev):
 
 
 # ------------------------------------------------------------------------------------- stand-alone pieces
-@pytest.mark.parametrize("S", [1, 2, 5, 37, 300])
+@pytest.mark.parametrize("S", [1, 2, 5, 37, 300, 2048])
 def test_conv_prep_bit_exact(qt, dev, S):
     gen = torch.Generator().manual_seed(100 + S)
     cw, A_log, dtb, gw = layer_params(1)
@@ -68,16 +68,17 @@ def test_conv_prep_bit_exact(qt, dev, S):
     check_equal('np.array_equal(to_np(v), ov)', to_np(v), ov)
 
 
-def test_normalize_qk_and_compute_g_bit_exact(qt, dev):
-    gen = torch.Generator().manual_seed(7)
+@pytest.mark.parametrize("B,T", [(2, 5), (4, 512)])               # the larger one: millions of values, for the one-in-10^5 cases
+def test_normalize_qk_and_compute_g_bit_exact(qt, dev, B, T):
+    gen = torch.Generator().manual_seed(7 + T)
     cw, A_log, dtb, gw = layer_params(2)
-    q = rand_bf(gen, (2, 5, 16, 128), 2)
-    k = rand_bf(gen, (2, 5, 16, 128), 2)
+    q = rand_bf(gen, (B, T, 16, 128), 2)
+    k = rand_bf(gen, (B, T, 16, 128), 2)
     qn, kn = qt.gated_delta.normalize_qk(to_dev(q, dev, BF16), to_dev(k, dev, BF16), inv_scale=128 ** -0.5, eps=1e-6)
     oq, ok = O.normalize_qk(q, k)
     check_equal('np.array_equal(to_np(qn), oq)', to_np(qn), oq)
     check_equal('np.array_equal(to_np(kn), ok)', to_np(kn), ok)
-    a = rand_bf(gen, (2, 5, 16), 2)
+    a = rand_bf(gen, (B, T, 16), 2)
     g = qt.gated_delta.compute_g(to_dev(A_log, dev), to_dev(a, dev, BF16), to_dev(dtb, dev, BF16))
     og, _ = O.gates(a, a, A_log, dtb)
     assert g.dtype == torch.float32
