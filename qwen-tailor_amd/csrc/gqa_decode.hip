@@ -156,8 +156,8 @@ template <int M>
 __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_new,
                                                            const bf16_t* __restrict__ v_new, bf16_t* Kp, bf16_t* Vp,
                                                            const int* __restrict__ slots, const int* __restrict__ pos,
-                                                           float* __restrict__ part_o, float* __restrict__ part_ml, int B,
-                                                           int Lmax, int min_tiles, int n_slots) {
+                                                           float* __restrict__ part_o, float* __restrict__ part_ml,
+                                                           int* __restrict__ seg_tab, int B, int Lmax, int min_tiles, int n_slots) {
     constexpr int R = 4 * M;
     __shared__ int seg_start[MAX_SEG + 1];
     // one V tile and one K tile per wavefront, in one array: at the end the same memory holds the four wavefronts' scaled O
@@ -171,6 +171,8 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     AD_MARK(0);
     const int nseg = B * AKV;
     const int total = build_segments<M>(seg_start, slots, pos, nseg, Lmax, n_slots);
+    if (blockIdx.x == 0)                                         // the merge kernel reads the table instead of building it again
+        for (int i = threadIdx.x; i <= nseg; i += 256) seg_tab[i] = seg_start[i];
     const int per = tiles_per_wg(total, gridDim.x, min_tiles);
     const int wt0 = blockIdx.x * per, wt1 = min(wt0 + per, total);
     if (wt0 >= wt1) return;
@@ -350,18 +352,15 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
 constexpr int MAX_SPLITS = 4096;
 template <int M>
 __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                         const int* __restrict__ slots, const int* __restrict__ pos,
-                                                         bf16_t* __restrict__ out, int B, int Lmax, int nwg, int min_tiles,
-                                                         int n_slots) {
+                                                         const int* __restrict__ seg_tab, bf16_t* __restrict__ out, int B, int nwg,
+                                                         int min_tiles) {
     constexpr int R = 4 * M;
-    __shared__ int seg_start[MAX_SEG + 1];
     __shared__ float fs_s[MAX_SPLITS];
     __shared__ float red_m[4], red_l[4];
     __shared__ __align__(16) float acc_s[4][AD];
     const int r = blockIdx.x % R, sg = blockIdx.x / R, kvh = sg % AKV, b = sg / AKV;
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
-    const int total = build_segments<M>(seg_start, slots, pos, B * AKV, Lmax, n_slots);
-    const int ss = seg_start[sg], se = seg_start[sg + 1];
+    const int total = seg_tab[B * AKV], ss = seg_tab[sg], se = seg_tab[sg + 1];   // written by the partial kernel
     if (se == ss) return;                                        // a skipped row
     const int per = tiles_per_wg(total, nwg, min_tiles);
     const int wg0 = ss / per, ns = (se - 1) / per - wg0 + 1;     // the workgroups that hold tiles of this segment
@@ -420,11 +419,13 @@ static int partial_grid() {            // one workgroup per CU of the current de
     return cus < MAX_WG ? cus : MAX_WG;
 }
 
+constexpr long SEG_TAB_BYTES = ((MAX_SEG + 1) * 4 + 15) / 16 * 16;   // the segment table, after the partial results
+
 // bytes of workspace qt_gqa_attn_decode needs for (B sequences, M rows each, pool length Lmax); CH is accepted for callers
 // written against the fixed-split form and does not change the size
 long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH) {
     if (B < 0 || M < 1 || Lmax < 1 || CH < 16) return -1;
-    return ((long)MAX_WG + (long)B * AKV) * (4 * M) * (AD + 2) * 4;
+    return ((long)MAX_WG + (long)B * AKV) * (4 * M) * (AD + 2) * 4 + SEG_TAB_BYTES;
 }
 
 int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
@@ -443,12 +444,13 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
     const int nwg = (int)(want < partial_grid() ? want : partial_grid());
     float* part_o = (float*)workspace;
     float* part_ml = part_o + ((size_t)MAX_WG + (size_t)B * AKV) * (4 * M) * AD;
+    int* seg_tab = reinterpret_cast<int*>(part_ml + ((size_t)MAX_WG + (size_t)B * AKV) * (4 * M) * 2);
     const dim3 g1((unsigned)nwg), g2((unsigned)(B * AKV * 4 * M));
 #define QT_ATTN_LAUNCH(MM)                                                                                                \
     hipLaunchKernelGGL(attn_partial_kernel<MM>, g1, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)k_new,         \
-                       (const bf16_t*)v_new, (bf16_t*)Kp, (bf16_t*)Vp, slots, pos, part_o, part_ml, B, Lmax, min_tiles, n_slots); \
-    hipLaunchKernelGGL(attn_merge_kernel<MM>, g2, dim3(256), 0, stream, part_o, part_ml, slots, pos, (bf16_t*)out, B, Lmax, nwg, \
-                       min_tiles, n_slots);
+                       (const bf16_t*)v_new, (bf16_t*)Kp, (bf16_t*)Vp, slots, pos, part_o, part_ml, seg_tab, B, Lmax, min_tiles,    \
+                       n_slots);                                                                                          \
+    hipLaunchKernelGGL(attn_merge_kernel<MM>, g2, dim3(256), 0, stream, part_o, part_ml, seg_tab, (bf16_t*)out, B, nwg, min_tiles);
     switch (M) {
         case 1: QT_ATTN_LAUNCH(1) break;
         case 2: QT_ATTN_LAUNCH(2) break;
