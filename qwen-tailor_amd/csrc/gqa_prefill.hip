@@ -532,11 +532,14 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
 
 namespace {
 
-int cu_count() {                       // CUs of the current device (256 if the query fails)
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-        n = 256;
-    return n;
+int cu_count() {                       // CUs of the current device (256 if the query fails), asked once
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        return n;
+    }();
+    return cus;
 }
 inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 304; }
 
