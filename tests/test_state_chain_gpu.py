@@ -103,3 +103,47 @@ def test_prefill_admission_decode_verify_commit_chain(qt, dev):
         check_equal(f"sequence {b}: conv window", to_np(st["conv"][0])[0], tail)
     # the third slot, the trash slot and the layers that were not driven stay zero
     assert float(P.ssm[0][2].abs().max()) == 0.0 and float(P.ssm[1].abs().max()) == 0.0 and float(P.conv[2].abs().max()) == 0.0
+
+
+def test_attention_prefill_admission_decode_verify_chain(qt, dev):
+    """One full-attention layer between its qkv projection and its output gate: causal prefill over the prompt -> the prompt's
+    K / V rows admitted into a slot (Pools.load) -> decode rows that append their keys -> a verify round of M rows; every output
+    row against the float64 causal attention over the whole history (qwen35/model.py:154-169, qwen35/batch.py:141-237, 431-447)."""
+    from qwen_tailor_amd.model import Cfg
+    S, D, M, Lmax, slot = 203, 3, 4, 256, 2
+    T = S + D + M
+    rng = np.random.default_rng(515)
+    qkv = bf(rng.standard_normal((T, O.QKV_W)))
+    qn, kn = bf(1 + 0.1 * rng.standard_normal(256)), bf(1 + 0.1 * rng.standard_normal(256))
+    dqkv, dqn, dkn = to_dev(qkv, dev, BF16), to_dev(qn, dev, BF16), to_dev(kn, dev, BF16)
+    # the oracle's whole history at once
+    oq, ok, ov = O.attn_qkv_prep(qkv, qn, kn, np.zeros(1, np.int32), T)             # one sequence of T rows: positions 0 .. T-1
+    ref = O.sdpa_causal(oq.transpose(1, 0, 2), ok.transpose(1, 0, 2), ov.transpose(1, 0, 2))      # [8, T, 256]
+    want = O.attn_out_gate(bf(ref.transpose(1, 0, 2)), qkv)
+    # prefill: rows 0 .. S-1
+    q, k, v = qt.attention.qkv_prep(dqkv[:S], dqn, dkn, to_dev(np.zeros(1, np.int32), dev), S)
+    Kc = torch.zeros((1, 2, Lmax, 256), dtype=BF16, device=dev)
+    Vc = torch.zeros((1, 2, Lmax, 256), dtype=BF16, device=dev)
+    Kc[0, :, :S], Vc[0, :, :S] = k.transpose(0, 1), v.transpose(0, 1)
+    o = qt.attention.scaled_dot_product_attention(q.transpose(0, 1)[None].contiguous(), Kc[:, :, :S], Vc[:, :, :S], scale=256 ** -0.5,
+                                                  mask="causal")
+    got = [to_np(qt.attention.out_gate(o[0].transpose(0, 1).contiguous(), dqkv[:S]))]
+    cfg = Cfg(layers=4)
+    P = qt.batch.Pools(cfg, 3, Lmax, device=dev)
+    P.load(slot, {"conv": [], "ssm": [], "kv": [(Kc, Vc)]}, S)
+    dslot = to_dev(np.array([slot], np.int32), dev)
+    pos = S
+    for rows in [1] * D + [M]:                                   # decode rows one by one, then a verify round of M rows
+        dpos = to_dev(np.array([pos], np.int32), dev)
+        q, k, v = qt.attention.qkv_prep(dqkv[pos:pos + rows], dqn, dkn, dpos, rows)
+        o = qt.batch.attn_b(q, k, v, P.K[0], P.V[0], dslot, dpos, M=rows)
+        got.append(to_np(qt.attention.out_gate(o, dqkv[pos:pos + rows])))
+        pos += rows
+    out = np.concatenate(got)
+    assert out.shape == want.shape
+    check_rel("prompt rows", out[:S], want[:S], 1e-2, rel_l2)
+    for r in range(S, T):
+        check_rel(f"row {r}", out[r], want[r], 1e-2, rel_l2)
+    check_equal("keys in the pool", to_np(P.K[0][slot, :, :T]), ok.transpose(1, 0, 2))
+    check_equal("values in the pool", to_np(P.V[0][slot, :, :T]), ov.transpose(1, 0, 2))
+    assert float(P.K[0][0].abs().max()) == 0.0 and float(P.K[0][3].abs().max()) == 0.0          # other slots and the trash slot
