@@ -147,3 +147,28 @@ def test_attention_prefill_admission_decode_verify_chain(qt, dev):
     check_equal("keys in the pool", to_np(P.K[0][slot, :, :T]), ok.transpose(1, 0, 2))
     check_equal("values in the pool", to_np(P.V[0][slot, :, :T]), ov.transpose(1, 0, 2))
     assert float(P.K[0][0].abs().max()) == 0.0 and float(P.K[0][3].abs().max()) == 0.0          # other slots and the trash slot
+
+
+@pytest.mark.parametrize("T1,T2", [(150, 100), (64, 7), (33, 300)])
+def test_prefill_resumed_from_a_checkpoint_equals_one_prefill(qt, dev, T1, T2):
+    """A prompt prefilled in two pieces, the second starting from the first's state as a prefix-cache hit would (conv window and
+    recurrent state carried over): same outputs and final state as one prefill of the whole prompt, within the chunked form's
+    tolerance (the chunk borders differ), the conv window bit for bit; both against the sequential float64 restatement."""
+    gen = torch.Generator().manual_seed(T1 * 1000 + T2)
+    cw, A_log, dtb, gw = layer_params(T1 + T2)
+    rows = rand_bf(gen, (T1 + T2, PW), 1.0)
+    cs0 = rand_bf(gen, (3, CD))
+    S0 = (torch.randn((16, 128, 128), generator=gen) * 0.02).numpy()
+    dcw, dA, ddt, dgw = to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev), to_dev(gw, dev)
+    drows = to_dev(rows, dev, BF16)
+    whole, conv_w, ssm_w = qt.prefill.gdn_core(drows, to_dev(cs0[None], dev, BF16), to_dev(S0[None], dev), dcw, dA, ddt, dgw)
+    o1, conv1, ssm1 = qt.prefill.gdn_core(drows[:T1], to_dev(cs0[None], dev, BF16), to_dev(S0[None], dev), dcw, dA, ddt, dgw)
+    o2, conv2, ssm2 = qt.prefill.gdn_core(drows[T1:], conv1, ssm1, dcw, dA, ddt, dgw)
+    want, _, tail, state = O.prefill_gdn(rows, cs0, cw, A_log, dtb, S0, gw)
+    pieces = np.concatenate([to_np(o1), to_np(o2)])
+    check_rel("two pieces against one prefill", pieces, to_np(whole), 2e-3, rel_l2)
+    check_rel("two pieces against the restatement", pieces, want, 2e-3, rel_l2)
+    check_rel("final state against one prefill", to_np(ssm2), to_np(ssm_w), 2e-3, rel_l2)
+    check_rel("final state against the restatement", to_np(ssm2)[0], state, 2e-3, rel_l2)
+    check_tensors_equal("conv window", conv2, conv_w)
+    check_equal("conv window against the restatement", to_np(conv2)[0], tail)
