@@ -248,9 +248,15 @@ __device__ __forceinline__ void row16_bcast_all(float v, float (&r)[N]) {
 // Lane c of the row evaluates entry c % N only and the results are broadcast, so the double-precision rsqrt runs once per lane.
 template <int N>
 __device__ __forceinline__ void rsqrt_rows(const float (&ss)[N], float eps, float (&r)[N], int c) {
+    // (each candidate passes through an empty asm: a bare chain of selects is turned into an indexed read of a stack array,
+    // and a kernel that uses scratch memory at all starts its wavefronts more slowly)
     float mine = ss[0];
 #pragma unroll
-    for (int i = 1; i < N; i++) mine = (c % N == i) ? ss[i] : mine;
+    for (int i = 1; i < N; i++) {
+        float cand = ss[i];
+        asm volatile("" : "+v"(cand));
+        mine = (c % N == i) ? cand : mine;
+    }
     const float rv = rsqrt_rn(mine / 128.0f + eps);
     row16_bcast_all<N>(rv, r);
 }
