@@ -541,7 +541,7 @@ int cu_count() {                       // CUs of the current device (256 if the 
     }();
     return cus;
 }
-inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 304; }
+inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 288; }   // from 4577 rows on (4096: 127 / 142 us, 4608: 163 / 158 us)
 
 // The key split of a launch: tmax = 0 (none) or the tiles per part, parts = grid width, split_blocks = blocks with several parts.
 // Only launches that leave CUs without a workgroup are split (fewer than 2048 query rows: a short continuation of a long
@@ -584,7 +584,7 @@ KeySplit plan_split_nh(int S, int L, int q_pos0, int nh, int min_gain) {
 // The form of a launch, by measurement (us at q_pos0 = 0, one head per wavefront in its best form / two heads with the split:
 // S = 1280 30.6 / 35.7, 1536 39.4 / 37.7, 2048 57.5 / 47.0, 2560 70.2 / 64.6, 3072 84.4 / 88.5, 4096 130 / 132; after a prefix
 // two heads win by more: 1536 rows after 1000 keys 63.4 / 52.8, 2048 after 6000 201 / 174):
-//   from about 4800 rows on     two heads per wavefront, unsplit (enough 32-row blocks to balance themselves);
+//   from about 4600 rows on     two heads per wavefront, unsplit (enough 32-row blocks to balance themselves);
 //   from about 1500 rows on     two heads per wavefront with the key split, where the launch leaves room for it and, for a
 //                               whole prompt, up to about 2800 rows (a tile of a 32-row block costs 2.4 us against 2 x 1.6 -
 //                               2 us for two 16-row blocks, but its parts are twice the size);
