@@ -261,6 +261,35 @@ def test_prefill_causal_head_strides(qt, dev, S, P0):
     assert bool((outs[:, S:] == 7.0).all()), "rows between the heads were written"
 
 
+def test_prefill_causal_split_equals_unsplit_on_random_shapes(qt, dev):
+    """Forty launches of random size and prefix, each run with the workspace its split asks for and without one (unsplit): the two
+    agree to rounding, every output row is written, and the workspace need stays within the bound for its key count."""
+    from qwen_tailor_amd import _lib as QL
+    rng = np.random.default_rng(20240)
+    g = torch.Generator().manual_seed(20240)
+    nsplit = 0
+    for case in range(40):
+        S = int(rng.choice([rng.integers(1, 200), rng.integers(200, 1500), rng.integers(1500, 3000)]))
+        P0 = int(rng.choice([0, rng.integers(1, 300), rng.integers(300, 9000)]))
+        L = S + P0
+        q = torch.randn((8, S, 256), generator=g).bfloat16().to(dev)
+        K = torch.randn((2, L, 256), generator=g).bfloat16().to(dev)
+        V = torch.randn((2, L, 256), generator=g).bfloat16().to(dev)
+        nws = QL.lib().qt_gqa_prefill_workspace_bytes_for(S, L, P0)
+        assert 0 <= nws <= QL.lib().qt_gqa_prefill_workspace_bytes(L), (S, P0, nws)
+        nsplit += nws > 0
+        outs = []
+        for ws_bytes in (nws, 0):
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+            out = torch.full((8, S, 256), float("nan"), dtype=BF16, device=dev)
+            QL.call("qt_gqa_prefill_causal", QL.ptr(q), QL.ptr(K), QL.ptr(V), QL.ptr(out), QL.ptr(ws) if ws_bytes else None, ws_bytes,
+                    S, L, P0, S * 256, L * 256, QL.stream())
+            outs.append(to_np(out))
+        assert np.isfinite(outs[0]).all() and np.isfinite(outs[1]).all(), (case, S, P0)
+        check_attn(f"case {case}: S={S} P0={P0}", outs[0], outs[1])
+    assert nsplit >= 10, nsplit                                   # the sample does exercise the split
+
+
 def test_prefill_causal_rejects_queries_past_the_keys(qt, dev):
     from qwen_tailor_amd import _lib as QL
     t = torch.zeros((1, 8, 32, 256), dtype=BF16, device=dev)
