@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import glob
+import hashlib
 import os
 import subprocess
 from concurrent.futures import ThreadPoolExecutor
@@ -10,6 +11,28 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 SO = os.path.join(CSRC, "libqwen_tailor_hip.so")
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]
+
+
+HASH = SO + ".srchash"
+
+
+def source_hash() -> str:
+    """sha256 over the names and contents of every source the library is built from (csrc/*.hip, csrc/*.h) and the flags"""
+    h = hashlib.sha256(" ".join(FLAGS).encode())
+    for path in sorted(glob.glob(os.path.join(CSRC, "*.hip")) + glob.glob(os.path.join(CSRC, "*.h"))):
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def is_current() -> bool:
+    """True if the built library exists and was built from the sources as they are now."""
+    try:
+        with open(HASH) as f:
+            return os.path.exists(SO) and f.read().strip() == source_hash()
+    except OSError:
+        return False
 
 
 def _hipcc():
@@ -25,6 +48,7 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     if not srcs:
         raise RuntimeError(f"no HIP sources under {CSRC}")
     hipcc = _hipcc()
+    digest = source_hash()                  # taken before compiling: an edit made during the build leaves the library stale
     objs = [s[:-4] + ".o" for s in srcs]
 
     def one(pair):
@@ -42,6 +66,8 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
     os.replace(SO + ".tmp", SO)
+    with open(HASH, "w") as f:
+        f.write(digest + "\n")
     return SO
 
 

@@ -43,10 +43,11 @@ _SIGS = {
 
 
 def lib():
-    """The loaded library.  Builds it first if no built library is present; raises if that is impossible."""
+    """The loaded library.  Builds it first if no built library is present or if it was built from other sources than the
+    ones in csrc/ now (a hash of the sources is stored beside it); raises if that is impossible."""
     global _lib
     if _lib is None:
-        if not os.path.exists(_build.SO):
+        if not _build.is_current():
             _build.build()
         L = ctypes.CDLL(_build.SO)
         for name, args in _SIGS.items():

@@ -35,15 +35,22 @@ def deltanet_b(proj, conv_pool, conv_w, A_log, dt_bias, ssm_pool, slots, pos, ro
     return y
 
 
-_WORKSPACE = {}
+_WORKSPACE = {}          # (device index, stream handle) -> uint8 tensor
+_RETIRED = []            # outgrown buffers: kept for the life of the process, a captured HIP graph may still hold their address
+_WS_MIN = 32 << 20       # first allocation: enough for 256 sequences x 4 rows, so that growth is rare
 
 
 def _workspace(dev, nbytes):
-    """Split-K scratch of the attention kernel: one cached buffer per device, grown on demand (the C ABI never allocates)."""
-    buf = _WORKSPACE.get(dev)
+    """Split-K scratch of the attention kernel (the C ABI never allocates): one buffer per (device, stream), because launches
+    on different streams may overlap.  A buffer that is outgrown is replaced but never freed: a HIP graph captured earlier
+    replays with the old address.  Callers that manage memory themselves pass `workspace=` to attn_b instead."""
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    buf = _WORKSPACE.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
-        _WORKSPACE[dev] = buf
+        if buf is not None:
+            _RETIRED.append(buf)
+        buf = torch.empty(max(nbytes, _WS_MIN), dtype=torch.uint8, device=dev)
+        _WORKSPACE[key] = buf
     return buf
 
 
@@ -71,10 +78,11 @@ def split_size(Lmax: int, B: int = 16) -> int:
     return 128
 
 
-def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None):
+def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None, workspace=None):
     """q [R,H,D], k / v [R,KV,D] (normed + roped), pools [S+1,KV,Lmax,D]; R = B*M rows (row b*M+j = position pos[b]+j of slot
     slots[b]; slots / pos int32 [B]).  Returns o [R,H,D] bf16 and appends k / v at pos[b]+j (in place)
-    (qwen35/batch.py:230-237)."""
+    (qwen35/batch.py:230-237).  workspace: optional uint8 device tensor of at least qt_gqa_attn_workspace_bytes(B, M, Lmax, split)
+    bytes for the split-K partial results (default: a buffer cached per device and stream)."""
     q = L.dev(q, BF16, "q", (None, 8, 256))
     R = q.shape[0]
     if M < 1 or M > 4 or R % M:
@@ -89,7 +97,12 @@ def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None):
     nbytes = L.lib().qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)
     if nbytes < 0:
         raise ValueError("attn_b: bad split size")
-    ws = _workspace(q.device, nbytes)
+    if workspace is None:
+        ws = _workspace(q.device, nbytes)
+    else:
+        ws = L.dev(workspace, torch.uint8, "workspace")
+        if ws.numel() < nbytes:
+            raise ValueError(f"attn_b: workspace of {ws.numel()} bytes, {nbytes} needed")
     o = torch.empty((R, 8, 256), dtype=BF16, device=q.device)
     L.call("qt_gqa_attn_decode", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(Kp), L.ptr(Vp), L.ptr(slots), L.ptr(pos), L.ptr(o), L.ptr(ws),
            ws.numel(), B, M, Lmax, n_slots, CH, L.stream())
@@ -199,16 +212,25 @@ class Pools:
         blit_batch(jobs)                                         # one launch for the whole sequence (the reference issues 48 blits)
 
     def read(self, slot: int, pos: int, max_len: int | None = None):
-        """The slot's state as a single-sequence state dict of fresh tensors (qwen35/batch.py:449-462)."""
+        """The slot's state as a single-sequence state dict of fresh tensors (qwen35/batch.py:449-462): the inverse of load,
+        one launch of the strided copy kernel; K / V rows from `pos` on are zero."""
         ml = max_len or self.Lmax
         par = pos & 1
-        st = {"kv": [], "conv": [c[slot * 2 + par][None].clone() for c in self.conv],
-              "ssm": [s[slot][None].clone() for s in self.ssm]}
+        nkv, D = self.cfg.n_kv, self.cfg.head_dim
+        n = min(pos, ml)
+        st = {"kv": [], "conv": [torch.empty((1, 3, CD), dtype=BF16, device=c.device) for c in self.conv],
+              "ssm": [torch.empty((1, HV, DV, DK), dtype=torch.float32, device=s.device) for s in self.ssm]}
+        jobs = []
+        for i in range(len(self.conv)):
+            jobs.append((st["conv"][i], self.conv[i], 3 * CD, 0, (slot * 2 + par) * 3 * CD, 1, 0, 0))
+            jobs.append((st["ssm"][i], self.ssm[i], HV * DV * DK, 0, slot * HV * DV * DK, 1, 0, 0))
         for K, V in zip(self.K, self.V):
-            def one(P):
-                n = min(pos, ml)
-                out = torch.zeros((1, P.shape[1], ml, P.shape[3]), dtype=P.dtype, device=P.device)
-                out[0, :, :n].copy_(P[slot, :, :n])
-                return out
-            st["kv"].append((one(K), one(V)))
+            pair = []
+            for P in (K, V):
+                out = torch.zeros((1, nkv, ml, D), dtype=P.dtype, device=P.device)
+                if n:
+                    jobs.append((out, P, n * D, 0, slot * nkv * self.Lmax * D, nkv, ml * D, self.Lmax * D))
+                pair.append(out)
+            st["kv"].append(tuple(pair))
+        blit_batch(jobs)
         return st

@@ -294,22 +294,6 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
 // ------------------------------------------------------------------------------------------------------------------
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-// PA_MARK(i): phase time stamps of the phase A kernel for profiling builds (a build that defines QT_PHASE_A_PROF supplies
-// pa_prof_buf [workgroup][wavefront][16]); compiles to nothing otherwise
-#ifdef QT_PHASE_A_PROF
-__device__ long long* pa_prof_buf;
-#define PA_MARK(i)                                                                                                      \
-    do {                                                                                                                \
-        if ((threadIdx.x & 63) == 0) {                                                                                  \
-            long long* pa_p_ = pa_prof_buf + ((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;                        \
-            pa_p_[i] = clock64();                                                                                       \
-            if ((i) == 0) pa_p_[14] = wall_clock64();                                                                   \
-            if ((i) == 10) pa_p_[15] = wall_clock64();                                                                  \
-        }                                                                                                               \
-    } while (0)
-#else
-#define PA_MARK(i)
-#endif
 
 constexpr int QS_LD = DK + 8;        // row strides (elements) of the LDS tiles: keep 16-byte alignment, spread the banks
 constexpr int KT_LD = C;             // K^T / V^T rows are unpadded; their 16-byte chunks are XOR-swizzled by (row >> 3) & 7
@@ -414,7 +398,6 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
         }
     }
 
-    PA_MARK(0);
     // ---- gates of the chunk's tokens (gdn_nax.py:80-104): wave 0, one token per lane
     if (w == 0) {
         const int t = t0 + lane;
@@ -442,7 +425,6 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
     } else {
         silu_table_fill(L.tab, silu_tab, tid, 256);
         __syncthreads();
-        PA_MARK(1);
         const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
         uint4 pk[4][3];
         float ss[8], rr[8];
@@ -454,7 +436,6 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
                                                     pk[j][part]);
                 if (part < 2) ss[2 * j + part] = (float)row16_sum_d(sq);
             }
-        PA_MARK(2);
         rsqrt_rows<8>(ss, qk_eps(), rr, cc);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -470,9 +451,7 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
             stage_token(L, tl, cc, pq, pkk, pv);
         }
     }
-    PA_MARK(3);
     __syncthreads();
-    PA_MARK(4);
 
     // ---- K K^T (lower tiles) -> L, and (Q K^T)^T -> Am, on bf16 MFMA.  Wave w: row of tiles ti = 3 - w of K K^T and the
     // Am / Qg tiles of ct = w.  L stays in registers until every wave is done with Qs / Ks, whose LDS it then takes over.
@@ -532,7 +511,6 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
             *reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8) = to_half8(qf);
         }
     }
-    PA_MARK(5);
     __syncthreads();
     for (int i = tid; i < C * LS_LD; i += 256) L.Ts[i] = 0.f;                   // blocks of T above the diagonal stay zero
     {
@@ -545,7 +523,6 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
             }
     }
     __syncthreads();
-    PA_MARK(6);
 
     // ---- T = (I + L)^-1 by blocks of 16 (exact fp32: forward substitution on the diagonal blocks, fp32 MFMA below them)
     f32x4 TR[4];                                   // TR[d] = block (w + d, w) of T, accumulator layout
@@ -568,7 +545,6 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
             L.Ts[(16 * w + 4 * g + r) * LS_LD + 16 * w + n] = v;
         }
     }
-    PA_MARK(7);
     __syncthreads();
 #pragma unroll
     for (int d = 1; d < 4; d++) {
@@ -590,9 +566,7 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
             for (int r = 0; r < 4; r++) L.Ts[(16 * I + 4 * g + r) * LS_LD + 16 * w + n] = TR[d][r];
         }
     }
-    PA_MARK(8);
     __syncthreads();
-    PA_MARK(9);
 
     // ---- Wn^T = -(gamma K)^T Tb^T and U = Tb V on fp16 MFMA; wave w owns the chunk rows of tile ct = w
     {
@@ -651,7 +625,6 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
             }
         }
     }
-    PA_MARK(10);
 }
 
 }  // namespace

@@ -106,16 +106,6 @@ constexpr int MAX_SEG = 2048;          // segments (2 per sequence) a launch can
 // positions in the flat tile space, so that a workgroup whose range crosses a segment border gets fewer tiles to stream.
 constexpr int VISIT_TILES = 5;
 
-// AD_MARK(i): time stamps of the constant-rate clock for profiling builds (QT_ATTN_DECODE_PROF defines ad_prof_buf[workgroup][8])
-#ifdef QT_ATTN_DECODE_PROF
-__device__ long long* ad_prof_buf;
-#define AD_MARK(i)                                                                              \
-    do {                                                                                        \
-        if (threadIdx.x == 0) ad_prof_buf[(size_t)blockIdx.x * 8 + (i)] = wall_clock64();       \
-    } while (0)
-#else
-#define AD_MARK(i)
-#endif
 
 // Exclusive prefix of the segments' tile counts -> seg_start[0 .. nseg] (LDS); returns the total.  Rows whose slot or position
 // is out of range own no tiles (they are skipped by both kernels).  Every thread of the workgroup must call it.
@@ -168,7 +158,6 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     static_assert(sizeof(bf16_t) * 4 * 16 * (VL_LD + KL_LD) >= sizeof(float) * 4 * 16 * AD, "the four O tiles must fit into the K / V tiles");
     float* const mo = reinterpret_cast<float*>(tile_s);
 
-    AD_MARK(0);
     const int nseg = B * AKV;
     const int total = build_segments<M>(seg_start, slots, pos, nseg, Lmax, n_slots);
     if (blockIdx.x == 0)                                         // the merge kernel reads the table instead of building it again
@@ -185,7 +174,6 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int hw = lane >> 5, cl = lane & 31;
 
-    AD_MARK(1);
   for (int sg = sg0; sg < nseg && seg_start[sg] < wt1; sg++) {
     const int ss = seg_start[sg], se = seg_start[sg + 1];
     if (se == ss) continue;                                      // a skipped row
@@ -232,7 +220,6 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
 #pragma unroll
         for (int i = 0; i < 8; i++) vv[i] = __builtin_nontemporal_load(row_ptr(vbase, w, i));
         __builtin_amdgcn_sched_barrier(0);
-        AD_MARK(2);
         for (int t = w; t < ntiles; t += 4) {
             const int tn = t + 4 < ntiles ? t + 4 : t;           // the last step re-reads its own tile
             const int nvalid = min(16, hi - (lo + t * 16));
@@ -263,7 +250,6 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
             wave_lds_sync();
         }
     }
-    AD_MARK(3);
     if (first && w == 3) {
         // The M new keys of this sequence, straight from the inputs (batch.py:143-145), with the causal rule among them:
         // key i is visible to query token j only if i <= j.  Not pipelined: it runs once per sequence.
@@ -302,7 +288,6 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
         }
     }
 
-    AD_MARK(4);
     // ---- merge the 4 wavefronts (deterministic order); lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
@@ -327,7 +312,6 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
             for (int r = 0; r < 4; r++) mo[(w * R + 4 * g + r) * AD + 16 * j + n] = O[j][r] * f[r];
     }
     __syncthreads();
-    AD_MARK(5);
     float* po = part_o + pslot * R * AD;
 #pragma unroll
     for (int i = tid; i < R * AD / 4; i += 256) {
@@ -342,7 +326,6 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
         part_ml[(pslot * R + tid) * 2 + 1] = ll;
     }
     __syncthreads();                                             // the LDS tiles are reused by the next segment
-    AD_MARK(6);
   }
 }
 
@@ -409,13 +392,7 @@ constexpr int MAX_WG = 1024;           // upper bound of the partial kernel's gr
 
 static int partial_grid() {            // one workgroup per CU of the current device: measured faster than two (the stream is
                                        // bandwidth-bound with 64 KiB in flight per CU; a second workgroup only adds queueing)
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        cus = n;
-    }
+    const int cus = qt::cu_count();
     return cus < MAX_WG ? cus : MAX_WG;
 }
 
@@ -428,23 +405,15 @@ long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH) {
     return ((long)MAX_WG + (long)B * AKV) * (4 * M) * (AD + 2) * 4 + SEG_TAB_BYTES;
 }
 
-int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
-                       const int32_t* pos, void* out, void* workspace, long workspace_bytes, int B, int M, int Lmax,
-                       int n_slots, int CH, hipStream_t stream) {
-    if (!q || !k_new || !v_new || !Kp || !Vp || !slots || !pos || !out || !workspace) return QT_ERR_NULL;
-    if (B < 0 || Lmax < 1 || n_slots < 1 || CH < 16 || CH % 16) return QT_ERR_DIM;
-    if (M < 1 || M > 4 || B * AKV > MAX_SEG) return QT_ERR_UNSUPPORTED;
-    if (B == 0) return QT_OK;
-    for (const void* p : {q, k_new, v_new, (const void*)Kp, (const void*)Vp, (const void*)workspace})
-        if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
-    if (workspace_bytes < qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)) return -6;
+// Both entry points: checks, grid size and the two launches.  The partial results of at most `slot_cap` slots
+// (slot = workgroup + segment < grid + 2 B) start at part_o / part_ml; seg_tab holds 2 B + 1 ints.
+static int attn_launch(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
+                       const int32_t* pos, void* out, float* part_o, float* part_ml, int* seg_tab, int max_grid, int B, int M,
+                       int Lmax, int n_slots, int CH, hipStream_t stream) {
     const int min_tiles = CH / 16;                               // a workgroup takes at least CH keys
     const long max_tiles = (long)B * AKV * ((Lmax + 15) / 16);
     const long want = (max_tiles + min_tiles - 1) / min_tiles;
-    const int nwg = (int)(want < partial_grid() ? want : partial_grid());
-    float* part_o = (float*)workspace;
-    float* part_ml = part_o + ((size_t)MAX_WG + (size_t)B * AKV) * (4 * M) * AD;
-    int* seg_tab = reinterpret_cast<int*>(part_ml + ((size_t)MAX_WG + (size_t)B * AKV) * (4 * M) * 2);
+    const int nwg = (int)(want < max_grid ? want : max_grid);
     const dim3 g1((unsigned)nwg), g2((unsigned)(B * AKV * 4 * M));
 #define QT_ATTN_LAUNCH(MM)                                                                                                \
     hipLaunchKernelGGL(attn_partial_kernel<MM>, g1, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)k_new,         \
@@ -457,8 +426,35 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
         case 3: QT_ATTN_LAUNCH(3) break;
         default: QT_ATTN_LAUNCH(4) break;
     }
+#undef QT_ATTN_LAUNCH
     QT_CHECK_LAUNCH();
     return QT_OK;
+}
+
+static int attn_check(const void* q, const void* k_new, const void* v_new, const void* Kp, const void* Vp, const int32_t* slots,
+                      const int32_t* pos, const void* out, int B, int M, int Lmax, int n_slots, int CH) {
+    if (!q || !k_new || !v_new || !Kp || !Vp || !slots || !pos || !out) return QT_ERR_NULL;
+    if (B < 0 || Lmax < 1 || n_slots < 1 || CH < 16 || CH % 16) return QT_ERR_DIM;
+    if (M < 1 || M > 4 || B * AKV > MAX_SEG) return QT_ERR_UNSUPPORTED;
+    for (const void* p : {q, k_new, v_new, Kp, Vp})
+        if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
+    return QT_OK;
+}
+
+int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
+                       const int32_t* pos, void* out, void* workspace, long workspace_bytes, int B, int M, int Lmax,
+                       int n_slots, int CH, hipStream_t stream) {
+    if (!workspace) return QT_ERR_NULL;
+    if (const int rc = attn_check(q, k_new, v_new, Kp, Vp, slots, pos, out, B, M, Lmax, n_slots, CH)) return rc;
+    if (B == 0) return QT_OK;
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u) return QT_ERR_ALIGN;
+    if (workspace_bytes < qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)) return -6;
+    const size_t cap = (size_t)MAX_WG + (size_t)B * AKV;
+    float* part_o = (float*)workspace;
+    float* part_ml = part_o + cap * (4 * M) * AD;
+    int* seg_tab = reinterpret_cast<int*>(part_ml + cap * (4 * M) * 2);
+    return attn_launch(q, k_new, v_new, Kp, Vp, slots, pos, out, part_o, part_ml, seg_tab, partial_grid(), B, M, Lmax, n_slots, CH,
+                       stream);
 }
 
 }  // extern "C"

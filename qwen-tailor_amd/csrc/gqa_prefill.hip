@@ -37,30 +37,8 @@ constexpr float LAZY = 8.0f;            // log2 of the growth of a row maximum t
 constexpr int KT = 64;                 // keys per tile
 constexpr int TILE = KT * AD;          // elements of one K or V tile in LDS (32 KiB), rows unpadded, chunks swizzled
 
-// AP_MARK(i): phase time stamps for profiling builds (QT_ATTN_PREFILL_PROF defines ap_prof_buf[workgroup][wave][8]: shader-clock
-// ticks per phase, summed over the tiles in scalar registers and stored once at the end); otherwise only a scheduling fence
-#ifdef QT_ATTN_PREFILL_PROF
-__device__ long long* ap_prof_buf;
-#define AP_MARK(i)                                  \
-    do {                                            \
-        const long long now_ = clock64();           \
-        ap_acc_[i] += now_ - ap_last_;              \
-        ap_last_ = now_;                            \
-    } while (0)
-#define AP_INIT()                                   \
-    long long ap_acc_[8] = {0, 0, 0, 0, 0, 0, 0, 0}; \
-    long long ap_last_ = clock64()
-#define AP_STORE()                                                                                              \
-    do {                                                                                                        \
-        if ((threadIdx.x & 63) == 0)                                                                            \
-            for (int i_ = 0; i_ < 8; i_++)                                                                      \
-                ap_prof_buf[((size_t)((blockIdx.x % AKV) * (gridDim.x / AKV) + blockIdx.x / AKV) * 4 + (threadIdx.x >> 6)) * 8 + i_] = ap_acc_[i_]; \
-    } while (0)
-#else
-#define AP_MARK(i) __builtin_amdgcn_sched_barrier(0)     /* the phases of a tile are scheduled separately */
-#define AP_INIT()
-#define AP_STORE()
-#endif
+// PHASE_FENCE(): the phases of a tile are scheduled separately
+#define PHASE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
 __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -249,7 +227,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     };
 
     f32x4 accs[2][NH][4];                                        // scores of tile t live in accs[t & 1]
-    AP_INIT();
     // One tile, software-pipelined around ONE workgroup barrier X(t):
     //     before X(t): the scores of tile t are in registers (computed during tile t - 1), P.V of tile t - 1 is done
     //     at X(t):     K(t + 1) and V(t) have landed; K(t)'s buffer takes K(t + 2), V(t - 1)'s buffer takes V(t + 1)
@@ -266,9 +243,9 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         const bf16_t* const k_nxt = PAR ? k_s0 : k_s1;           // K(t + 1)
         const bf16_t* const v_cur = PAR ? v_s1 : v_s0;           // V(t)
         bf16_t* const v_nxt = PAR ? v_s0 : v_s1;                 // V(t - 1): consumed, refilled with V(t + 1)
-        AP_MARK(0);
+        PHASE_FENCE();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wavefront's loads of K(t + 1), V(t) have landed in LDS
-        AP_MARK(1);
+        PHASE_FENCE();
         __syncthreads();                                         // X(t)
         // While scores of a further tile are due (then L > KT), this wavefront's 16 loads of K(t + 2) and V(t + 1) are spread
         // over the steps below: a burst would stall on the memory pipeline's queue.  There a tile index past the end loads the
@@ -279,7 +256,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             if (t + 2 < tb) load_rows(kg, k_cur, t + 2);
             if (t + 1 < tb) load_rows(vg, v_nxt, t + 1);
         }
-        AP_MARK(2);
+        PHASE_FENCE();
         if (t >= tw) return;                               // wavefront-uniform: the upper row block may see one tile more
         // only tiles that touch the diagonal or the end of the sequence need the mask (wavefront-uniform)
         if (t * KT + KT - 1 > q_pos0 + r0 || t * KT + KT > L) {
@@ -328,7 +305,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 c_s[w][hh][n] = corr;                            // all four groups store the same value: no divergent branch
                 rescale |= corr != 1.0f;
             }
-            AP_MARK(3);
+            PHASE_FENCE();
             const unsigned step_off0 = SC ? opaque_off0() : 0u;
             // 32 steps: two score MFMAs of tile t + 1 (one K fragment x both heads) and one softmax element of tile t
             float pv_prev = 0.f;
@@ -380,7 +357,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         else
             body(std::false_type{});
         wave_lds_sync();
-        AP_MARK(4);
+        PHASE_FENCE();
         if (__any(rescale)) {                                    // wavefront-uniform: most tiles leave every row's max alone
 #pragma unroll
             for (int hh = 0; hh < NH; hh++) {
@@ -394,7 +371,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 Lsum[hh] *= c4;
             }
         }
-        AP_MARK(5);
+        PHASE_FENCE();
         // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs and serve
         // both heads; the row sums are one more column block, P . 1 (the sum of exactly the rounded values that multiply V)
         {
@@ -426,7 +403,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        AP_MARK(6);
+        PHASE_FENCE();
         wave_lds_sync();                                         // c_s is rewritten by the next tile
     };
 
@@ -442,7 +419,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             if (t + 1 < tb) tile(t + 1, std::integral_constant<int, 1>{});
         }
     }
-    AP_STORE();
     if (nparts > 1) {
         // One part of several: leave O, m, l of this wavefront's heads as they are.  A row that sees no key of this part (its
         // last key lies before the part's first) has exponentiated masked scores against a masked maximum: it is written as
@@ -532,15 +508,6 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
 
 namespace {
 
-int cu_count() {                       // CUs of the current device (256 if the query fails), asked once
-    static const int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        return n;
-    }();
-    return cus;
-}
 inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 288; }   // from 4577 rows on (4096: 127 / 142 us, 4608: 163 / 158 us)
 
 // The key split of a launch: tmax = 0 (none) or the tiles per part, parts = grid width, split_blocks = blocks with several parts.

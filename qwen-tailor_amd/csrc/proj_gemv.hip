@@ -228,23 +228,12 @@ __global__ __launch_bounds__(64 * NWV) void wide_gemm_kernel(const bf16_t* __res
 // x fragments read from LDS.  Accumulator element i of lane (n, g) is feature 4 g + i of row 16 ms + n: four adjacent
 // features, stored as 8 bytes.  grid = ceil(N / (16 WPB)), block = 64 WPB.
 constexpr int XK = 1024;
-// XL_MARK(i): time stamps of the constant-rate clock for profiling builds (QT_XLDS_PROF defines xl_prof_buf[workgroup][8])
-#ifdef QT_XLDS_PROF
-__device__ long long* xl_prof_buf;
-#define XL_MARK(i)                                                                              \
-    do {                                                                                        \
-        if (threadIdx.x == 0) xl_prof_buf[(size_t)blockIdx.x * 8 + (i)] = wall_clock64();       \
-    } while (0)
-#else
-#define XL_MARK(i)
-#endif
 template <int MS, int WPB, int EPI>
 __global__ __launch_bounds__(64 * WPB) void xlds_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ x,
                                                         const bf16_t* __restrict__ res, bf16_t* __restrict__ y, int M, int N) {
     __shared__ __align__(1024) bf16_t x_s[16 * MS * XK];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const int n0 = (blockIdx.x * WPB + w) * 16;                   // this wavefront's feature block (may lie past N)
-    XL_MARK(0);
     // W first (it comes from HBM): the wavefront's block is 32 loads, all in flight at once
     u32x4 a[XK / 32];
     {
@@ -260,13 +249,10 @@ __global__ __launch_bounds__(64 * WPB) void xlds_gemm_kernel(const bf16_t* __res
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                          (__attribute__((address_space(3))) void*)(x_s + h * 512), 16, 0, 0);
     }
-    XL_MARK(1);
     // (a direct-to-LDS load in flight makes the compiler wait for every outstanding load before the first use of any, so the
     // products cannot start under the tail of the W stream; both streams are drained here)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    XL_MARK(2);
     __syncthreads();
-    XL_MARK(3);
     f32x4 acc[MS];
 #pragma unroll
     for (int ms = 0; ms < MS; ms++) acc[ms] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -291,7 +277,6 @@ __global__ __launch_bounds__(64 * WPB) void xlds_gemm_kernel(const bf16_t* __res
                                                              acc[ms], 0, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    XL_MARK(4);
     const int f0 = n0 + 4 * g;                                    // first of this lane's four features (N is a multiple of 4)
     if (f0 >= N) return;                                          // (also a wavefront whose whole block lies past N)
 #pragma unroll
@@ -311,7 +296,6 @@ __global__ __launch_bounds__(64 * WPB) void xlds_gemm_kernel(const bf16_t* __res
             *reinterpret_cast<uint2*>(y + o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
         }
     }
-    XL_MARK(5);
 }
 
 template <int MS, int WPB>
@@ -381,15 +365,6 @@ void launch_gemm(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, b
     }
 }
 
-int cu_count() {                       // CUs of the current device (256 if the query fails), asked once
-    static const int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        return n;
-    }();
-    return cus;
-}
 
 }  // namespace
 

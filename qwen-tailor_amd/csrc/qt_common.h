@@ -316,6 +316,26 @@ __device__ __forceinline__ unsigned xcd_remap(unsigned id, unsigned n) {
 
 }  // namespace qt
 
+// CUs of the current device (256 if the query fails).  Cached per device id in atomics: any thread may ask, for any device,
+// and the launch paths pay for the runtime query once per device.
+#include <atomic>
+namespace qt {
+inline int cu_count() {
+    constexpr int MAX_DEV = 64;
+    static std::atomic<int> cache[MAX_DEV];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev >= 0 && dev < MAX_DEV) {
+        const int c = cache[dev].load(std::memory_order_relaxed);
+        if (c > 0) return c;
+    }
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    if (dev >= 0 && dev < MAX_DEV) cache[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+}  // namespace qt
+
 // error codes of the C ABI
 #define QT_OK 0
 #define QT_ERR_DIM (-1)
@@ -323,6 +343,7 @@ __device__ __forceinline__ unsigned xcd_remap(unsigned id, unsigned n) {
 #define QT_ERR_NULL (-3)
 #define QT_ERR_UNSUPPORTED (-4)
 #define QT_ERR_LAUNCH (-5)
+#define QT_ERR_WORKSPACE (-6)
 
 #define QT_CHECK_LAUNCH()                                   \
     do {                                                    \

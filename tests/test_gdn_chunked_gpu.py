@@ -43,12 +43,12 @@ def test_phase_b_on_reference_records(qt, dev, T):
     check_rel("y rel-L2", to_np(y), oy[0], 2e-3, rel_l2)
 
 
-def proj_inputs(seed, T, scale=1.0):
+def proj_inputs(seed, T, scale=1.0, state_scale=0.02):
     gen = torch.Generator().manual_seed(seed)
     cw, A_log, dtb, gw = layer_params(seed)
     proj = rand_bf(gen, (T, PW), scale)
     cs = rand_bf(gen, (3, CD))
-    S0 = (torch.randn((16, 128, 128), generator=gen) * 0.02).numpy()
+    S0 = (torch.randn((16, 128, 128), generator=gen) * state_scale).numpy()
     return proj, cs, cw, A_log, dtb, gw, S0
 
 
@@ -123,6 +123,42 @@ def test_config2_chunked_prefill(qt, dev, T):
     check_tensors_equal("gdn_core output", o4, out)
     check_tensors_equal("gdn_core state", s4, s1)
     check_equal("gdn_core conv tail", to_np(conv4)[0], otail)
+
+
+@pytest.mark.parametrize("T", [8192, 8131])
+def test_config2_long_prefill(qt, dev, T):
+    """config 2's longest sweep point (T = 8192: a chain of 128 chunks, each step rounding its operands to half precision) and
+    the same with a partial last chunk, from a nonzero state, through the layer core (reference entry qwen35/gdn_nax.py:413-426).
+    The per-head errors are checked too: a head whose state decays fast must not hide behind the slow ones."""
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(2002 + T, T)
+    o4, conv4, s4 = qt.prefill.gdn_core(to_dev(proj, dev, BF16), to_dev(cs[None], dev, BF16), to_dev(S0[None], dev), to_dev(cw, dev, BF16),
+                                        to_dev(A_log, dev), to_dev(dtb, dev), to_dev(gw, dev))
+    oo, oy, otail, os_ = O.prefill_gdn(proj, cs, cw, A_log, dtb, S0, gw)
+    e1 = check_rel("final state rel-L2", to_np(s4)[0], os_, 2e-3, rel_l2)
+    e2 = check_rel("final state max", to_np(s4)[0], os_, 2e-3, rel_max)
+    e3 = check_rel("gated output rel-L2", to_np(o4), oo, 2e-3, rel_l2)
+    got, ref = to_np(o4).reshape(T, 16, 128), oo.reshape(T, 16, 128)
+    for h in range(16):
+        check_rel(f"head {h} state rel-L2", to_np(s4)[0, h], os_[h], 2e-3, rel_l2)
+        check_rel(f"head {h} output rel-L2", got[:, h], ref[:, h], 2e-3, rel_l2)
+    for lo in range(0, T, 1024):                                              # no stretch of the sequence is worse than the bound
+        check_rel(f"tokens {lo}.. output rel-L2", got[lo:lo + 1024], ref[lo:lo + 1024], 2e-3, rel_l2)
+    check_equal("conv tail", to_np(conv4)[0], otail)
+    print(f"T={T}: state L2 {e1:.2e} max {e2:.2e}, out {e3:.2e}")
+
+
+@pytest.mark.parametrize("T,state_scale", [(300, 0.3), (300, 1.0), (2048, 0.3), (2048, 1.0)])
+def test_chunked_prefill_large_initial_state(qt, dev, T, state_scale):
+    """initial states at the scales the reference's own tests draw (N(0,1) * 0.1 and * 0.3 in tests/gdn_fuse.py, bench/gdn_nax.py:25-30)
+    and a unit-variance one: the half-precision operands of the chain must carry them"""
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(500 + T, T, state_scale=state_scale)
+    o4, conv4, s4 = qt.prefill.gdn_core(to_dev(proj, dev, BF16), to_dev(cs[None], dev, BF16), to_dev(S0[None], dev), to_dev(cw, dev, BF16),
+                                        to_dev(A_log, dev), to_dev(dtb, dev), to_dev(gw, dev))
+    oo, oy, otail, os_ = O.prefill_gdn(proj, cs, cw, A_log, dtb, S0, gw)
+    check_rel("final state rel-L2", to_np(s4)[0], os_, 2e-3, rel_l2)
+    check_rel("final state max", to_np(s4)[0], os_, 2e-3, rel_max)
+    check_rel("gated output rel-L2", to_np(o4), oo, 2e-3, rel_l2)
+    check_rel("first chunk's gated output rel-L2", to_np(o4)[:64], oo[:64], 2e-3, rel_l2)
 
 
 @pytest.mark.parametrize("T", [1, 2, 3, 5, 64, 65, 200])

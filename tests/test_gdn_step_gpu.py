@@ -336,6 +336,66 @@ def test_deltanet_bm_layout_of_reference_test(qt, dev):
             check_equal('np.array_equal(to_np(ssm_pool[e]), sp[e])', to_np(ssm_pool[e]), sp[e])
 
 
+def test_deltanet_b_config1_thousand_steps(qt, dev):
+    """benchmark config 1 at its stated length: B = 16 slots, 1000 consecutive steps.  The C oracle (float64 dot products) runs
+    free from its own state; state within 1e-4 relative and y within one bf16 ulp at EVERY step, conv windows bit-exact (so the
+    kernel's float32 re-association y = g (S.q) + delta (k.q) is observed over the whole run, not over a dozen steps)."""
+    B, steps = 16, 1000
+    gen = torch.Generator().manual_seed(1001)
+    cw, A_log, dtb, gw = layer_params(9)
+    ssm = (torch.randn((B + 1, 16, 128, 128), generator=gen) * 0.02).numpy()
+    cp = rand_bf(gen, ((B + 1) * 2, 3, CD))
+    slots = torch.randperm(B, generator=gen).numpy().astype(np.int32)
+    pos = torch.randint(0, 1000, (B,), generator=gen).numpy().astype(np.int32)
+    conv_pool, ssm_pool = to_dev(cp, dev, BF16), to_dev(ssm, dev)
+    dcw, dA, ddt, dslots = to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev), to_dev(slots, dev)
+    ocp, ossm = C.to_bf16_bits(cp), ssm.copy()
+    cwb = C.to_bf16_bits(cw).reshape(-1)
+    worst = 0.0
+    for step in range(steps):
+        proj = rand_bf(gen, (B, PW))
+        y = qt.batch.deltanet_b(to_dev(proj, dev, BF16), conv_pool, dcw, dA, ddt, ssm_pool, dslots, to_dev(pos, dev))
+        oy = C.from_bf16_bits(C.decode_step(C.to_bf16_bits(proj), ocp, cwb, A_log, dtb, ossm, slots, pos, acc64=True, nthreads=8))
+        got = to_np(ssm_pool)
+        for b in range(B):
+            e = rel_max(got[slots[b]], ossm[slots[b]])
+            worst = max(worst, e)
+            if not e <= 1e-4:
+                raise AssertionError(f"step {step}, row {b}: state relative error {e:.3e} > 1e-4")
+        check_ulp(f"y at step {step}", to_np(y), oy)
+        if step % 50 == 0 or step == steps - 1:
+            check_equal(f"conv pool at step {step}", to_np(conv_pool), C.from_bf16_bits(ocp))
+        pos = pos + 1
+    check_equal("trash slot", to_np(ssm_pool[B]), ssm[B])
+    print(f"1000 steps at B=16: worst state error {worst:.2e}")
+
+
+def test_deltanet_bm_config4_size(qt, dev):
+    """benchmark config 4's GatedDeltaNet half at its stated size: B = 16 sequences x M = 4 draft tokens, every snapshot
+    against the oracle (reference call: qwen35/batch_spec.py:142-150)."""
+    rng = np.random.default_rng(1004)
+    cw, A_log, dtb, gw = layer_params(12)
+    NS, B, M = 16, 16, 4
+    sslots = rng.permutation(NS).astype(np.int32)[:B]
+    sels = rng.integers(0, M, B).astype(np.int32)
+    pars = rng.integers(0, 2, B).astype(np.int32)
+    cp = bf(rng.standard_normal(((NS + 1) * 2, M, 3, CD)))
+    sp = (rng.standard_normal((NS + 1, M, 16, 128, 128)) * 0.02).astype(np.float32)
+    proj = bf(rng.standard_normal((B * M, PW)))
+    conv_pool, ssm_pool = to_dev(cp, dev, BF16), to_dev(sp, dev)
+    y = qt.batch_spec.deltanet_bm(to_dev(proj, dev, BF16), conv_pool, to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev),
+                                  ssm_pool, to_dev(sslots, dev), to_dev(sels, dev), to_dev(pars, dev), M)
+    ocp, osp = cp.copy(), sp.copy()
+    oy = O.deltanet_bm(proj, ocp, cw, A_log, dtb, osp, sslots, sels, pars, M)
+    check_equal("conv pool", to_np(conv_pool), ocp)
+    got = to_np(ssm_pool)
+    for b in range(B):
+        for j in range(M):
+            check_rel(f"snapshot {j} of sequence {b}", got[sslots[b], j], osp[sslots[b], j], 1e-4, rel_max)
+    check_ulp("y", to_np(y), oy)
+    check_equal("trash entry", got[NS], sp[NS])
+
+
 @pytest.mark.parametrize("B", [1, 5, 32, 64])
 def test_deltanet_b_gnorm_equals_two_launches(qt, dev, B):
     """the decode step with the gated RMSNorm fused in == deltanet_b followed by gnorm_rows (batch.py:497-499), bit for bit,

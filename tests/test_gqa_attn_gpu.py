@@ -34,7 +34,9 @@ def run_case(qt, dev, rng, S, Lmax, slots, pos, M, split=None):
                         M, split=split)
     oK, oV = Kp.copy(), Vp.copy()
     ref = O.attn_b(q, kn, vn, oK, oV, slots, pos, M)
-    check_attn(f"o (M={M})", to_np(o), ref)
+    got = to_np(o)
+    for r in range(B * M):                                                     # per query row: a short row's large outputs must not
+        check_attn(f"o row {r} (sequence {r // M}, M={M})", got[r], ref[r])    # hide a long row's small ones
     check_equal("K pool (appended rows, everything else untouched)", to_np(dK), oK)
     check_equal("V pool", to_np(dV), oV)
     return to_np(o)
@@ -85,6 +87,40 @@ def test_attn_b_out_of_range_rows_are_skipped(qt, dev):
     check_tensors_equal("pools untouched", Vp, V0)
     with pytest.raises(ValueError):
         qt.batch.attn_b(q, kn, kn, Kp, Vp, torch.tensor([0], dtype=torch.int32, device=dev), torch.tensor([0], dtype=torch.int32, device=dev), M=5)
+
+
+@pytest.mark.parametrize("B,M", [(64, 1), (64, 4), (40, 1), (40, 3), (130, 2)])
+def test_attn_b_many_sequences(qt, dev, B, M):
+    """more (sequence, KV head) segments than one 64-lane scan step of the segment table holds (B > 32), many segments per
+    workgroup, and more segments than workgroups' worth of tiles: ragged positions including 0, 1 and the last position that
+    fits, a few rows with an out-of-range slot or a full sequence (skipped: their outputs are not defined and not compared),
+    every other row against the oracle row by row, the pools bit-exact outside the appended rows"""
+    rng = np.random.default_rng(100 * B + M)
+    S, Lmax = B + 3, 640
+    slots = rng.permutation(S)[:B].astype(np.int32)
+    pos = rng.integers(0, Lmax - M, B).astype(np.int32)
+    pos[:6] = [0, 1, Lmax - M, 15, 16, 17]
+    pos[B // 2:B // 2 + 8] = rng.integers(0, 40, 8)                             # a run of very short sequences: many segments in one workgroup
+    bad = np.zeros(B, bool)
+    slots[7], bad[7] = S + 5, True                                              # slot outside the pool
+    slots[B - 2], bad[B - 2] = -1, True
+    pos[9], bad[9] = Lmax - M + 1, True                                         # the M rows would not fit
+    Kp = bf(rng.standard_normal((S + 1, 2, Lmax, 256)))
+    Vp = bf(rng.standard_normal((S + 1, 2, Lmax, 256)))
+    q = bf(rng.standard_normal((B * M, 8, 256)))
+    kn = bf(rng.standard_normal((B * M, 2, 256)))
+    vn = bf(rng.standard_normal((B * M, 2, 256)))
+    dK, dV = to_dev(Kp, dev, BF16), to_dev(Vp, dev, BF16)
+    o = to_np(qt.batch.attn_b(to_dev(q, dev, BF16), to_dev(kn, dev, BF16), to_dev(vn, dev, BF16), dK, dV, to_dev(slots, dev),
+                              to_dev(pos, dev), M))
+    oK, oV = Kp.copy(), Vp.copy()
+    good = np.flatnonzero(~bad)
+    rows = (good[:, None] * M + np.arange(M)[None]).ravel()
+    ref = O.attn_b(q[rows], kn[rows], vn[rows], oK, oV, slots[good], pos[good], M)
+    for i, r in enumerate(rows):
+        check_attn(f"row {r} (sequence {r // M}, pos {pos[r // M]})", o[r], ref[i])
+    check_equal("K pool (appended rows, everything else untouched)", to_np(dK), oK)
+    check_equal("V pool", to_np(dV), oV)
 
 
 def test_attn_b_config3_ragged_long(qt, dev):
