@@ -10,7 +10,7 @@
  * device; `stream` is a hipStream_t (passed as void* so that this header needs no HIP include).  No entry point
  * allocates, synchronises or keeps global state; all work is enqueued on `stream`.  Return value: 0 on success, or
  *   -1 bad dimension, -2 misaligned pointer, -3 null pointer, -4 unsupported shape, -5 launch failure,
- *   -6 workspace too small.
+ *   -6 workspace too small, -7 size beyond the maximum of the allocation-free entry point.
  * Rows whose slot index lies outside the pool (or whose position would overflow it) are skipped by the kernels: nothing
  * outside the caller's buffers is ever read or written.
  */
@@ -89,6 +89,16 @@ long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH);
 int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
                        const int32_t* pos, void* out, void* workspace, long workspace_bytes, int B, int M, int Lmax,
                        int n_slots, int CH, qt_stream_t stream);
+
+/* qt_gqa_attn_decode without the workspace argument.  No counterpart in the reference: it is for callers that cannot
+ * allocate device memory or pass a workspace along (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation).  The split-K partial results live in an 8.1 MiB static device array inside the library (one copy per GPU, held
+ * until the process ends), so B <= 128 (otherwise -7) and the partial kernel's grid is capped at 256 workgroups; same kernels,
+ * same results as qt_gqa_attn_decode.  The entry point allocates nothing; its first call on a device looks the array's address up
+ * (make that call outside graph capture).  All calls on one GPU share the array: calls that overlap there (two streams, two
+ * threads) race, so serialise them. */
+int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
+                              const int32_t* pos, void* out, int B, int M, int Lmax, int n_slots, int CH, qt_stream_t stream);
 
 /* Chunked (chunk = 64) GatedDeltaNet prefill, two phases (qwen35/gdn_nax.py:394-426: prep_a / gdn_chunked's phase A, phase_b).
  * Phase A is parallel over (chunk, head): it takes q, k, v [S,16,128] bf16 (qt_gdn_conv_prep's outputs) and the gate inputs in

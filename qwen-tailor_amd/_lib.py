@@ -14,7 +14,7 @@ _lib = None
 _vp, _i, _l, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
 
 ERRORS = {-1: "bad dimension", -2: "misaligned pointer", -3: "null pointer", -4: "unsupported shape", -5: "kernel launch failed",
-          -6: "workspace too small"}
+          -6: "workspace too small", -7: "size beyond the maximum of the allocation-free entry point"}
 
 _SIGS = {
     "qt_gdn_decode_step": [_vp] * 9 + [_i, _i, _i, _vp],
@@ -28,6 +28,7 @@ _SIGS = {
     "qt_gated_rmsnorm": [_vp, _vp, _vp, _vp, _l, _f, _vp],
     "qt_gdn_recurrent": [_vp] * 8 + [_i] * 6 + [_vp],
     "qt_gqa_attn_decode": [_vp] * 9 + [_l, _i, _i, _i, _i, _i, _vp],
+    "qt_gqa_attn_decode_static": [_vp] * 8 + [_i, _i, _i, _i, _i, _vp],
     "qt_gdn_phase_b": [_vp] * 7 + [_i, _vp],
     "qt_gdn_phase_b_norm": [_vp] * 8 + [_f, _vp, _i, _vp],
     "qt_gqa_prefill_causal": [_vp] * 5 + [_l, _i, _i, _i, _l, _l, _vp],

@@ -457,4 +457,42 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
                        stream);
 }
 
+// ---- the same operator for callers that cannot allocate: the partial results live in a static device array -------------------
+constexpr int ST_MAX_B = 128;          // sequences per call of the allocation-free entry point
+constexpr int ST_MAX_WG = 256;         // its partial kernel's grid is capped here (one workgroup per CU on MI355X)
+constexpr size_t ST_CAP = (size_t)ST_MAX_WG + (size_t)ST_MAX_B * AKV;
+constexpr size_t ST_BYTES = ST_CAP * 16 * (AD + 2) * 4 + SEG_TAB_BYTES;        // 8.1 MiB
+static __device__ __align__(256) unsigned char scratch[ST_BYTES];
+
+// Device address of `scratch` on the current device, looked up once per device (every GPU holds its own copy of the array
+// at its own address).  In host code the array's name is only a handle for this lookup, never a pointer to pass on.
+static int scratch_address(unsigned char** out) {
+    constexpr int MAX_DEV = 64;
+    static std::atomic<unsigned char*> cache[MAX_DEV];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) return QT_ERR_LAUNCH;
+    unsigned char* p = cache[dev].load(std::memory_order_acquire);
+    if (!p) {
+        if (hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return QT_ERR_LAUNCH;
+        cache[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return QT_OK;
+}
+
+int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
+                              const int32_t* pos, void* out, int B, int M, int Lmax, int n_slots, int CH, hipStream_t stream) {
+    if (const int rc = attn_check(q, k_new, v_new, Kp, Vp, slots, pos, out, B, M, Lmax, n_slots, CH)) return rc;
+    if (B > ST_MAX_B) return QT_ERR_STATIC_MAX;
+    if (B == 0) return QT_OK;
+    unsigned char* base = nullptr;
+    if (const int rc = scratch_address(&base)) return rc;
+    // Nothing in the array has to start at zero: every partial slot and table entry a launch reads was written by that launch.
+    float* part_o = reinterpret_cast<float*>(base);
+    float* part_ml = part_o + ST_CAP * (4 * M) * AD;
+    int* seg_tab = reinterpret_cast<int*>(part_ml + ST_CAP * (4 * M) * 2);
+    const int grid = partial_grid() < ST_MAX_WG ? partial_grid() : ST_MAX_WG;
+    return attn_launch(q, k_new, v_new, Kp, Vp, slots, pos, out, part_o, part_ml, seg_tab, grid, B, M, Lmax, n_slots, CH, stream);
+}
+
 }  // extern "C"

@@ -344,6 +344,7 @@ inline int cu_count() {
 #define QT_ERR_UNSUPPORTED (-4)
 #define QT_ERR_LAUNCH (-5)
 #define QT_ERR_WORKSPACE (-6)
+#define QT_ERR_STATIC_MAX (-7)
 
 #define QT_CHECK_LAUNCH()                                   \
     do {                                                    \
