@@ -103,8 +103,11 @@ int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_ne
 /* Chunked (chunk = 64) GatedDeltaNet prefill, two phases (qwen35/gdn_nax.py:394-426: prep_a / gdn_chunked's phase A, phase_b).
  * Phase A is parallel over (chunk, head): it takes q, k, v [S,16,128] bf16 (qt_gdn_conv_prep's outputs) and the gate inputs in
  * proj [S,8224], and computes the gates, K K^T / Q K^T on bf16 MFMA, the 64 x 64 unit-lower-triangular inverse in fp32 and the
- * state-independent MFMA operands of phase B.  It fills three caller-owned buffers of qt_gdn_chunk_{ops,u,gc}_bytes(S) bytes:
- * `ops` (half-precision operand tiles), `U` and `gC` (f32).
+ * state-independent MFMA operands of phase B.  It fills three caller-owned buffers of qt_gdn_chunk_{ops,u,gc}_bytes(S) bytes, all
+ * 16-byte aligned: `ops` and `U` (half-precision operand tiles) and `gC` (f32: per (chunk, head) the 64 per-token decay
+ * factors gamma and dec and the chunk's total decay, which phase B applies to accumulator rows).
+ * Intermediate operands are half precision (fp16: 11 significant bits, largest finite value 65504): conv outputs |v| and
+ * states |S| beyond that are not representable and are not supported; values below 6e-5 lose precision gracefully.
  * Phase B: state_in / state_out [16,128,128] f32, y [S,16,128] bf16.  It runs as a serial kernel over the chunks (the state
  * chain, which leaves the per-chunk B operands in `snap`, qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned)
  * and a kernel parallel over (chunk, head) that computes the outputs from `snap`.
@@ -115,17 +118,17 @@ long qt_gdn_chunk_u_bytes(int S);
 long qt_gdn_chunk_gc_bytes(int S);
 long qt_gdn_chunk_snap_bytes(int S);
 int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v, const float* A_log, const float* dt_bias,
-                   void* ops, float* U, float* gC, int S, qt_stream_t stream);
+                   void* ops, void* U, float* gC, int S, qt_stream_t stream);
 /* qt_gdn_phase_a with qt_gdn_conv_prep fused in (the reference's fused prep kernel, qwen35/gdn_nax.py:394-401 prep_a, with the
  * conv-state roll of qwen35/prefill.py:262-263): q, k, v are computed from proj [S,8224], conv_state [3,6144] and conv_w
  * [6144*4] inside the kernel (same bits as qt_gdn_conv_prep).  q, k, v: all three null, or all three [S,16,128] bf16 outputs.
  * conv_out: null or [3,6144] bf16, receives the new conv window (must not alias conv_state).  silu_table as qt_gdn_conv_prep. */
 int qt_gdn_phase_a_conv(const void* proj, const void* conv_state, const void* conv_w, const void* silu_table, const float* A_log,
-                        const float* dt_bias, void* q, void* k, void* v, void* conv_out, void* ops, float* U, float* gC, int S,
+                        const float* dt_bias, void* q, void* k, void* v, void* conv_out, void* ops, void* U, float* gC, int S,
                         qt_stream_t stream);
-int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
+int qt_gdn_phase_b(const void* ops, const void* U, const float* gC, void* snap, const float* state_in, float* state_out,
                    void* y, int S, qt_stream_t stream);
-int qt_gdn_phase_b_norm(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
+int qt_gdn_phase_b_norm(const void* ops, const void* U, const float* gC, void* snap, const float* state_in, float* state_out,
                         const void* proj, const float* gw, float eps, void* out, int S, qt_stream_t stream);
 
 /* Causal prefill attention: the mx.fast.scaled_dot_product_attention(..., mask="causal") call of the full-attention layers

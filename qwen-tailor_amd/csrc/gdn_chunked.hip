@@ -6,9 +6,11 @@
 //     L  = strict_lower(beta_i G_ij K K^T),  Tb = (I + L)^-1 diag(beta),  A = lower_incl(G * Q K^T)
 //     D  = Tb (V - gamma * (K S0^T)),   Y = gamma * (Q S0^T) + A D,   S1 = gamma_C S0 + (dec * D)^T K
 // Phase A (parallel over (chunk, head)) folds everything that does not depend on the state into MFMA operands
-//     Wn = -Tb (gamma * K),  U = Tb V,  Qg = gamma * Q,  Kd = (dec * K)^T,  Am = A
+//     Wn = -Tb (gamma * K),  U = Tb V,  Qh = Q,  Kh = K^T,  Am = A      (half precision; gamma, dec, gamma_C as floats)
 // so that the serial phase B is four register-resident GEMMs per chunk:
-//     D = U + Wn S0^T;   Y = Qg S0^T + Am D;   S1^T = gamma_C S0^T + Kd D.
+//     D = U + Wn S0^T;   Y = gamma * (Qh S0^T) + Am D;   S1^T = gamma_C S0^T + Kh (dec * D).
+// The per-token factors gamma and dec are applied by the consumers to accumulator rows (four multiplications per tile)
+// instead of by phase A to every operand element.
 //
 // Phase B runs one wavefront per (head, 16-wide dv slice).  The state slice S^T [128 dk x 16 dv] lives in the MFMA
 // accumulator layout (lane (n, g): rows 4g..4g+3 of column n); an accumulator pair, converted to half precision, IS the
@@ -30,10 +32,12 @@ constexpr int C = 64;                           // chunk size
 constexpr int NCT = C / 16;                     // 16-row tiles along the chunk
 constexpr int OP_W = 0;                         // offsets (in halves) of the operands inside one (chunk, head) record
 constexpr int OP_Q = OP_W + NCT * 4 * 512;      // Wn: [ct 4][kb 4][lane 64][8]
-constexpr int OP_K = OP_Q + NCT * 4 * 512;      // Qg: same;  Kd: [mt 8][kb2 2][64][8]
+constexpr int OP_K = OP_Q + NCT * 4 * 512;      // Qh: same;  Kh: [mt 8][kb2 2][64][8]
 constexpr int OP_A = OP_K + 8 * 2 * 512;        // Am: [ct 4][kb2 2][64][8]
 constexpr int OP_HALVES = OP_A + NCT * 2 * 512; // 28672 halves = 56 KiB per (chunk, head)
-constexpr int U_FLOATS = 8 * NCT * 64 * 4;      // U: [slice 8][ct 4][lane 64][4] f32 = 32 KiB per (chunk, head)
+constexpr int U_HALVES = 8 * NCT * 64 * 4;      // U: [slice 8][ct 4][lane 64][4] halves = 16 KiB per (chunk, head)
+constexpr int G_GAM = 0, G_DEC = C, G_GC = 2 * C;   // gate record of a (chunk, head): gamma[64] | dec[64] | gamma_C, 0, 0, 0
+constexpr int GATE_FLOATS = 2 * C + 4;
 
 __device__ __forceinline__ half8 pack_half8(const f32x4& a, const f32x4& b) {
     half8 h;
@@ -44,17 +48,17 @@ __device__ __forceinline__ half8 pack_half8(const f32x4& a, const f32x4& b) {
 
 // Phase B runs in two kernels.
 //
-// The chain kernel is the serial part: S_{c+1}^T = gamma_c S_c^T + Kd_c D_c with D_c = U_c + Wn_c S_c^T.  It does not
+// The chain kernel is the serial part: S_{c+1}^T = gamma_c S_c^T + Kh_c (dec_c * D_c) with D_c = U_c + Wn_c S_c^T.  It does not
 // compute outputs; it leaves, per (chunk, head, slice), the two half-precision B operands that the outputs need
-// (S_c^T and D_c, 6 KiB) in `snap`.  The output kernel then computes Y_c = Qg_c S_c^T + Am_c D_c for all chunks in parallel.
-// Splitting the outputs off halves the bytes the serial kernel has to pull per step (W and Kd: 32 of the 56 KiB).
+// (S_c^T and D_c, 6 KiB) in `snap`.  The output kernel then computes Y_c = gamma_c * (Qh_c S_c^T) + Am_c D_c for all chunks in
+// parallel.  Splitting the outputs off halves the bytes the serial kernel has to pull per step (W and Kh: 32 of the 56 KiB).
 //
 // Chain kernel: one workgroup of 5 wavefronts per (head, 16-wide dv slice).  MFMA wavefront w owns rows 16w..16w+15 of D
 // (the chunk's tokens) and rows 32w..32w+31 of S^T (dk): per chunk it pulls only its 8 operand tiles (8 KiB) and keeps
 // PB_DEP chunks of them in flight in registers, so the latency of a load is covered by PB_DEP chain steps.  Two exchanges
 // through LDS per step make up for the split: every wavefront publishes its block of S^T as the fp16 B operand and reads
-// all four (barrier E1), and publishes its rows of D and reads both k-blocks (barrier E2).  The fifth wavefront copies
-// exactly these two LDS areas to `snap`: the MFMA wavefronts issue loads only, which keeps their vmcnt waits partial
+// all four (barrier E1), and publishes its rows of D (scaled by dec for the update, and plain for the outputs) and reads both
+// k-blocks (barrier E2).  The fifth wavefront copies S^T and the plain D from LDS to `snap`: the MFMA wavefronts issue loads only, which keeps their vmcnt waits partial
 // (a store in flight next to loads forces every wait to zero on this target).
 constexpr int PB_DEP = 4;                        // chunks of operands in flight per MFMA wavefront
 constexpr int SNAP_S = 4 * 512;                  // halves: S^T as B operand, [kb 4][lane 64][8]
@@ -62,16 +66,18 @@ constexpr int SNAP_D = 2 * 512;                  // halves: D as B operand, [kb2
 constexpr int SNAP_HALVES = SNAP_S + SNAP_D;     // 6 KiB per (chunk, head, slice)
 constexpr int KORD[4] = {0, 2, 1, 3};            // order in which a step consumes its Kd tiles (two independent accumulators)
 
-__global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, const float* U, const float* gC, const float* st_in,
-                                                        float* st_out, _Float16* snap, int NC) {
+__global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, const _Float16* U, const float* gates,
+                                                        const float* st_in, float* st_out, _Float16* snap, int NC) {
     // heads that share an XCD's L2 keep their 8 slices there: workgroup id = xcd + 8 k, head = xcd + 8 (k / 8), slice = k % 8
     const int xcd = blockIdx.x & 7, kq = blockIdx.x >> 3;
     const int h = xcd + 8 * (kq >> 3), sl = kq & 7;
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     __shared__ __align__(16) _Float16 sb_x[SNAP_S];
-    __shared__ __align__(16) _Float16 db_x[SNAP_D];
+    __shared__ __align__(16) _Float16 db_x[SNAP_D];          // dec * D: the B operand of the state update
+    __shared__ __align__(16) _Float16 dn_x[SNAP_D];          // D itself: what the output kernel needs
     const half8* sbx = reinterpret_cast<const half8*>(sb_x) + lane;
     const half8* dbx = reinterpret_cast<const half8*>(db_x) + lane;
+    const half8* dnx = reinterpret_cast<const half8*>(dn_x) + lane;
 
     if (w == 4) {
         half8* dst = reinterpret_cast<half8*>(snap + ((size_t)h * 8 + sl) * SNAP_HALVES) + lane;
@@ -85,9 +91,9 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
             dst[128] = a2;
             dst[192] = a3;
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            __builtin_amdgcn_s_barrier();                                       // E2: db_x holds D_c
+            __builtin_amdgcn_s_barrier();                                       // E2: dn_x holds D_c
             asm volatile("" ::: "memory");
-            const half8 d0 = dbx[0], d1 = dbx[64];
+            const half8 d0 = dnx[0], d1 = dnx[64];
             dst[256] = d0;
             dst[320] = d1;
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -103,12 +109,15 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
         ST[1] = *reinterpret_cast<const f32x4*>(sp + 16);
     }
     const half8* opb = reinterpret_cast<const half8*>(ops + (size_t)h * OP_HALVES) + lane;
-    const f32x4* upb = reinterpret_cast<const f32x4*>(U + (size_t)h * U_FLOATS + (size_t)(sl * NCT + w) * 256) + lane;
-    const size_t ost = (size_t)HV * OP_HALVES / 8, ust = (size_t)HV * U_FLOATS / 4;
-    const int wq = (OP_W / 8) + w * 4 * 64, kq0 = (OP_K / 8) + w * 4 * 64;       // W[ct = w][kb], Kd[mt = 2w + i][kb2]
+    const half4* upb = reinterpret_cast<const half4*>(U + (size_t)h * U_HALVES + (size_t)(sl * NCT + w) * 256) + lane;
+    const float* gpb = gates + (size_t)h * GATE_FLOATS;
+    const size_t ost = (size_t)HV * OP_HALVES / 8, ust = (size_t)HV * U_HALVES / 4, gst = (size_t)HV * GATE_FLOATS;
+    const int wq = (OP_W / 8) + w * 4 * 64, kq0 = (OP_K / 8) + w * 4 * 64;       // W[ct = w][kb], Kh[mt = 2w + i][kb2]
+    const int dq = G_DEC + 16 * w + 4 * g;                                       // dec of this lane's four rows of D
 
     half8 Wt[PB_DEP][4], Kt[PB_DEP][4];
-    f32x4 Ut[PB_DEP];
+    half4 Ut[PB_DEP];
+    f32x4 dect[PB_DEP];
     float gct[PB_DEP];                       // the chunk's decay rides in the FIFO as one more (lane-uniform) vector load
 #pragma unroll
     for (int j = 0; j < PB_DEP; j++) {                                          // same issue order as inside the steps
@@ -116,9 +125,10 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
 #pragma unroll
         for (int i = 0; i < 4; i++) Wt[j][i] = opb[cc * ost + wq + i * 64];
         Ut[j] = upb[cc * ust];
+        dect[j] = *reinterpret_cast<const f32x4*>(gpb + cc * gst + dq);
 #pragma unroll
         for (int i = 0; i < 4; i++) Kt[j][KORD[i]] = opb[cc * ost + kq0 + KORD[i] * 64];
-        gct[j] = gC[(size_t)cc * HV + h];
+        gct[j] = gpb[cc * gst + G_GC];
     }
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" ::: "memory");
@@ -152,13 +162,19 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
         D1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Wt[j][3], Sb[3], D1, 0, 0, 0);
         Wt[j][3] = on[wq + 192];
         __builtin_amdgcn_sched_barrier(0);
-        const f32x4 D = (D0 + D1) + Ut[j];
+        const f32x4 Uf = {(float)Ut[j][0], (float)Ut[j][1], (float)Ut[j][2], (float)Ut[j][3]};
+        const f32x4 D = (D0 + D1) + Uf;
         Ut[j] = upb[cn * ust];
         __builtin_amdgcn_sched_barrier(0);
-        half4 dh;
+        const f32x4 Dd = D * dect[j];
+        dect[j] = *reinterpret_cast<const f32x4*>(gpb + cn * gst + dq);
+        __builtin_amdgcn_sched_barrier(0);
+        half4 dh, ddh;
         dh[0] = (_Float16)D[0]; dh[1] = (_Float16)D[1]; dh[2] = (_Float16)D[2]; dh[3] = (_Float16)D[3];
+        ddh[0] = (_Float16)Dd[0]; ddh[1] = (_Float16)Dd[1]; ddh[2] = (_Float16)Dd[2]; ddh[3] = (_Float16)Dd[3];
         // B-operand layout of D: k-block w / 2, halves 4 (w & 1) .. + 3 of the lane's eight
-        reinterpret_cast<half4*>(db_x)[((w >> 1) * 64 + lane) * 2 + (w & 1)] = dh;
+        reinterpret_cast<half4*>(db_x)[((w >> 1) * 64 + lane) * 2 + (w & 1)] = ddh;
+        reinterpret_cast<half4*>(dn_x)[((w >> 1) * 64 + lane) * 2 + (w & 1)] = dh;
         ST[0] *= gct[j];
         ST[1] *= gct[j];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -177,7 +193,7 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
         __builtin_amdgcn_sched_barrier(0);
         ST[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Kt[j][3], Db1, ST[1], 0, 0, 0);
         Kt[j][3] = on[kq0 + 192];
-        gct[j] = gC[(size_t)cn * HV + h];
+        gct[j] = gpb[cn * gst + G_GC];
         __builtin_amdgcn_sched_barrier(0);
     };
     int c = 0;
@@ -198,14 +214,15 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
 }
 static_assert(PB_DEP == 4, "the chain loop is unrolled by hand for four FIFO entries");
 
-// Output kernel: Y_c = Qg_c S_c^T + Am_c D_c for one (chunk, head) per workgroup of 4 wavefronts; wavefront w covers the dv
+// Output kernel: Y_c = gamma_c * (Qh_c S_c^T) + Am_c D_c for one (chunk, head) per workgroup of 4 wavefronts; wavefront w covers the dv
 // slices 2w and 2w+1.  The 64 x 128 tile goes through LDS as bf16 and leaves either as y [S,16,128] or, with NORM, straight
 // through the gated RMSNorm (same arithmetic as the stand-alone kernel: 16 lanes per row, 8 columns each; batch.py:338-343).
 constexpr int YS_LD = DV + 8;
 template <bool NORM>
 __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restrict__ ops, const _Float16* __restrict__ snap,
-                                                         bf16_t* __restrict__ y, const bf16_t* __restrict__ proj,
-                                                         const float* __restrict__ gw, float eps, int S) {
+                                                         const float* __restrict__ gates, bf16_t* __restrict__ y,
+                                                         const bf16_t* __restrict__ proj, const float* __restrict__ gw, float eps,
+                                                         int S) {
     const int rec = blockIdx.x, c = rec / HV, h = rec % HV;
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     __shared__ __align__(16) bf16_t ys[C * YS_LD];
@@ -223,6 +240,9 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
     for (int i = 0; i < 16; i++) Qt[i] = op[(OP_Q / 8) + i * 64];
 #pragma unroll
     for (int i = 0; i < 8; i++) At[i] = op[(OP_A / 8) + i * 64];
+    f32x4 gam[NCT];                                                             // gamma of this lane's four rows of every row tile
+#pragma unroll
+    for (int ct = 0; ct < NCT; ct++) gam[ct] = *reinterpret_cast<const f32x4*>(gates + (size_t)rec * GATE_FLOATS + G_GAM + 16 * ct + 4 * g);
 #pragma unroll
     for (int s = 0; s < 2; s++) {
         f32x4 Y[NCT];
@@ -232,6 +252,8 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
         for (int kb = 0; kb < 4; kb++)
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Qt[ct * 4 + kb], Sb[s][kb], Y[ct], 0, 0, 0);
+#pragma unroll
+        for (int ct = 0; ct < NCT; ct++) Y[ct] *= gam[ct];
 #pragma unroll
         for (int kb2 = 0; kb2 < 2; kb2++)
 #pragma unroll
@@ -291,35 +313,35 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
 
 // ------------------------------------------------------------------------------------------------------------------
 // Phase A: one workgroup of 256 threads per (chunk, head).
+//
+// The kernel is bound by its vector-ALU instruction count (two wavefronts per SIMD, little else to overlap with), so q, k
+// and v are converted to half precision ONCE, when they are staged into LDS, and every MFMA operand is then a plain LDS
+// read: row-major 16-byte reads for K K^T and Q K^T, the transposing load ds_read_b64_tr_b16 where the contraction runs
+// over the tokens (K^T for Wn and Kh, V for U).  The per-token factors gamma and dec never touch an operand element:
+// gamma goes into Tb's columns for Wn, and the chain / output kernels apply dec and gamma to accumulator rows.
 // ------------------------------------------------------------------------------------------------------------------
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 
-
-constexpr int QS_LD = DK + 8;        // row strides (elements) of the LDS tiles: keep 16-byte alignment, spread the banks
-constexpr int KT_LD = C;             // K^T / V^T rows are unpadded; their 16-byte chunks are XOR-swizzled by (row >> 3) & 7
+constexpr int QS_LD = DK + 8;        // row stride (halves) of Qs / Ks: 16-byte row reads of 16 rows hit distinct banks
+constexpr int VS_LD = DV + 16;       // row stride of Vs: the transposing loads (4 rows x 32 bytes per 16 lanes) hit distinct banks
 constexpr int LS_LD = C + 4;
+constexpr float LOG2E = 1.4426950408889634f;
 
-// element (row d, token t) of the transposed tiles: chunk (t >> 3) ^ ((d >> 3) & 7), so that the 2-byte transposing writes of
-// a wavefront (16 lanes = 16 values of d >> 3, same t) spread over the banks while a 16-byte read stays one chunk
-__device__ __forceinline__ int kt_at(int d, int t) { return d * KT_LD + ((((t >> 3) ^ (d >> 3)) & 7) << 3) + (t & 7); }
-
-struct PhaseALds {                       // 68 KiB: two workgroups per CU
+struct PhaseALds {                       // 70 KiB: two workgroups per CU
+    __align__(16) _Float16 Ks[C * QS_LD];
+    __align__(16) _Float16 Vs[C * VS_LD];
     union {
-        struct {                         // first half of the kernel: the chunk's q, k rows
-            __align__(16) bf16_t Qs[C * QS_LD];
-            __align__(16) bf16_t Ks[C * QS_LD];
-        };
-        struct {                         // second half: L = strict_lower(beta G K K^T) and T = (I + L)^-1
-            __align__(16) float Ls[C * LS_LD];
-            __align__(16) float Ts[C * LS_LD];
-        };
+        __align__(16) _Float16 Qs[C * QS_LD];    // until Q K^T is done
+        __align__(16) float Ls[C * LS_LD];       // then L = strict_lower(beta G K K^T)
     };
-    __align__(16) bf16_t KT[DK * KT_LD];
-    __align__(16) bf16_t VT[DV * KT_LD];
-    float Lc[C], beta[C], gam[C], dec[C];
-};
-struct PhaseALdsConv : PhaseALds {       // + the silu_bf16 table of the fused conv: 75 KiB, still two workgroups per CU
-    __align__(16) bf16_t tab[SILU_TAB_SIZE];
+    union {
+        struct {                                 // fused conv only: the silu_bf16 table and this head's conv taps
+            __align__(16) bf16_t tab[SILU_TAB_SIZE];
+            __align__(16) bf16_t taps[3 * DK * 4];
+        };
+        __align__(16) float Ts[C * LS_LD];       // afterwards T = (I + L)^-1
+    };
+    float Lc2[C], beta[C], gam[C], dec[C];       // Lc2 = log2(e) * cumsum(log g)
 };
 
 __device__ __forceinline__ half8 to_half8(const float (&v)[8]) {
@@ -328,38 +350,51 @@ __device__ __forceinline__ half8 to_half8(const float (&v)[8]) {
     for (int j = 0; j < 8; j++) h[j] = (_Float16)v[j];
     return h;
 }
-__device__ __forceinline__ void unpack4(uint2 w, float* f) {
-    f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
+__device__ __forceinline__ half8 bf8_to_half8(const uint4& w) {      // exact for |x| >= 2^-14 (bf16 carries 8 significant bits)
+    float f[8];
+    unpack8(w, f);
+    return to_half8(f);
+}
+// transposing LDS load: within a group of 16 lanes, lane 4 q + i receives element i of the 8-byte chunks addressed by lanes
+// q, q + 4, q + 8, q + 12.  With lane n of group g pointing at (row r0 + n / 4, columns c0 + 4 (n % 4) .. + 3), lane n receives
+// rows r0 .. r0 + 3 of column c0 + n.
+__device__ __forceinline__ half4 lds_tr4(const _Float16* p) {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(const_cast<_Float16*>(p)));
+    return __builtin_bit_cast(half4, v);
+}
+// MFMA operand whose contraction index runs over the chunk's tokens, from a row-major [token][ld] tile: lane (n, g) gets
+// column c0 + n of tokens kperm(kb2, g, 0..7) = 32 kb2 + 4 g + {0..3}, 32 kb2 + 16 + 4 g + {0..3}.
+__device__ __forceinline__ half8 tokens_operand(const _Float16* base, int ld, int kb2, int c0, int n, int g) {
+    const _Float16* p = base + (32 * kb2 + 4 * g + (n >> 2)) * ld + c0 + 4 * (n & 3);
+    const half4 lo = lds_tr4(p), hi = lds_tr4(p + 16 * ld);
+    half8 r;
+    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+    return r;
 }
 
-// Stores one token's normalized q, k and v (8 channels of each, bf16 pairs) into the row-major and transposed LDS tiles.
+// Stores one token's normalized q, k and v (8 channels of each, bf16 pairs) as half precision into the row-major LDS tiles.
 __device__ __forceinline__ void stage_token(PhaseALds& L, int tl, int cc, const uint4& rq, const uint4& rk, const uint4& rv) {
-    *reinterpret_cast<uint4*>(&L.Qs[tl * QS_LD + cc * 8]) = rq;
-    *reinterpret_cast<uint4*>(&L.Ks[tl * QS_LD + cc * 8]) = rk;
-    const uint32_t kw[4] = {rk.x, rk.y, rk.z, rk.w};
-    const uint32_t vw[4] = {rv.x, rv.y, rv.z, rv.w};
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        L.KT[kt_at(cc * 8 + 2 * e, tl)] = (bf16_t)(kw[e] & 0xffffu);
-        L.KT[kt_at(cc * 8 + 2 * e + 1, tl)] = (bf16_t)(kw[e] >> 16);
-        L.VT[kt_at(cc * 8 + 2 * e, tl)] = (bf16_t)(vw[e] & 0xffffu);
-        L.VT[kt_at(cc * 8 + 2 * e + 1, tl)] = (bf16_t)(vw[e] >> 16);
-    }
+    *reinterpret_cast<half8*>(&L.Qs[tl * QS_LD + cc * 8]) = bf8_to_half8(rq);
+    *reinterpret_cast<half8*>(&L.Ks[tl * QS_LD + cc * 8]) = bf8_to_half8(rk);
+    *reinterpret_cast<half8*>(&L.Vs[tl * VS_LD + cc * 8]) = bf8_to_half8(rv);
 }
 
-// Phase A of one (chunk, head).  FROM_PROJ = false: q, k, v [S,16,128] bf16 are inputs (convolved, normalized: conv_prep's
-// outputs).  FROM_PROJ = true: they are computed here from the projection rows (conv4 + SiLU + q/k norm with the arithmetic of
-// conv_prep_kernel, bit for bit; qwen35/prefill.py:96-134) and, with WRITE_QKV, also stored; the workgroups of the last chunk
+// Phase A of one (chunk, head).  from_proj = false: q, k, v [S,16,128] bf16 are inputs (convolved, normalized: conv_prep's
+// outputs).  from_proj = true: they are computed here from the projection rows (conv4 + SiLU + q/k norm with the arithmetic of
+// conv_prep_kernel, bit for bit; qwen35/prefill.py:96-134) and, with write_qkv, also stored; the workgroups of the last chunk
 // write the new conv window (the last three input rows, prefill.py:262-263) to conv_out if it is given.
-// proj [S,8224] supplies the gate inputs a, b in both forms.
-template <bool FROM_PROJ, bool WRITE_QKV>
-__global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __restrict__ proj, bf16_t* qi, bf16_t* ki, bf16_t* vi,
+// proj [S,8224] supplies the gate inputs a, b in both forms.  The two forms are ONE kernel with uniform branches, not two
+// template instances: everything after the staging of q, k, v is then the same machine code, so both forms give the same bits
+// (two instances are scheduled and contracted independently by the compiler and differed in the last place now and then).
+__global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bool from_proj, const bool write_qkv,
+                                                          const bf16_t* __restrict__ proj, bf16_t* qi, bf16_t* ki, bf16_t* vi,
                                                           const bf16_t* __restrict__ cs, const bf16_t* __restrict__ cw,
                                                           const bf16_t* __restrict__ silu_tab, bf16_t* __restrict__ conv_out,
                                                           const float* __restrict__ A_log, const float* __restrict__ dt_bias,
-                                                          _Float16* __restrict__ ops, float* __restrict__ U,
-                                                          float* __restrict__ gC, int S) {
-    __shared__ typename std::conditional<FROM_PROJ, PhaseALdsConv, PhaseALds>::type L;
+                                                          _Float16* __restrict__ ops, _Float16* __restrict__ U,
+                                                          float* __restrict__ gates, int S) {
+    __shared__ PhaseALds L;
     const int c = blockIdx.x / HV, h = blockIdx.x % HV, t0 = c * C;
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
     const size_t rec = (size_t)c * HV + h;
@@ -367,29 +402,33 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
     const int gi = tid >> 4, cc = tid & 15;
 
     // ---- the chunk's rows: every load is issued before anything else; rows past the end are zero (gdn_nax.py:172-174)
-    uint4 raw[4][3];                               // !FROM_PROJ: token rr * 16 + gi, a lane 8 consecutive columns
-    uint4 rw[3][7], wt[3][4];                      // FROM_PROJ: input rows 4 gi - 3 .. 4 gi + 3 of 8 channels of q, k, v; their taps
-    if constexpr (!FROM_PROJ) {
+    // one register array for both forms.  !from_proj: rw[p][rr] = token rr * 16 + gi of q / k / v, a lane 8 consecutive columns;
+    // from_proj: rw[p][d] = input row 4 gi - 3 + d of 8 channels of part p
+    uint4 rw[3][7];
+    if (!from_proj) {
 #pragma unroll
         for (int rr = 0; rr < 4; rr++) {
             const int t = t0 + rr * 16 + gi;
             const size_t o = ((size_t)min(t, S - 1) * HV + h) * DK + cc * 8;
-            raw[rr][0] = *reinterpret_cast<const uint4*>(qi + o);
-            raw[rr][1] = *reinterpret_cast<const uint4*>(ki + o);
-            raw[rr][2] = *reinterpret_cast<const uint4*>(vi + o);
-            if (t >= S) raw[rr][0] = raw[rr][1] = raw[rr][2] = make_uint4(0, 0, 0, 0);
+            rw[0][rr] = *reinterpret_cast<const uint4*>(qi + o);
+            rw[1][rr] = *reinterpret_cast<const uint4*>(ki + o);
+            rw[2][rr] = *reinterpret_cast<const uint4*>(vi + o);
+            if (t >= S) rw[0][rr] = rw[1][rr] = rw[2][rr] = make_uint4(0, 0, 0, 0);
         }
     } else {
 #pragma unroll
         for (int part = 0; part < 3; part++) {
             const int ch0 = part * KD + h * DK + cc * 8;
 #pragma unroll
-            for (int e = 0; e < 4; e++) wt[part][e] = *reinterpret_cast<const uint4*>(cw + (size_t)(ch0 + 2 * e) * 4);
-#pragma unroll
             for (int d = 0; d < 7; d++) {
                 const int tt = min(t0 + 4 * gi - 3 + d, S - 1);
                 rw[part][d] = *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0);
             }
+        }
+        // the head's conv taps (3 x 128 channels x 4 taps) go through LDS: every token group needs the same 3 KiB
+        if (tid < 192) {
+            const int part = tid >> 6, i = tid & 63;
+            reinterpret_cast<uint4*>(L.taps)[tid] = reinterpret_cast<const uint4*>(cw + (size_t)(part * KD + h * DK) * 4)[i];
         }
         if (conv_out && c == (S - 1) / C && tid < 3 * 48) {            // new conv window: input rows S-3 .. S-1 of this head's channels
             const int r = tid / 48, part = (tid % 48) >> 4, ch0 = part * KD + h * DK + (tid & 15) * 8, tt = S - 3 + r;
@@ -413,15 +452,26 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
             if (lane >= d) lc += o;
         }
         const float tot = __shfl(lc, 63, 64);
-        L.Lc[lane] = lc;
-        L.beta[lane] = be;
-        L.gam[lane] = expf(lc);
-        L.dec[lane] = expf(tot - lc);
-        if (lane == 63) gC[rec] = expf(lc);
-    }
-    if constexpr (!FROM_PROJ) {
+        float rs = lg;                                          // decay from token t to the chunk's end: a suffix sum of its own,
 #pragma unroll
-        for (int rr = 0; rr < 4; rr++) stage_token(L, rr * 16 + gi, cc, raw[rr][0], raw[rr][1], raw[rr][2]);
+        for (int d = 1; d < 64; d <<= 1) {                      // not tot - lc (two large prefix sums that nearly cancel)
+            const float o = __shfl_down(rs, d, 64);
+            if (lane + d < 64) rs += o;
+        }
+        const float suf = __shfl_down(rs, 1, 64);
+        const float gm = expf(lc), dc = lane == 63 ? 1.f : expf(suf);
+        L.Lc2[lane] = lc * LOG2E;
+        L.beta[lane] = be;
+        L.gam[lane] = gm;
+        L.dec[lane] = dc;
+        float* gp = gates + rec * GATE_FLOATS;
+        gp[G_GAM + lane] = gm;
+        gp[G_DEC + lane] = dc;
+        if (lane >= 60) gp[G_GC + lane - 60] = lane == 60 ? expf(tot) : 0.f;
+    }
+    if (!from_proj) {
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) stage_token(L, rr * 16 + gi, cc, rw[0][rr], rw[1][rr], rw[2][rr]);
     } else {
         silu_table_fill(L.tab, silu_tab, tid, 256);
         __syncthreads();
@@ -429,20 +479,23 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
         uint4 pk[4][3];
         float ss[8], rr[8];
 #pragma unroll
-        for (int part = 0; part < 3; part++)
+        for (int part = 0; part < 3; part++) {
+            uint4 wt[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) wt[e] = *reinterpret_cast<const uint4*>(&L.taps[(part * DK + cc * 8 + 2 * e) * 4]);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const double sq = conv8_silu_packed(L.tab, rw[part][j], rw[part][j + 1], rw[part][j + 2], rw[part][j + 3], wt[part],
-                                                    pk[j][part]);
+                const double sq = conv8_silu_packed(L.tab, rw[part][j], rw[part][j + 1], rw[part][j + 2], rw[part][j + 3], wt, pk[j][part]);
                 if (part < 2) ss[2 * j + part] = (float)row16_sum_d(sq);
             }
+        }
         rsqrt_rows<8>(ss, qk_eps(), rr, cc);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int tl = 4 * gi + j, t = t0 + tl;
             uint4 pq = scale8_packed(pk[j][0], rr[2 * j], scq), pkk = scale8_packed(pk[j][1], rr[2 * j + 1], sck), pv = pk[j][2];
             if (t >= S) pq = pkk = pv = make_uint4(0, 0, 0, 0);
-            if (WRITE_QKV && t < S) {
+            if (write_qkv && t < S) {
                 const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
                 *reinterpret_cast<uint4*>(qi + o) = pq;
                 *reinterpret_cast<uint4*>(ki + o) = pkk;
@@ -453,11 +506,15 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
     }
     __syncthreads();
 
-    // ---- K K^T (lower tiles) -> L, and (Q K^T)^T -> Am, on bf16 MFMA.  Wave w: row of tiles ti = 3 - w of K K^T and the
-    // Am / Qg tiles of ct = w.  L stays in registers until every wave is done with Qs / Ks, whose LDS it then takes over.
+    // ---- K K^T (lower tiles) -> L, and (Q K^T)^T -> Am, on MFMA.  Wave w: row of tiles ti = 3 - w of K K^T and the Am / Qh
+    // tiles of ct = w, plus the Kh tiles of mt = 2 w, 2 w + 1.  L stays in registers until every wave is done with Qs, whose
+    // LDS it then takes over.  G_ij = exp(Lc_i - Lc_j) = exp2(Lc2_i - Lc2_j).
     f32x4 Lreg[4];
     {
         const int ti = 3 - w;
+        f32x4 lci, bei;                                        // Lc2 and beta of this lane's rows i = 16 ti + 4 g + r
+        lci = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * ti + 4 * g]);
+        bei = *reinterpret_cast<const f32x4*>(&L.beta[16 * ti + 4 * g]);
 #pragma unroll
         for (int tj = 0; tj < 4; tj++) {
             Lreg[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -465,19 +522,20 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
                 f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kb = 0; kb < 4; kb++) {
-                    const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * ti + n) * QS_LD + 32 * kb + 8 * g]));
-                    const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]));
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+                    const half8 a = *reinterpret_cast<const half8*>(&L.Ks[(16 * ti + n) * QS_LD + 32 * kb + 8 * g]);
+                    const half8 b = *reinterpret_cast<const half8*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
                 }
-                const int j = 16 * tj + n;
+                const float lcj = L.Lc2[16 * tj + n];
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const int i = 16 * ti + 4 * g + r;
-                    Lreg[tj][r] = i > j ? L.beta[i] * expf(L.Lc[i] - L.Lc[j]) * acc[r] : 0.f;
+                    const float v = bei[r] * __builtin_amdgcn_exp2f(lci[r] - lcj) * acc[r];
+                    Lreg[tj][r] = (tj < ti || 4 * g + r > n) ? v : 0.f;
                 }
             }
         }
         const int ct = w, co = 16 * ct + n;                         // Am: rows c_out = 16 ct + n, k = c_in (permuted)
+        const float lco = L.Lc2[co];
         for (int kb2 = 0; kb2 < 2; kb2++) {
             f32x4 part[2];
 #pragma unroll
@@ -487,32 +545,38 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
                 if (tj <= ct) {
 #pragma unroll
                     for (int kb = 0; kb < 4; kb++) {
-                        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]));
-                        const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 8 * g]));
-                        part[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, part[hf], 0, 0, 0);
+                        const half8 a = *reinterpret_cast<const half8*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]);
+                        const half8 b = *reinterpret_cast<const half8*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 8 * g]);
+                        part[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, part[hf], 0, 0, 0);
                     }
+                    const f32x4 lcj = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * tj + 4 * g]);
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        const int ci = 16 * tj + 4 * g + r;
-                        part[hf][r] = ci <= co ? expf(L.Lc[co] - L.Lc[ci]) * part[hf][r] : 0.f;
+                        const float v = __builtin_amdgcn_exp2f(lco - lcj[r]) * part[hf][r];
+                        part[hf][r] = (tj < ct || 4 * g + r <= n) ? v : 0.f;
                     }
                 }
             }
             *reinterpret_cast<half8*>(op + OP_A + (ct * 2 + kb2) * 512 + lane * 8) = pack_half8(part[0], part[1]);
         }
-        // Qg = gamma * Q (rows of tile ct), k index permuted
-        const float gm = L.gam[16 * ct + n];
+        // Qh = Q (rows of tile ct), k index permuted: two 8-byte pieces of the row
         for (int kb = 0; kb < 4; kb++) {
-            float qf[8];
-            unpack4(*reinterpret_cast<const uint2*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 4 * g]), qf);
-            unpack4(*reinterpret_cast<const uint2*>(&L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 16 + 4 * g]), qf + 4);
-#pragma unroll
-            for (int j = 0; j < 8; j++) qf[j] *= gm;
-            *reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8) = to_half8(qf);
+            const _Float16* qr = &L.Qs[(16 * ct + n) * QS_LD + 32 * kb + 4 * g];
+            const half4 lo = *reinterpret_cast<const half4*>(qr), hi = *reinterpret_cast<const half4*>(qr + 16);
+            half8 qh;
+            qh[0] = lo[0]; qh[1] = lo[1]; qh[2] = lo[2]; qh[3] = lo[3];
+            qh[4] = hi[0]; qh[5] = hi[1]; qh[6] = hi[2]; qh[7] = hi[3];
+            *reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8) = qh;
+        }
+        // Kh = K^T (rows dk of tiles 2w, 2w+1), k index permuted
+        for (int mm = 0; mm < 2; mm++) {
+            const int mt = 2 * w + mm;
+            for (int kb2 = 0; kb2 < 2; kb2++)
+                *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g);
         }
     }
     __syncthreads();
-    for (int i = tid; i < C * LS_LD; i += 256) L.Ts[i] = 0.f;                   // blocks of T above the diagonal stay zero
+    for (int i = tid; i < C * LS_LD / 4; i += 256) reinterpret_cast<f32x4*>(L.Ts)[i] = f32x4{0.f, 0.f, 0.f, 0.f};   // blocks above the diagonal stay zero
     {
         const int ti = 3 - w;
 #pragma unroll
@@ -568,19 +632,28 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
     }
     __syncthreads();
 
-    // ---- Wn^T = -(gamma K)^T Tb^T and U = Tb V on fp16 MFMA; wave w owns the chunk rows of tile ct = w
+    // ---- Wn^T = K^T (-Tb gamma)^T and U = Tb V on fp16 MFMA; wave w owns the chunk rows of tile ct = w.  Both Tb operands hold
+    // Tb[16 ct + n][kperm(kb2, g, 0..7)]: as the A operand of U, and (columns scaled by -gamma) as the B operand of Wn^T.
     {
         const int ct = w, nkb = ct < 2 ? 1 : 2;                     // Tb is lower triangular: columns past the row tile are zero
-        half8 tb[2];
+        half8 tbU[2], tbW[2];
 #pragma unroll
         for (int kb2 = 0; kb2 < 2; kb2++) {
-            float v[8];
+            float u[8], v[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int cp = 32 * kb2 + 8 * g + j;
-                v[j] = L.Ts[(16 * ct + n) * LS_LD + cp] * L.beta[cp];
+            for (int hf = 0; hf < 2; hf++) {
+                const int cp = 32 * kb2 + 16 * hf + 4 * g;
+                const f32x4 t4 = *reinterpret_cast<const f32x4*>(&L.Ts[(16 * ct + n) * LS_LD + cp]);
+                const f32x4 b4 = *reinterpret_cast<const f32x4*>(&L.beta[cp]);
+                const f32x4 g4 = *reinterpret_cast<const f32x4*>(&L.gam[cp]);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    u[4 * hf + r] = t4[r] * b4[r];
+                    v[4 * hf + r] = -u[4 * hf + r] * g4[r];
+                }
             }
-            tb[kb2] = to_half8(v);
+            tbU[kb2] = to_half8(u);
+            tbW[kb2] = to_half8(v);
         }
         for (int kb = 0; kb < 4; kb++) {
             f32x4 acc[2];
@@ -591,38 +664,22 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
 #pragma unroll
                 for (int kb2 = 0; kb2 < 2; kb2++) {
                     if (kb2 >= nkb) continue;
-                    float kf[8];
-                    unpack8(*reinterpret_cast<const uint4*>(&L.KT[kt_at(16 * mt + n, 32 * kb2 + 8 * g)]), kf);
-#pragma unroll
-                    for (int j = 0; j < 8; j++) kf[j] *= -L.gam[32 * kb2 + 8 * g + j];
-                    acc[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(to_half8(kf), tb[kb2], acc[hf], 0, 0, 0);
+                    acc[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g), tbW[kb2], acc[hf], 0, 0, 0);
                 }
             }
             *reinterpret_cast<half8*>(op + OP_W + (ct * 4 + kb) * 512 + lane * 8) = pack_half8(acc[0], acc[1]);
         }
-        float* up = U + rec * U_FLOATS;
+        _Float16* up = U + rec * U_HALVES;
         for (int sl = 0; sl < 8; sl++) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kb2 = 0; kb2 < 2; kb2++) {
                 if (kb2 >= nkb) continue;
-                float vf[8];
-                unpack8(*reinterpret_cast<const uint4*>(&L.VT[kt_at(16 * sl + n, 32 * kb2 + 8 * g)]), vf);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tb[kb2], to_half8(vf), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tbU[kb2], tokens_operand(L.Vs, VS_LD, kb2, 16 * sl, n, g), acc, 0, 0, 0);
             }
-            *reinterpret_cast<f32x4*>(up + ((sl * NCT + ct) * 64 + lane) * 4) = acc;
-        }
-        // Kd = (dec * K)^T (rows dk of tiles 2w, 2w+1), k index permuted
-        for (int mm = 0; mm < 2; mm++) {
-            const int mt = 2 * w + mm;
-            for (int kb2 = 0; kb2 < 2; kb2++) {
-                float kf[8];
-                unpack4(*reinterpret_cast<const uint2*>(&L.KT[kt_at(16 * mt + n, 32 * kb2 + 4 * g)]), kf);
-                unpack4(*reinterpret_cast<const uint2*>(&L.KT[kt_at(16 * mt + n, 32 * kb2 + 16 + 4 * g)]), kf + 4);
-#pragma unroll
-                for (int j = 0; j < 8; j++) kf[j] *= L.dec[32 * kb2 + 16 * (j >> 2) + 4 * g + (j & 3)];
-                *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = to_half8(kf);
-            }
+            half4 uh;
+            uh[0] = (_Float16)acc[0]; uh[1] = (_Float16)acc[1]; uh[2] = (_Float16)acc[2]; uh[3] = (_Float16)acc[3];
+            *reinterpret_cast<half4*>(up + ((sl * NCT + ct) * 64 + lane) * 4) = uh;
         }
     }
 }
@@ -631,17 +688,17 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bf16_t* __res
 
 extern "C" {
 
-// sizes (bytes) of the phase A -> phase B buffers for S tokens: ops, U, gC
+// sizes (bytes) of the phase A -> phase B buffers for S tokens: ops, U (half precision), gC (the gate records)
 long qt_gdn_chunk_ops_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * OP_HALVES * 2; }
-long qt_gdn_chunk_u_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * U_FLOATS * 4; }
-long qt_gdn_chunk_gc_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * 4; }
+long qt_gdn_chunk_u_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * U_HALVES * 2; }
+long qt_gdn_chunk_gc_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * GATE_FLOATS * 4; }
 
-static int phase_b_launch(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
+static int phase_b_launch(const void* ops, const void* U, const float* gC, void* snap, const float* state_in, float* state_out,
                           void* y, const void* proj, const float* gw, float eps, bool norm, int S, hipStream_t stream) {
     if (!ops || !U || !gC || !snap || !state_in || !state_out || !y) return QT_ERR_NULL;
     if (norm && (!proj || !gw)) return QT_ERR_NULL;
     if (S < 0) return QT_ERR_DIM;
-    for (const void* p : {ops, (const void*)U, (const void*)snap, (const void*)state_in, (const void*)state_out, (const void*)y, proj})
+    for (const void* p : {ops, U, (const void*)gC, (const void*)snap, (const void*)state_in, (const void*)state_out, (const void*)y, proj})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     const int NC = (S + C - 1) / C;
     if (NC == 0) {
@@ -650,66 +707,61 @@ static int phase_b_launch(const void* ops, const float* U, const float* gC, void
             return QT_ERR_LAUNCH;
         return QT_OK;
     }
-    hipLaunchKernelGGL(gdn_chain_kernel, dim3(HV * 8), dim3(320), 0, stream, (const _Float16*)ops, U, gC, state_in, state_out,
+    hipLaunchKernelGGL(gdn_chain_kernel, dim3(HV * 8), dim3(320), 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in, state_out,
                        (_Float16*)snap, NC);
     QT_CHECK_LAUNCH();
     if (norm)
         hipLaunchKernelGGL(gdn_output_kernel<true>, dim3(NC * HV), dim3(256), 0, stream, (const _Float16*)ops,
-                           (const _Float16*)snap, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S);
+                           (const _Float16*)snap, gC, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S);
     else
         hipLaunchKernelGGL(gdn_output_kernel<false>, dim3(NC * HV), dim3(256), 0, stream, (const _Float16*)ops,
-                           (const _Float16*)snap, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S);
+                           (const _Float16*)snap, gC, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }
 
 long qt_gdn_chunk_snap_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * 8 * SNAP_HALVES * 2; }
 
-int qt_gdn_phase_b(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out, void* y,
+int qt_gdn_phase_b(const void* ops, const void* U, const float* gC, void* snap, const float* state_in, float* state_out, void* y,
                    int S, hipStream_t stream) {
     return phase_b_launch(ops, U, gC, snap, state_in, state_out, y, nullptr, nullptr, 0.f, false, S, stream);
 }
 
-int qt_gdn_phase_b_norm(const void* ops, const float* U, const float* gC, void* snap, const float* state_in, float* state_out,
+int qt_gdn_phase_b_norm(const void* ops, const void* U, const float* gC, void* snap, const float* state_in, float* state_out,
                         const void* proj, const float* gw, float eps, void* out, int S, hipStream_t stream) {
     return phase_b_launch(ops, U, gC, snap, state_in, state_out, out, proj, gw, eps, true, S, stream);
 }
 
 int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v, const float* A_log, const float* dt_bias,
-                   void* ops, float* U, float* gC, int S, hipStream_t stream) {
+                   void* ops, void* U, float* gC, int S, hipStream_t stream) {
     if (!proj || !q || !k || !v || !A_log || !dt_bias || !ops || !U || !gC) return QT_ERR_NULL;
     if (S < 0) return QT_ERR_DIM;
     if (S == 0) return QT_OK;
-    for (const void* p : {proj, q, k, v, (const void*)ops, (const void*)U})
+    for (const void* p : {proj, q, k, v, (const void*)ops, (const void*)U, (const void*)gC})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     const int NC = (S + C - 1) / C;
-    hipLaunchKernelGGL((gdn_phase_a_kernel<false, false>), dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (bf16_t*)q,
+    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(256), 0, stream, false, false, (const bf16_t*)proj, (bf16_t*)q,
                        (bf16_t*)k, (bf16_t*)v, (const bf16_t*)nullptr, (const bf16_t*)nullptr, (const bf16_t*)nullptr,
-                       (bf16_t*)nullptr, A_log, dt_bias, (_Float16*)ops, U, gC, S);
+                       (bf16_t*)nullptr, A_log, dt_bias, (_Float16*)ops, (_Float16*)U, gC, S);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }
 
 int qt_gdn_phase_a_conv(const void* proj, const void* conv_state, const void* conv_w, const void* silu_table, const float* A_log,
-                        const float* dt_bias, void* q, void* k, void* v, void* conv_out, void* ops, float* U, float* gC, int S,
+                        const float* dt_bias, void* q, void* k, void* v, void* conv_out, void* ops, void* U, float* gC, int S,
                         hipStream_t stream) {
     if (!proj || !conv_state || !conv_w || !A_log || !dt_bias || !ops || !U || !gC) return QT_ERR_NULL;
     if ((q || k || v) && !(q && k && v)) return QT_ERR_NULL;
     if (S < 0) return QT_ERR_DIM;
     if (S == 0) return QT_OK;
     for (const void* p : {proj, conv_state, conv_w, silu_table, (const void*)q, (const void*)k, (const void*)v, (const void*)conv_out,
-                          (const void*)ops, (const void*)U})
+                          (const void*)ops, (const void*)U, (const void*)gC})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if (conv_out == conv_state) return QT_ERR_UNSUPPORTED;          // the old window is still being read when the new one is written
     const int NC = (S + C - 1) / C;
-    if (q)
-        hipLaunchKernelGGL((gdn_phase_a_kernel<true, true>), dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj, (bf16_t*)q,
-                           (bf16_t*)k, (bf16_t*)v, (const bf16_t*)conv_state, (const bf16_t*)conv_w, (const bf16_t*)silu_table,
-                           (bf16_t*)conv_out, A_log, dt_bias, (_Float16*)ops, U, gC, S);
-    else
-        hipLaunchKernelGGL((gdn_phase_a_kernel<true, false>), dim3(NC * HV), dim3(256), 0, stream, (const bf16_t*)proj,
-                           (bf16_t*)nullptr, (bf16_t*)nullptr, (bf16_t*)nullptr, (const bf16_t*)conv_state, (const bf16_t*)conv_w,
-                           (const bf16_t*)silu_table, (bf16_t*)conv_out, A_log, dt_bias, (_Float16*)ops, U, gC, S);
+    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(256), 0, stream, true, q != nullptr, (const bf16_t*)proj, (bf16_t*)q,
+                       (bf16_t*)k, (bf16_t*)v, (const bf16_t*)conv_state, (const bf16_t*)conv_w, (const bf16_t*)silu_table,
+                       (bf16_t*)conv_out, A_log, dt_bias, (_Float16*)ops, (_Float16*)U, gC, S);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

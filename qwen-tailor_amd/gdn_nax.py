@@ -2,7 +2,7 @@
 
 Chunk size is 64 (the reference's is 16; the chunked form is an identity for every chunk size).  The three buffers that
 travel from phase A to phase B keep the reference's argument slots (Tbuf, Abuf, gv) but hold this implementation's own
-records: the packed half-precision MFMA operands, the U accumulators, and the per-chunk decay gamma_C."""
+records: the packed half-precision MFMA operands, the U tiles (half precision), and the per-token / per-chunk decay factors."""
 from __future__ import annotations
 
 import torch
@@ -23,7 +23,7 @@ TG = 64
 def _alloc_records(S, dev):
     lib = L.lib()
     ops = torch.empty(lib.qt_gdn_chunk_ops_bytes(S) // 2, dtype=torch.float16, device=dev)
-    U = torch.empty(lib.qt_gdn_chunk_u_bytes(S) // 4, dtype=torch.float32, device=dev)
+    U = torch.empty(lib.qt_gdn_chunk_u_bytes(S) // 2, dtype=torch.float16, device=dev)
     gC = torch.empty(lib.qt_gdn_chunk_gc_bytes(S) // 4, dtype=torch.float32, device=dev)
     return ops, U, gC
 
@@ -67,9 +67,9 @@ def gdn_chunked(q, k, v, proj, A_log, dt_bias, state, relaxed=True, flags=DEFAUL
 
 
 def _phase_b_args(S, Tb, Am, gv, state):
-    ops, U, gC = L.dev(Tb, torch.float16, "Tb"), L.dev(Am, torch.float32, "Am"), L.dev(gv, torch.float32, "gv")
+    ops, U, gC = L.dev(Tb, torch.float16, "Tb"), L.dev(Am, torch.float16, "Am"), L.dev(gv, torch.float32, "gv")
     lib = L.lib()
-    if ops.numel() * 2 < lib.qt_gdn_chunk_ops_bytes(S) or U.numel() * 4 < lib.qt_gdn_chunk_u_bytes(S) or \
+    if ops.numel() * 2 < lib.qt_gdn_chunk_ops_bytes(S) or U.numel() * 2 < lib.qt_gdn_chunk_u_bytes(S) or \
             gC.numel() * 4 < lib.qt_gdn_chunk_gc_bytes(S):
         raise ValueError("phase_b: the phase A records are too small for this many tokens")
     state = L.dev(state, torch.float32, "state").reshape(1, HV, DV, DK)

@@ -1,6 +1,6 @@
 """numpy restatement of what phase A of the chunked prefill hands to phase B (test infrastructure): the per-(chunk, head)
-records Wn = -Tb (gamma*K), U = Tb V, Qg = gamma*Q, Kd = (dec*K)^T, Am = A, packed in the MFMA operand layouts the HIP
-kernels use.  Built from oracle.chunk_matrices (float64), so it checks both phase B and, later, phase A."""
+records Wn = -Tb (gamma*K), U = Tb V, Qh = Q, Kh = K^T, Am = A and the gate record (gamma, dec, gamma_C), packed in the MFMA
+operand layouts the HIP kernels use.  Built from oracle.chunk_matrices (float64), so it checks both phase B and, later, phase A."""
 import numpy as np
 
 from oracle import gdn_oracle as O
@@ -33,12 +33,12 @@ def c_tiles(mat, n_mt):
 
 def chunk_records(q, k, v, lg, beta):
     """q, k, v [T,16,128]; lg, beta [T,16] -> dict of unpacked float64 matrices per (chunk, head) and the packed buffers
-    ops [NC,16,28672] (float16), U [NC,16,8,4,64,4] (float32), gC [NC,16] (float32)."""
+    ops [NC,16,28672] (float16), U [NC,16,8,4,64,4] (float16), gC [NC,16,132] (float32: gamma[64] | dec[64] | gamma_C, 0, 0, 0)."""
     T = q.shape[0]
     NC = (T + C - 1) // C
     ops = np.zeros((NC, 16, 28672), np.float16)
-    U = np.zeros((NC, 16, 8, 4, 64, 4), np.float32)
-    gC = np.zeros((NC, 16), np.float32)
+    U = np.zeros((NC, 16, 8, 4, 64, 4), np.float16)
+    gC = np.zeros((NC, 16, 132), np.float32)
     raw = {}
     for c in range(NC):
         t0, n = c * C, min(C, T - c * C)
@@ -48,13 +48,13 @@ def chunk_records(q, k, v, lg, beta):
             Tb, A, gam, dec = O.chunk_matrices(qc[:, h], kc[:, h], lc[:, h], bc[:, h])
             Wn = -Tb @ (gam[:, None] * kc[:, h])
             Uu = Tb @ vc[:, h]
-            Qg = gam[:, None] * qc[:, h]
-            Kd = (dec[:, None] * kc[:, h]).T
-            raw[(c, h)] = dict(Wn=Wn, U=Uu, Qg=Qg, Kd=Kd, Am=A, gC=gam[-1])
+            Qg = qc[:, h]
+            Kd = kc[:, h].T
+            raw[(c, h)] = dict(Wn=Wn, U=Uu, Qh=Qg, Kh=Kd, Am=A, gC=gam[-1], gam=gam, dec=dec)
             rec = np.concatenate([a_tiles(Wn, 4, 4).ravel(), a_tiles(Qg, 4, 4).ravel(), a_tiles(Kd, 8, 2).ravel(),
                                   a_tiles(A, 4, 2).ravel()])
             ops[c, h] = rec.astype(np.float16)
             for s in range(8):
                 U[c, h, s] = c_tiles(Uu[:, 16 * s:16 * s + 16], 4)
-            gC[c, h] = gam[-1]
+            gC[c, h, :64], gC[c, h, 64:128], gC[c, h, 128] = gam, dec, gam[-1]
     return raw, ops, U, gC
