@@ -127,6 +127,8 @@ def time_graph(torch, fn, reps=200, inner=10):
     st = torch.cuda.Stream()
     g = torch.cuda.CUDAGraph()
     with torch.cuda.stream(st):
+        fn()                                          # once on the capture stream: per-stream scratch buffers exist before the capture
+        torch.cuda.synchronize()
         with torch.cuda.graph(g, stream=st):
             for _ in range(inner):
                 fn()

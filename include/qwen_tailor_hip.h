@@ -108,9 +108,11 @@ int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_ne
  * factors gamma and dec and the chunk's total decay, which phase B applies to accumulator rows).
  * Intermediate operands are half precision (fp16: 11 significant bits, largest finite value 65504): conv outputs |v| and
  * states |S| beyond that are not representable and are not supported; values below 6e-5 lose precision gracefully.
- * Phase B: state_in / state_out [16,128,128] f32, y [S,16,128] bf16.  It runs as a serial kernel over the chunks (the state
- * chain, which leaves the per-chunk B operands in `snap`, qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned)
- * and a kernel parallel over (chunk, head) that computes the outputs from `snap`.
+ * Phase B: state_in / state_out [16,128,128] f32, y [S,16,128] bf16.  One launch with two kinds of workgroups: 128 run the
+ * serial state chain over the chunks and leave the per-chunk B operands in `snap`; the others compute the outputs of a
+ * chunk as soon as the chain has published it.  `snap`: qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned; its
+ * first 33 KiB (qt_gdn_chunk_snap_bytes(0) bytes) are the progress words of the launch and MUST BE ZERO when a launch starts.  A launch leaves them zero, so
+ * the caller zeroes them once; launches that use the same `snap` must not overlap.
  * qt_gdn_phase_b_norm is the same with prefill.gated_norm (qwen35/prefill.py:241-244) fused into the output kernel: it
  * writes out [S,2048] bf16 = gated RMSNorm of y with z = proj[:,6144:8192] and weight gw [128] f32 instead of y. */
 long qt_gdn_chunk_ops_bytes(int S);

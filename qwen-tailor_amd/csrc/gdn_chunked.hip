@@ -46,61 +46,124 @@ __device__ __forceinline__ half8 pack_half8(const f32x4& a, const f32x4& b) {
     return h;
 }
 
-// Phase B runs in two kernels.
+// Phase B has two roles.
 //
-// The chain kernel is the serial part: S_{c+1}^T = gamma_c S_c^T + Kh_c (dec_c * D_c) with D_c = U_c + Wn_c S_c^T.  It does not
-// compute outputs; it leaves, per (chunk, head, slice), the two half-precision B operands that the outputs need
-// (S_c^T and D_c, 6 KiB) in `snap`.  The output kernel then computes Y_c = gamma_c * (Qh_c S_c^T) + Am_c D_c for all chunks in
-// parallel.  Splitting the outputs off halves the bytes the serial kernel has to pull per step (W and Kh: 32 of the 56 KiB).
+// Chain workgroups (128) run the serial part: S_{c+1}^T = gamma_c S_c^T + Kh_c (dec_c * D_c) with D_c = U_c + Wn_c S_c^T.
+// They compute no outputs; they leave, per (chunk, head, slice), the two half-precision B operands that the outputs need
+// (S_c^T and D_c, 6 KiB) in `snap`.  Output units compute Y_c = gamma_c * (Qh_c S_c^T) + Am_c D_c from them.  Splitting the
+// outputs off the chain halves the bytes the serial workgroups have to pull per step (W and Kh: 32 of the 56 KiB).
 //
-// Chain kernel: one workgroup of 5 wavefronts per (head, 16-wide dv slice).  MFMA wavefront w owns rows 16w..16w+15 of D
-// (the chunk's tokens) and rows 32w..32w+31 of S^T (dk): per chunk it pulls only its 8 operand tiles (8 KiB) and keeps
-// PB_DEP chunks of them in flight in registers, so the latency of a load is covered by PB_DEP chain steps.  Two exchanges
-// through LDS per step make up for the split: every wavefront publishes its block of S^T as the fp16 B operand and reads
-// all four (barrier E1), and publishes its rows of D (scaled by dec for the update, and plain for the outputs) and reads both
-// k-blocks (barrier E2).  The fifth wavefront copies S^T and the plain D from LDS to `snap`: the MFMA wavefronts issue loads only, which keeps their vmcnt waits partial
-// (a store in flight next to loads forces every wait to zero on this target).
+// Short sequences run the roles as two launches (chain, then one output workgroup per (chunk, head)).  Long ones run them as
+// ONE launch: the chain publishes how many chunks are complete in a progress word per (head, slice) and the output units
+// take the chunks as their snapshots appear, so only the last chunks' outputs remain when the chain ends.  In that form
+// snapshots and progress words cross CUs (and XCDs, whose L2s are not coherent with each other) inside one launch, so they
+// are written and read with device-scope accesses that go to memory; everything else uses plain accesses.  The writer never
+// waits for its newest stores: it publishes chunk c - PUB_LAG once at most the stores of the PUB_LAG newest chunks are still
+// in flight (stores of one wavefront complete in order).  Every workgroup of that launch is resident at once (512 threads,
+// one workgroup per CU, at most 256 of them), so a consumer's producer is always running; a consumer that does not see its
+// snapshot within SPIN_LIMIT polls gives up, sets the error word and computes on what is there, so that every wavefront
+// ends.  The last output workgroup to finish clears the progress words: the flag area is zero before and after every launch
+// (the caller zeroes it once).
+//
+// Chain role: 5 wavefronts per (head, 16-wide dv slice).  MFMA wavefront w owns rows 16w..16w+15 of D (the chunk's tokens) and
+// rows 32w..32w+31 of S^T (dk): per chunk it pulls only its 8 operand tiles (8 KiB) and keeps PB_DEP chunks of them in flight
+// in registers, so the latency of a load is covered by PB_DEP chain steps.  Two exchanges through LDS per step make up for
+// the split: every wavefront publishes its block of S^T as the fp16 B operand and reads all four (barrier E1), and publishes
+// its rows of D (scaled by dec for the update, and plain for the outputs) and reads both k-blocks (barrier E2).  The fifth
+// wavefront copies S^T and the plain D from LDS to `snap`: the MFMA wavefronts issue loads only, which keeps their vmcnt
+// waits partial (a store in flight next to loads forces every wait to zero on this target).
 constexpr int PB_DEP = 4;                        // chunks of operands in flight per MFMA wavefront
 constexpr int SNAP_S = 4 * 512;                  // halves: S^T as B operand, [kb 4][lane 64][8]
 constexpr int SNAP_D = 2 * 512;                  // halves: D as B operand, [kb2 2][lane 64][8]
 constexpr int SNAP_HALVES = SNAP_S + SNAP_D;     // 6 KiB per (chunk, head, slice)
-constexpr int KORD[4] = {0, 2, 1, 3};            // order in which a step consumes its Kd tiles (two independent accumulators)
+constexpr int KORD[4] = {0, 2, 1, 3};            // order in which a step consumes its Kh tiles (two independent accumulators)
+constexpr int N_CHAIN = HV * 8;                  // chain workgroups
+constexpr int PUB_LAG = 8;                       // a chunk is published when at most this many newer chunks' stores are in flight
+constexpr int FLAG_STRIDE = 64;                  // ints between progress words: every word has a 256-byte stretch of its own
+constexpr int FLAG_WORDS = (N_CHAIN + 1) * FLAG_STRIDE;   // flag area at the head of `snap` (33 KiB): progress [128] | done count, error
+constexpr int FLAG_DONE = N_CHAIN * FLAG_STRIDE, FLAG_ERR = FLAG_DONE + 1;
+constexpr int FLAG_HALVES = FLAG_WORDS * 2;
+constexpr int SPIN_LIMIT = 1 << 21;              // polls (about a second) before a consumer gives up
+constexpr int UNITS_PER_HEAD = 16;               // output units (half workgroups) per head: unit r takes chunks r, r + 16, ...
+constexpr int FUSED_MIN_CHUNKS = 64;             // from 4096 tokens on the one-launch form wins (measured: 2048 tokens 37 / 35 us, 8192 134 / 155 us)
+typedef unsigned long long u64;
 
-__global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, const _Float16* U, const float* gates,
-                                                        const float* st_in, float* st_out, _Float16* snap, int NC) {
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+// 16 bytes per lane as ONE device-scope store (a wavefront then writes eight whole 128-byte lines; the compiler's own
+// device-scope stores are at most 8 bytes wide).  Counted by vmcnt like any other store.
+__device__ __forceinline__ void store_coherent(_Float16* p, const half8& v) {
+    const u32x4 q = __builtin_bit_cast(u32x4, v);
+    // (the s_nop is the wait state this target wants between a store of more than 8 bytes and a write to its data registers;
+    // the compiler inserts it for its own stores and cannot see into this one)
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(q) : "memory");
+}
+template <bool COHERENT>
+__device__ __forceinline__ void store_snap(_Float16* p, const half8& v) {
+    if (COHERENT) store_coherent(p, v);
+    else *reinterpret_cast<half8*>(p) = v;
+}
+__device__ __forceinline__ half8 load_coherent(const _Float16* p) {
+    ulonglong2 q;
+    q.x = __hip_atomic_load(reinterpret_cast<const u64*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    q.y = __hip_atomic_load(reinterpret_cast<const u64*>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_bit_cast(half8, q);
+}
+
+template <bool COHERENT>
+__device__ __forceinline__ half8 load_snap(const _Float16* p) {
+    return COHERENT ? load_coherent(p) : *reinterpret_cast<const half8*>(p);
+}
+
+struct ChainLds {
+    __align__(16) _Float16 sb_x[SNAP_S];
+    __align__(16) _Float16 db_x[SNAP_D];          // dec * D: the B operand of the state update
+    __align__(16) _Float16 dn_x[SNAP_D];          // D itself: what the output workgroups need
+};
+
+// blk = (head, slice) index of this workgroup; wavefronts 0..3 compute, wavefront 4 writes snapshots and publishes progress
+template <bool PUBLISH>
+__device__ __forceinline__ void chain_role(ChainLds& L, int blk, const _Float16* ops, const _Float16* U, const float* gates,
+                                           const float* st_in, float* st_out, _Float16* snaps, int* flags, int NC) {
     // heads that share an XCD's L2 keep their 8 slices there: workgroup id = xcd + 8 k, head = xcd + 8 (k / 8), slice = k % 8
-    const int xcd = blockIdx.x & 7, kq = blockIdx.x >> 3;
+    const int xcd = blk & 7, kq = blk >> 3;
     const int h = xcd + 8 * (kq >> 3), sl = kq & 7;
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
-    __shared__ __align__(16) _Float16 sb_x[SNAP_S];
-    __shared__ __align__(16) _Float16 db_x[SNAP_D];          // dec * D: the B operand of the state update
-    __shared__ __align__(16) _Float16 dn_x[SNAP_D];          // D itself: what the output kernel needs
-    const half8* sbx = reinterpret_cast<const half8*>(sb_x) + lane;
-    const half8* dbx = reinterpret_cast<const half8*>(db_x) + lane;
-    const half8* dnx = reinterpret_cast<const half8*>(dn_x) + lane;
+    const half8* sbx = reinterpret_cast<const half8*>(L.sb_x) + lane;
+    const half8* dbx = reinterpret_cast<const half8*>(L.db_x) + lane;
+    const half8* dnx = reinterpret_cast<const half8*>(L.dn_x) + lane;
 
     if (w == 4) {
-        half8* dst = reinterpret_cast<half8*>(snap + ((size_t)h * 8 + sl) * SNAP_HALVES) + lane;
-        const size_t cst = (size_t)HV * 8 * SNAP_HALVES / 8;                    // half8 per chunk
+        _Float16* dst = snaps + ((size_t)h * 8 + sl) * SNAP_HALVES + lane * 8;
+        const size_t cst = (size_t)HV * 8 * SNAP_HALVES;                        // halves per chunk
+        int* flag = flags + (h * 8 + sl) * FLAG_STRIDE;
         for (int c = 0; c < NC; c++) {
             __builtin_amdgcn_s_barrier();                                       // E1: sb_x holds S_c^T
             asm volatile("" ::: "memory");
             const half8 a0 = sbx[0], a1 = sbx[64], a2 = sbx[128], a3 = sbx[192];
-            dst[0] = a0;
-            dst[64] = a1;
-            dst[128] = a2;
-            dst[192] = a3;
+            store_snap<PUBLISH>(dst, a0);
+            store_snap<PUBLISH>(dst + 512, a1);
+            store_snap<PUBLISH>(dst + 1024, a2);
+            store_snap<PUBLISH>(dst + 1536, a3);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();                                       // E2: dn_x holds D_c
             asm volatile("" ::: "memory");
             const half8 d0 = dnx[0], d1 = dnx[64];
-            dst[256] = d0;
-            dst[320] = d1;
+            store_snap<PUBLISH>(dst + 2048, d0);
+            store_snap<PUBLISH>(dst + 2560, d1);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             dst += cst;
+            if (PUBLISH && c >= PUB_LAG) {                                      // 6 stores per chunk (+ one progress store per step)
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(7 * PUB_LAG) : "memory");
+                if (lane == 0) __hip_atomic_store(flag, c - PUB_LAG + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (PUBLISH) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (lane == 0) __hip_atomic_store(flag, NC, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         return;
     }
+    if (w > 4) return;
 
     f32x4 ST[2];
     {
@@ -140,7 +203,7 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
         constexpr int j = decltype(J)::value;
         const int cn = min(c + PB_DEP, NC - 1);
         const half8* on = opb + cn * ost;
-        reinterpret_cast<half8*>(sb_x)[w * 64 + lane] = pack_half8(ST[0], ST[1]);
+        reinterpret_cast<half8*>(L.sb_x)[w * 64 + lane] = pack_half8(ST[0], ST[1]);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();                                           // E1
         asm volatile("" ::: "memory");
@@ -173,8 +236,8 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
         dh[0] = (_Float16)D[0]; dh[1] = (_Float16)D[1]; dh[2] = (_Float16)D[2]; dh[3] = (_Float16)D[3];
         ddh[0] = (_Float16)Dd[0]; ddh[1] = (_Float16)Dd[1]; ddh[2] = (_Float16)Dd[2]; ddh[3] = (_Float16)Dd[3];
         // B-operand layout of D: k-block w / 2, halves 4 (w & 1) .. + 3 of the lane's eight
-        reinterpret_cast<half4*>(db_x)[((w >> 1) * 64 + lane) * 2 + (w & 1)] = ddh;
-        reinterpret_cast<half4*>(dn_x)[((w >> 1) * 64 + lane) * 2 + (w & 1)] = dh;
+        reinterpret_cast<half4*>(L.db_x)[((w >> 1) * 64 + lane) * 2 + (w & 1)] = ddh;
+        reinterpret_cast<half4*>(L.dn_x)[((w >> 1) * 64 + lane) * 2 + (w & 1)] = dh;
         ST[0] *= gct[j];
         ST[1] *= gct[j];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -214,100 +277,182 @@ __global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, con
 }
 static_assert(PB_DEP == 4, "the chain loop is unrolled by hand for four FIFO entries");
 
-// Output kernel: Y_c = gamma_c * (Qh_c S_c^T) + Am_c D_c for one (chunk, head) per workgroup of 4 wavefronts; wavefront w covers the dv
-// slices 2w and 2w+1.  The 64 x 128 tile goes through LDS as bf16 and leaves either as y [S,16,128] or, with NORM, straight
-// through the gated RMSNorm (same arithmetic as the stand-alone kernel: 16 lanes per row, 8 columns each; batch.py:338-343).
+// Output role: Y_c = gamma_c * (Qh_c S_c^T) + Am_c D_c for one (chunk, head) at a time per unit of 4 wavefronts (a workgroup
+// holds two units); wavefront w of the unit covers the dv slices 2w and 2w+1.  The 64 x 128 tile goes through LDS as bf16 and
+// leaves either as y [S,16,128] or, with NORM, straight through the gated RMSNorm (same arithmetic as the stand-alone kernel:
+// 16 lanes per row, 8 columns each; batch.py:338-343).  Both units of a workgroup run the same number of rounds, so that they
+// meet at the same workgroup barriers.
 constexpr int YS_LD = DV + 8;
+template <bool NORM, bool WAIT>
+__device__ __forceinline__ void output_role(bf16_t* ys, volatile int* ready, int unit, int units_per_head, const _Float16* __restrict__ ops,
+                                            const _Float16* snaps, int* flags, const float* __restrict__ gates,
+                                            bf16_t* __restrict__ y, const bf16_t* __restrict__ proj, const float* __restrict__ gw,
+                                            float eps, int S, int NC) {
+    const int h = unit % HV, r0 = unit / HV;
+    const int tid = threadIdx.x & 255, w = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int rounds = (NC + units_per_head - 1) / units_per_head;
+    for (int rd = 0; rd < rounds; rd++) {
+        const int c = r0 + rd * units_per_head;
+        const bool active = c < NC;                                             // uniform over the unit
+        if (active) {
+            const size_t rec = (size_t)c * HV + h;
+            const half8* op = reinterpret_cast<const half8*>(ops + rec * OP_HALVES) + lane;
+            half8 Sb[2][4], Db[2][2], Qt[16], At[8];
+            // what does not depend on the chain is requested before the wait
+#pragma unroll
+            for (int i = 0; i < 16; i++) Qt[i] = op[(OP_Q / 8) + i * 64];
+#pragma unroll
+            for (int i = 0; i < 8; i++) At[i] = op[(OP_A / 8) + i * 64];
+            f32x4 gam[NCT];                                                     // gamma of this lane's four rows of every row tile
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) gam[ct] = *reinterpret_cast<const f32x4*>(gates + rec * GATE_FLOATS + G_GAM + 16 * ct + 4 * g);
+            // wait until the chain has published chunk c for all eight slices of the head: the unit's first wavefront polls (lanes
+            // 0..7, one progress word each, about once a microsecond: thousands of pollers on one memory line would hold up the
+            // chain's own progress stores) and passes the news on through LDS, where the other three wavefronts wait
+            if (!WAIT) {
+            } else if (w == 0) {
+                const int* fp = flags + (h * 8 + (lane & 7)) * FLAG_STRIDE;
+                int spins = 0;
+                while (true) {
+                    int v = c + 1;
+                    if (lane < 8) v = __hip_atomic_load(fp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    asm volatile("" ::: "memory");                              // the snapshot loads stay behind the poll
+                    if (__all(v > c)) break;
+                    if (++spins > SPIN_LIMIT) {
+                        if (lane == 0) __hip_atomic_store(flags + FLAG_ERR, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(32);
+                }
+                if (lane == 0) *ready = c + 1;
+            } else {
+                while (*ready <= c) __builtin_amdgcn_s_sleep(2);
+                asm volatile("" ::: "memory");
+            }
+            const _Float16* sp = snaps + (rec * 8 + 2 * w) * SNAP_HALVES + lane * 8;
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+#pragma unroll
+                for (int kb = 0; kb < 4; kb++) Sb[s][kb] = load_snap<WAIT>(sp + s * SNAP_HALVES + kb * 512);
+#pragma unroll
+                for (int kb2 = 0; kb2 < 2; kb2++) Db[s][kb2] = load_snap<WAIT>(sp + s * SNAP_HALVES + SNAP_S + kb2 * 512);
+            }
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                f32x4 Y[NCT];
+#pragma unroll
+                for (int ct = 0; ct < NCT; ct++) Y[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kb = 0; kb < 4; kb++)
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Qt[ct * 4 + kb], Sb[s][kb], Y[ct], 0, 0, 0);
+#pragma unroll
+                for (int ct = 0; ct < NCT; ct++) Y[ct] *= gam[ct];
+#pragma unroll
+                for (int kb2 = 0; kb2 < 2; kb2++)
+#pragma unroll
+                    for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(At[ct * 2 + kb2], Db[s][kb2], Y[ct], 0, 0, 0);
+#pragma unroll
+                for (int ct = 0; ct < NCT; ct++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) ys[(ct * 16 + 4 * g + r) * YS_LD + (2 * w + s) * 16 + n] = f2bf(Y[ct][r]);
+            }
+        }
+        __syncthreads();
+        if (active) {
+            if (!NORM) {
+                const int row = tid >> 2, q4 = tid & 3;
+                const int t = c * C + row;
+                if (t < S) {
+                    const uint4* src = reinterpret_cast<const uint4*>(&ys[row * YS_LD + q4 * 32]);
+                    uint4* dst = reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV + q4 * 32);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) dst[i] = src[i];
+                }
+            } else {
+                const int cc = tid & 15;
+                float gwv[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) gwv[j] = gw[cc * 8 + j];
+                // the four rows of this 16-lane group: all sums of squares first, then one reciprocal square root per lane
+                uint4 yv4[4];
+                float ss4[4], inv4[4];
+#pragma unroll
+                for (int it = 0; it < 4; it++) {
+                    const int row = it * 16 + (tid >> 4);
+                    yv4[it] = *reinterpret_cast<const uint4*>(&ys[row * YS_LD + cc * 8]);
+                    float yy[8];
+                    unpack8(yv4[it], yy);
+                    double ss = 0.0;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
+                    ss4[it] = (float)row16_sum_d(ss);
+                }
+                rsqrt_rows<4>(ss4, eps, inv4, cc);
+#pragma unroll
+                for (int it = 0; it < 4; it++) {
+                    const int row = it * 16 + (tid >> 4);
+                    const int t = c * C + row;
+                    if (t >= S) continue;                                       // whole 16-lane groups leave together
+                    const uint4 zv = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
+                    float yy[8], zz[8];
+                    unpack8(yv4[it], yy);
+                    unpack8(zv, zz);
+                    uint32_t o[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv4[it]));
+                    reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV)[cc] =
+                        make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
+                }
+            }
+        }
+        __syncthreads();                                                        // ys is reused by the next round
+    }
+}
+
+// the two-launch form: 128 chain workgroups of 320 threads, then one output workgroup of 256 threads per (chunk, head)
+__global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
+                                                        float* st_out, _Float16* snap, int NC) {
+    __shared__ ChainLds chain_lds;
+    chain_role<false>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snap + FLAG_HALVES, nullptr, NC);
+}
 template <bool NORM>
 __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restrict__ ops, const _Float16* __restrict__ snap,
                                                          const float* __restrict__ gates, bf16_t* __restrict__ y,
                                                          const bf16_t* __restrict__ proj, const float* __restrict__ gw, float eps,
-                                                         int S) {
-    const int rec = blockIdx.x, c = rec / HV, h = rec % HV;
-    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+                                                         int S, int NC) {
     __shared__ __align__(16) bf16_t ys[C * YS_LD];
-    const half8* op = reinterpret_cast<const half8*>(ops + (size_t)rec * OP_HALVES) + lane;
-    const half8* sp = reinterpret_cast<const half8*>(snap + ((size_t)rec * 8 + 2 * w) * SNAP_HALVES) + lane;
-    half8 Sb[2][4], Db[2][2], Qt[16], At[8];
-#pragma unroll
-    for (int s = 0; s < 2; s++) {
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++) Sb[s][kb] = sp[s * (SNAP_HALVES / 8) + kb * 64];
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; kb2++) Db[s][kb2] = sp[s * (SNAP_HALVES / 8) + (SNAP_S / 8) + kb2 * 64];
+    // unit = blockIdx = chunk * HV + head, one round: output_role's unit u takes chunk u / HV + round * units_per_head
+    output_role<NORM, false>(ys, nullptr, blockIdx.x, NC, ops, snap + FLAG_HALVES, nullptr, gates, y, proj, gw, eps, S, NC);
+}
+
+// the one-launch form: grid = N_CHAIN + output workgroups (two units each), 512 threads: one workgroup per CU, all resident
+template <bool NORM>
+__global__ __launch_bounds__(512) void gdn_phase_b_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
+                                                          float* st_out, _Float16* snap, bf16_t* y, const bf16_t* proj,
+                                                          const float* gw, float eps, int S, int NC, int units_per_head) {
+    __shared__ ChainLds chain_lds;
+    __shared__ __align__(16) bf16_t ys[2][C * YS_LD];
+    __shared__ int ready[2];                                                    // chunks seen complete by each unit's polling wavefront
+    int* flags = reinterpret_cast<int*>(snap);
+    _Float16* snaps = snap + FLAG_HALVES;
+    if (blockIdx.x < N_CHAIN) {
+        chain_role<true>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snaps, flags, NC);
+        return;
     }
-#pragma unroll
-    for (int i = 0; i < 16; i++) Qt[i] = op[(OP_Q / 8) + i * 64];
-#pragma unroll
-    for (int i = 0; i < 8; i++) At[i] = op[(OP_A / 8) + i * 64];
-    f32x4 gam[NCT];                                                             // gamma of this lane's four rows of every row tile
-#pragma unroll
-    for (int ct = 0; ct < NCT; ct++) gam[ct] = *reinterpret_cast<const f32x4*>(gates + (size_t)rec * GATE_FLOATS + G_GAM + 16 * ct + 4 * g);
-#pragma unroll
-    for (int s = 0; s < 2; s++) {
-        f32x4 Y[NCT];
-#pragma unroll
-        for (int ct = 0; ct < NCT; ct++) Y[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++)
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Qt[ct * 4 + kb], Sb[s][kb], Y[ct], 0, 0, 0);
-#pragma unroll
-        for (int ct = 0; ct < NCT; ct++) Y[ct] *= gam[ct];
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; kb2++)
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(At[ct * 2 + kb2], Db[s][kb2], Y[ct], 0, 0, 0);
-#pragma unroll
-        for (int ct = 0; ct < NCT; ct++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) ys[(ct * 16 + 4 * g + r) * YS_LD + (2 * w + s) * 16 + n] = f2bf(Y[ct][r]);
-    }
+    if (threadIdx.x < 2) ready[threadIdx.x] = 0;
     __syncthreads();
-    if (!NORM) {
-        const int row = threadIdx.x >> 2, q4 = threadIdx.x & 3;
-        const int t = c * C + row;
-        if (t < S) {
-            const uint4* src = reinterpret_cast<const uint4*>(&ys[row * YS_LD + q4 * 32]);
-            uint4* dst = reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV + q4 * 32);
-#pragma unroll
-            for (int i = 0; i < 4; i++) dst[i] = src[i];
-        }
-    } else {
-        const int cc = threadIdx.x & 15;
-        float gwv[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) gwv[j] = gw[cc * 8 + j];
-        // the four rows of this 16-lane group: all sums of squares first, then one reciprocal square root per lane
-        uint4 yv4[4];
-        float ss4[4], inv4[4];
-#pragma unroll
-        for (int it = 0; it < 4; it++) {
-            const int row = it * 16 + (threadIdx.x >> 4);
-            yv4[it] = *reinterpret_cast<const uint4*>(&ys[row * YS_LD + cc * 8]);
-            float yy[8];
-            unpack8(yv4[it], yy);
-            double ss = 0.0;
-#pragma unroll
-            for (int j = 0; j < 4; j++) ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
-            ss4[it] = (float)row16_sum_d(ss);
-        }
-        rsqrt_rows<4>(ss4, eps, inv4, cc);
-#pragma unroll
-        for (int it = 0; it < 4; it++) {
-            const int row = it * 16 + (threadIdx.x >> 4);
-            const int t = c * C + row;
-            if (t >= S) continue;                                               // whole 16-lane groups leave together
-            const uint4 zv = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
-            float yy[8], zz[8];
-            unpack8(yv4[it], yy);
-            unpack8(zv, zz);
-            uint32_t o[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv4[it]));
-            reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV)[cc] =
-                make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
-        }
+    const int unit = (blockIdx.x - N_CHAIN) * 2 + (threadIdx.x >> 8);
+    output_role<NORM, true>(ys[threadIdx.x >> 8], ready + (threadIdx.x >> 8), unit, units_per_head, ops, snaps, flags, gates, y, proj, gw,
+                            eps, S, NC);
+    // the last output workgroup to finish leaves the flag area zero for the next launch: by then every chunk has been
+    // consumed, so every chain workgroup has made its last store to it
+    __shared__ int last;
+    if (threadIdx.x == 0) last = atomicAdd(flags + FLAG_DONE, 1) == (int)gridDim.x - N_CHAIN - 1;
+    __syncthreads();
+    if (last) {
+        if (threadIdx.x < N_CHAIN) __hip_atomic_store(flags + threadIdx.x * FLAG_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) __hip_atomic_store(flags + FLAG_DONE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -707,20 +852,32 @@ static int phase_b_launch(const void* ops, const void* U, const float* gC, void*
             return QT_ERR_LAUNCH;
         return QT_OK;
     }
-    hipLaunchKernelGGL(gdn_chain_kernel, dim3(HV * 8), dim3(320), 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in, state_out,
-                       (_Float16*)snap, NC);
-    QT_CHECK_LAUNCH();
-    if (norm)
-        hipLaunchKernelGGL(gdn_output_kernel<true>, dim3(NC * HV), dim3(256), 0, stream, (const _Float16*)ops,
-                           (const _Float16*)snap, gC, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S);
-    else
-        hipLaunchKernelGGL(gdn_output_kernel<false>, dim3(NC * HV), dim3(256), 0, stream, (const _Float16*)ops,
-                           (const _Float16*)snap, gC, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S);
+    if (NC >= FUSED_MIN_CHUNKS) {
+        // one launch: unit r of a head takes chunks r, r + UNITS_PER_HEAD, ...; two units per output workgroup
+        const dim3 grid(N_CHAIN + HV * UNITS_PER_HEAD / 2), block(512);
+        if (norm)
+            hipLaunchKernelGGL(gdn_phase_b_kernel<true>, grid, block, 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
+                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S, NC, UNITS_PER_HEAD);
+        else
+            hipLaunchKernelGGL(gdn_phase_b_kernel<false>, grid, block, 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
+                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S, NC,
+                               UNITS_PER_HEAD);
+    } else {
+        hipLaunchKernelGGL(gdn_chain_kernel, dim3(N_CHAIN), dim3(320), 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
+                           state_out, (_Float16*)snap, NC);
+        QT_CHECK_LAUNCH();
+        if (norm)
+            hipLaunchKernelGGL(gdn_output_kernel<true>, dim3(NC * HV), dim3(256), 0, stream, (const _Float16*)ops, (const _Float16*)snap,
+                               gC, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S, NC);
+        else
+            hipLaunchKernelGGL(gdn_output_kernel<false>, dim3(NC * HV), dim3(256), 0, stream, (const _Float16*)ops,
+                               (const _Float16*)snap, gC, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S, NC);
+    }
     QT_CHECK_LAUNCH();
     return QT_OK;
 }
 
-long qt_gdn_chunk_snap_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * 8 * SNAP_HALVES * 2; }
+long qt_gdn_chunk_snap_bytes(int S) { return S < 0 ? -1 : (long)FLAG_WORDS * 4 + (long)((S + C - 1) / C) * HV * 8 * SNAP_HALVES * 2; }
 
 int qt_gdn_phase_b(const void* ops, const void* U, const float* gC, void* snap, const float* state_in, float* state_out, void* y,
                    int S, hipStream_t stream) {

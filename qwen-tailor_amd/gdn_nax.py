@@ -66,6 +66,23 @@ def gdn_chunked(q, k, v, proj, A_log, dt_bias, state, relaxed=True, flags=DEFAUL
     return phase_b(q, k, v, ops, U, gC, state)
 
 
+_SNAP = {}            # (device index, stream handle) -> float16 tensor: flag area + chain snapshots
+_SNAP_RETIRED = []    # outgrown buffers stay alive: a captured HIP graph may hold their address
+
+
+def _snap_buffer(dev, nbytes):
+    """The buffer between phase B's chain and output workgroups, cached per (device, stream): its first KiB is the flag
+    area, which has to be zero before a launch and is left zero by it, so the buffer is zero-filled once, when it is made."""
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    buf = _SNAP.get(key)
+    if buf is None or buf.numel() * 2 < nbytes:
+        if buf is not None:
+            _SNAP_RETIRED.append(buf)
+        buf = torch.zeros(max(nbytes // 2, 8), dtype=torch.float16, device=dev)
+        _SNAP[key] = buf
+    return buf
+
+
 def _phase_b_args(S, Tb, Am, gv, state):
     ops, U, gC = L.dev(Tb, torch.float16, "Tb"), L.dev(Am, torch.float16, "Am"), L.dev(gv, torch.float32, "gv")
     lib = L.lib()
@@ -73,7 +90,7 @@ def _phase_b_args(S, Tb, Am, gv, state):
             gC.numel() * 4 < lib.qt_gdn_chunk_gc_bytes(S):
         raise ValueError("phase_b: the phase A records are too small for this many tokens")
     state = L.dev(state, torch.float32, "state").reshape(1, HV, DV, DK)
-    snap = torch.empty(max(lib.qt_gdn_chunk_snap_bytes(S) // 2, 8), dtype=torch.float16, device=state.device)
+    snap = _snap_buffer(state.device, lib.qt_gdn_chunk_snap_bytes(S))
     return ops, U, gC, snap, state, torch.empty_like(state)
 
 

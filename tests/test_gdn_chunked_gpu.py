@@ -125,14 +125,20 @@ def test_config2_chunked_prefill(qt, dev, T):
     check_equal("gdn_core conv tail", to_np(conv4)[0], otail)
 
 
-@pytest.mark.parametrize("T", [8192, 8131])
+@pytest.mark.parametrize("T", [8192, 8131, 4100])
 def test_config2_long_prefill(qt, dev, T):
-    """config 2's longest sweep point (T = 8192: a chain of 128 chunks, each step rounding its operands to half precision) and
-    the same with a partial last chunk, from a nonzero state, through the layer core (reference entry qwen35/gdn_nax.py:413-426).
+    """config 2's longest sweep point (T = 8192: a chain of 128 chunks, each step rounding its operands to half precision), the
+    same with a partial last chunk, and 65 chunks (the output units of the one-launch form of phase B, which these lengths
+    take, then run different numbers of rounds), from a nonzero state, through the layer core (reference entry
+    qwen35/gdn_nax.py:413-426).  Run twice on the same buffers: the second launch finds the progress words the first one left.
     The per-head errors are checked too: a head whose state decays fast must not hide behind the slow ones."""
     proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(2002 + T, T)
     o4, conv4, s4 = qt.prefill.gdn_core(to_dev(proj, dev, BF16), to_dev(cs[None], dev, BF16), to_dev(S0[None], dev), to_dev(cw, dev, BF16),
                                         to_dev(A_log, dev), to_dev(dtb, dev), to_dev(gw, dev))
+    o5, conv5, s5 = qt.prefill.gdn_core(to_dev(proj, dev, BF16), to_dev(cs[None], dev, BF16), to_dev(S0[None], dev), to_dev(cw, dev, BF16),
+                                        to_dev(A_log, dev), to_dev(dtb, dev), to_dev(gw, dev))
+    check_tensors_equal("second launch, outputs", o5, o4)
+    check_tensors_equal("second launch, state", s5, s4)
     oo, oy, otail, os_ = O.prefill_gdn(proj, cs, cw, A_log, dtb, S0, gw)
     e1 = check_rel("final state rel-L2", to_np(s4)[0], os_, 2e-3, rel_l2)
     e2 = check_rel("final state max", to_np(s4)[0], os_, 2e-3, rel_max)
