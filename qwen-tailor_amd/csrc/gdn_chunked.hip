@@ -457,35 +457,43 @@ __global__ __launch_bounds__(512) void gdn_phase_b_kernel(const _Float16* ops, c
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// Phase A: one workgroup of 256 threads per (chunk, head).
+// Phase A: one workgroup of 512 threads per (chunk, head), two workgroups per CU.
 //
-// The kernel is bound by its vector-ALU instruction count (two wavefronts per SIMD, little else to overlap with), so q, k
-// and v are converted to half precision ONCE, when they are staged into LDS, and every MFMA operand is then a plain LDS
-// read: row-major 16-byte reads for K K^T and Q K^T, the transposing load ds_read_b64_tr_b16 where the contraction runs
+// A (chunk, head) costs about 10^5 vector-ALU instructions of conv + SiLU + normalisation and a chain of dependent matrix
+// steps (K K^T, the 64 x 64 triangular inverse, the products with it) that keeps no unit busy.  The two run side by side:
+// wavefronts 0..3 (group M) convolve k, then walk the matrix chain while wavefronts 4..7 (group V) convolve q and v and
+// form A = lower(G * Q K^T).  Three workgroup barriers: table and taps ready; k and q staged; v staged.
+//
+// q, k and v are converted to half precision ONCE, when they are staged into LDS, and every MFMA operand is then a plain
+// LDS read: row-major 16-byte reads for K K^T and Q K^T, the transposing load ds_read_b64_tr_b16 where the contraction runs
 // over the tokens (K^T for Wn and Kh, V for U).  The per-token factors gamma and dec never touch an operand element:
 // gamma goes into Tb's columns for Wn, and the chain / output kernels apply dec and gamma to accumulator rows.
+//
+// The inverse T = (I + L)^-1, L = strict_lower(beta_i G_ij k_i . k_j), is exact fp32 work by blocks of 16 and stays inside
+// one wavefront per block ROW I: with LT = L^T and TT = T^T, column I of TT follows from (I + LT) TT = I as
+//     TT[I][I] = T_II^T,     TT[w][I] = -T_ww^T  sum_{J = w+1..I} LT[w][J] TT[J][I]        (w = I-1 .. 0).
+// In the accumulator layout (lane (n, g) holds rows 4g..4g+3 of column n) a block of TT is at once the B operand of the next
+// step and, read as a block of T, the A-operand layout (row n, columns 4g..4g+3) the products with T need; LT[w][J] as an
+// A operand is the accumulator layout of K_J K_w^T.  So no block of L or T goes through LDS except the four diagonal ones:
+// every wavefront of group M forms all four (lane group g inverts block g by forward substitution, column n per lane), and
+// writes them to the same LDS words (identical values; a wavefront reads back only after its own writes).
 // ------------------------------------------------------------------------------------------------------------------
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int QS_LD = DK + 8;        // row stride (halves) of Qs / Ks: 16-byte row reads of 16 rows hit distinct banks
 constexpr int VS_LD = DV + 16;       // row stride of Vs: the transposing loads (4 rows x 32 bytes per 16 lanes) hit distinct banks
-constexpr int LS_LD = C + 4;
+constexpr int ND_LD = 20;            // row stride (floats) of a diagonal block
+constexpr int ND_BLK = 16 * ND_LD + 4;   // floats between diagonal blocks: the four lane groups read distinct banks
 constexpr float LOG2E = 1.4426950408889634f;
 
-struct PhaseALds {                       // 70 KiB: two workgroups per CU
+struct PhaseALds {                       // 76.6 KiB: two workgroups per CU
     __align__(16) _Float16 Ks[C * QS_LD];
+    __align__(16) _Float16 Qs[C * QS_LD];
     __align__(16) _Float16 Vs[C * VS_LD];
-    union {
-        __align__(16) _Float16 Qs[C * QS_LD];    // until Q K^T is done
-        __align__(16) float Ls[C * LS_LD];       // then L = strict_lower(beta G K K^T)
-    };
-    union {
-        struct {                                 // fused conv only: the silu_bf16 table and this head's conv taps
-            __align__(16) bf16_t tab[SILU_TAB_SIZE];
-            __align__(16) bf16_t taps[3 * DK * 4];
-        };
-        __align__(16) float Ts[C * LS_LD];       // afterwards T = (I + L)^-1
-    };
+    __align__(16) bf16_t tab[SILU_TAB_SIZE];     // fused conv only: the silu_bf16 table and this head's conv taps
+    __align__(16) bf16_t taps[3 * DK * 4];
+    __align__(16) float Nd[4 * ND_BLK];          // diagonal blocks of L: [block][row][column]
+    __align__(16) float Td[4 * ND_BLK];          // their inverses, transposed: [block][column][row]
     float Lc2[C], beta[C], gam[C], dec[C];       // Lc2 = log2(e) * cumsum(log g)
 };
 
@@ -517,12 +525,104 @@ __device__ __forceinline__ half8 tokens_operand(const _Float16* base, int ld, in
     r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
     return r;
 }
+// K_I K_J^T for two 16-row blocks of Ks, accumulator layout: lane (n, g) gets k_{16 I + 4 g + r} . k_{16 J + n}
+__device__ __forceinline__ f32x4 kk_block(const _Float16* Ks, int I, int J, int n, int g) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kb = 0; kb < 4; kb++) {
+        const half8 a = *reinterpret_cast<const half8*>(&Ks[(16 * I + n) * QS_LD + 32 * kb + 8 * g]);
+        const half8 b = *reinterpret_cast<const half8*>(&Ks[(16 * J + n) * QS_LD + 32 * kb + 8 * g]);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+    }
+    return acc;
+}
 
-// Stores one token's normalized q, k and v (8 channels of each, bf16 pairs) as half precision into the row-major LDS tiles.
-__device__ __forceinline__ void stage_token(PhaseALds& L, int tl, int cc, const uint4& rq, const uint4& rk, const uint4& rv) {
-    *reinterpret_cast<half8*>(&L.Qs[tl * QS_LD + cc * 8]) = bf8_to_half8(rq);
-    *reinterpret_cast<half8*>(&L.Ks[tl * QS_LD + cc * 8]) = bf8_to_half8(rk);
-    *reinterpret_cast<half8*>(&L.Vs[tl * VS_LD + cc * 8]) = bf8_to_half8(rv);
+// The matrix chain of block row I (one wavefront of group M): returns Tb = T diag(beta) for rows 16 I + n as the two operand
+// forms of the products, tbU[kb2] = Tb[16 I + n][kperm(kb2, g, 0..7)] and tbW = the same with columns scaled by -gamma.
+template <int I>
+__device__ __forceinline__ void inverse_row(PhaseALds& L, int n, int g, half8 (&tbU)[2], half8 (&tbW)[2]) {
+    // diagonal blocks of L -> LDS (all four, in every wavefront)
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        const f32x4 acc = kk_block(L.Ks, b, b, n, g);
+        const f32x4 lci = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * b + 4 * g]);
+        const f32x4 bei = *reinterpret_cast<const f32x4*>(&L.beta[16 * b + 4 * g]);
+        const float lcj = L.Lc2[16 * b + n];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const float v = bei[r] * __builtin_amdgcn_exp2f(lci[r] - lcj) * acc[r];
+            L.Nd[b * ND_BLK + (4 * g + r) * ND_LD + n] = (4 * g + r > n) ? v : 0.f;
+        }
+    }
+    // lane (n, g): column n of the inverse of diagonal block g, by forward substitution
+    {
+        float x[16];
+        const float* nb = &L.Nd[g * ND_BLK];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float a = (i == n) ? 1.f : 0.f;
+#pragma unroll
+            for (int m = 0; m < i; m++) a -= nb[i * ND_LD + m] * x[m];
+            x[i] = a;
+        }
+        float* tb = &L.Td[g * ND_BLK + n * ND_LD];
+#pragma unroll
+        for (int i = 0; i < 16; i += 4) *reinterpret_cast<f32x4*>(tb + i) = f32x4{x[i], x[i + 1], x[i + 2], x[i + 3]};
+    }
+    __builtin_amdgcn_sched_barrier(0);                   // the substitution's sixteen values are dead before the blocks below are formed
+    // blocks of L below the diagonal that this row's recursion multiplies with: LB[J][w] = block (J, w), w < J <= I
+    f32x4 LB[4][4];
+#pragma unroll
+    for (int J = 1; J <= I; J++) {
+        const f32x4 lci = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * J + 4 * g]);
+        const f32x4 bei = *reinterpret_cast<const f32x4*>(&L.beta[16 * J + 4 * g]);
+#pragma unroll
+        for (int w = 0; w < J; w++) {
+            // (a zero offset passes through an empty asm: otherwise the rows of all four blocks stay in registers, 64 of the 128)
+            int zero = 0;
+            asm volatile("" : "+v"(zero));
+            const f32x4 acc = kk_block(L.Ks + zero, J, w, n, g);
+            const float lcj = L.Lc2[16 * w + n];
+#pragma unroll
+            for (int r = 0; r < 4; r++) LB[J][w][r] = bei[r] * __builtin_amdgcn_exp2f(lci[r] - lcj) * acc[r];
+        }
+    }
+    // column I of TT, upwards
+    f32x4 TT[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) TT[I][r] = L.Td[I * ND_BLK + (4 * g + r) * ND_LD + n];          // T_II[n][4 g + r]
+#pragma unroll
+    for (int w = I - 1; w >= 0; w--) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int J = w + 1; J <= I; J++)
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(LB[J][w][kk], TT[J][kk], acc, 0, 0, 0);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&L.Td[w * ND_BLK + n * ND_LD + 4 * g]);   // T_ww[4 g + kk][n]
+        f32x4 res = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) res = __builtin_amdgcn_mfma_f32_16x16x4f32(d4[kk], acc[kk], res, 0, 0, 0);
+        TT[w] = -res;
+    }
+    // TT[w][r] = T[16 I + n][16 w + 4 g + r]
+#pragma unroll
+    for (int kb2 = 0; kb2 < 2; kb2++) {
+        float u[8], v[8];
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            const int blk = 2 * kb2 + hf, cp = 16 * blk + 4 * g;
+            const f32x4 b4 = *reinterpret_cast<const f32x4*>(&L.beta[cp]);
+            const f32x4 g4 = *reinterpret_cast<const f32x4*>(&L.gam[cp]);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float t = (blk <= I) ? TT[blk <= I ? blk : 0][r] : 0.f;                   // blk is a constant after unrolling
+                u[4 * hf + r] = t * b4[r];
+                v[4 * hf + r] = -u[4 * hf + r] * g4[r];
+            }
+        }
+        tbU[kb2] = to_half8(u);
+        tbW[kb2] = to_half8(v);
+    }
 }
 
 // Phase A of one (chunk, head).  from_proj = false: q, k, v [S,16,128] bf16 are inputs (convolved, normalized: conv_prep's
@@ -532,7 +632,7 @@ __device__ __forceinline__ void stage_token(PhaseALds& L, int tl, int cc, const 
 // proj [S,8224] supplies the gate inputs a, b in both forms.  The two forms are ONE kernel with uniform branches, not two
 // template instances: everything after the staging of q, k, v is then the same machine code, so both forms give the same bits
 // (two instances are scheduled and contracted independently by the compiler and differed in the last place now and then).
-__global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bool from_proj, const bool write_qkv,
+__global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_proj, const bool write_qkv,
                                                           const bf16_t* __restrict__ proj, bf16_t* qi, bf16_t* ki, bf16_t* vi,
                                                           const bf16_t* __restrict__ cs, const bf16_t* __restrict__ cw,
                                                           const bf16_t* __restrict__ silu_tab, bf16_t* __restrict__ conv_out,
@@ -541,49 +641,52 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bool from_pro
                                                           float* __restrict__ gates, int S) {
     __shared__ PhaseALds L;
     const int c = blockIdx.x / HV, h = blockIdx.x % HV, t0 = c * C;
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    // (the wavefront number as a scalar: the branches on it are then real branches, which the barriers inside them need)
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool grpV = wv >= 4;                          // wavefronts 4..7
+    const int w = wv & 3;                               // wavefront within its group
+    const int gi = (tid & 255) >> 4, cc = tid & 15;     // conv: tokens 4 gi .. 4 gi + 3, channels 8 cc .. 8 cc + 7 of a part
     const size_t rec = (size_t)c * HV + h;
     _Float16* op = ops + rec * OP_HALVES;
-    const int gi = tid >> 4, cc = tid & 15;
+    bf16_t* const outA = grpV ? qi : ki;                // group M convolves k, group V q and then v
+    const int partA = grpV ? 0 : 1;
 
     // ---- the chunk's rows: every load is issued before anything else; rows past the end are zero (gdn_nax.py:172-174)
-    // one register array for both forms.  !from_proj: rw[p][rr] = token rr * 16 + gi of q / k / v, a lane 8 consecutive columns;
-    // from_proj: rw[p][d] = input row 4 gi - 3 + d of 8 channels of part p
-    uint4 rw[3][7];
+    // one register array per part for both forms.  !from_proj: rw[rr] = token rr * 16 + gi, a lane 8 consecutive columns;
+    // from_proj: rw[d] = input row 4 gi - 3 + d of 8 channels of the part
+    uint4 rwA[7], rwB[7];
     if (!from_proj) {
 #pragma unroll
         for (int rr = 0; rr < 4; rr++) {
             const int t = t0 + rr * 16 + gi;
             const size_t o = ((size_t)min(t, S - 1) * HV + h) * DK + cc * 8;
-            rw[0][rr] = *reinterpret_cast<const uint4*>(qi + o);
-            rw[1][rr] = *reinterpret_cast<const uint4*>(ki + o);
-            rw[2][rr] = *reinterpret_cast<const uint4*>(vi + o);
-            if (t >= S) rw[0][rr] = rw[1][rr] = rw[2][rr] = make_uint4(0, 0, 0, 0);
+            rwA[rr] = *reinterpret_cast<const uint4*>(outA + o);
+            if (grpV) rwB[rr] = *reinterpret_cast<const uint4*>(vi + o);
+            if (t >= S) rwA[rr] = rwB[rr] = make_uint4(0, 0, 0, 0);
         }
     } else {
+        const int chA = partA * KD + h * DK + cc * 8;
 #pragma unroll
-        for (int part = 0; part < 3; part++) {
-            const int ch0 = part * KD + h * DK + cc * 8;
-#pragma unroll
-            for (int d = 0; d < 7; d++) {
-                const int tt = min(t0 + 4 * gi - 3 + d, S - 1);
-                rw[part][d] = *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0);
-            }
+        for (int d = 0; d < 7; d++) {
+            const int tt = min(t0 + 4 * gi - 3 + d, S - 1);
+            rwA[d] = *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + chA : proj + (size_t)tt * PW + chA);
         }
         // the head's conv taps (3 x 128 channels x 4 taps) go through LDS: every token group needs the same 3 KiB
-        if (tid < 192) {
-            const int part = tid >> 6, i = tid & 63;
-            reinterpret_cast<uint4*>(L.taps)[tid] = reinterpret_cast<const uint4*>(cw + (size_t)(part * KD + h * DK) * 4)[i];
+        if (wv >= 5) {
+            const int i3 = tid - 320, part = i3 >> 6, i = i3 & 63;
+            reinterpret_cast<uint4*>(L.taps)[i3] = reinterpret_cast<const uint4*>(cw + (size_t)(part * KD + h * DK) * 4)[i];
         }
-        if (conv_out && c == (S - 1) / C && tid < 3 * 48) {            // new conv window: input rows S-3 .. S-1 of this head's channels
-            const int r = tid / 48, part = (tid % 48) >> 4, ch0 = part * KD + h * DK + (tid & 15) * 8, tt = S - 3 + r;
+        if (conv_out && c == (S - 1) / C && tid >= 64 && tid < 64 + 3 * 48) {   // new conv window: input rows S-3 .. S-1 of this head's channels
+            const int i3 = tid - 64;
+            const int r = i3 / 48, part = (i3 % 48) >> 4, ch0 = part * KD + h * DK + (i3 & 15) * 8, tt = S - 3 + r;
             *reinterpret_cast<uint4*>(conv_out + r * CD + ch0) =
                 *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + ch0 : proj + (size_t)tt * PW + ch0);
         }
     }
 
-    // ---- gates of the chunk's tokens (gdn_nax.py:80-104): wave 0, one token per lane
-    if (w == 0) {
+    // ---- gates of the chunk's tokens (gdn_nax.py:80-104): wavefront 0, one token per lane
+    if (wv == 0) {
         const int t = t0 + lane;
         float lg = 0.f, be = 0.f;
         if (t < S) {
@@ -614,72 +717,66 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bool from_pro
         gp[G_DEC + lane] = dc;
         if (lane >= 60) gp[G_GC + lane - 60] = lane == 60 ? expf(tot) : 0.f;
     }
-    if (!from_proj) {
+    if (from_proj) silu_table_fill(L.tab, silu_tab, tid, 512);
+    __syncthreads();
+
+    // ---- k (group M) and q (group V): conv + SiLU + L2 norm, staged as half precision
+    {
+        _Float16* dst = grpV ? L.Qs : L.Ks;
+        if (!from_proj) {
 #pragma unroll
-        for (int rr = 0; rr < 4; rr++) stage_token(L, rr * 16 + gi, cc, rw[0][rr], rw[1][rr], rw[2][rr]);
-    } else {
-        silu_table_fill(L.tab, silu_tab, tid, 256);
-        __syncthreads();
-        const float scq = BF(INV_SCALE * INV_SCALE), sck = BF(INV_SCALE);
-        uint4 pk[4][3];
-        float ss[8], rr[8];
+            for (int rr = 0; rr < 4; rr++) *reinterpret_cast<half8*>(&dst[(rr * 16 + gi) * QS_LD + cc * 8]) = bf8_to_half8(rwA[rr]);
+        } else {
+            const float sc = grpV ? BF(INV_SCALE * INV_SCALE) : BF(INV_SCALE);
+            uint4 wt[4], pk[4];
+            float ss[4], rr[4];
 #pragma unroll
-        for (int part = 0; part < 3; part++) {
-            uint4 wt[4];
+            for (int e = 0; e < 4; e++) wt[e] = *reinterpret_cast<const uint4*>(&L.taps[(partA * DK + cc * 8 + 2 * e) * 4]);
 #pragma unroll
-            for (int e = 0; e < 4; e++) wt[e] = *reinterpret_cast<const uint4*>(&L.taps[(part * DK + cc * 8 + 2 * e) * 4]);
+            for (int j = 0; j < 4; j++) ss[j] = (float)row16_sum_d(conv8_silu_packed(L.tab, rwA[j], rwA[j + 1], rwA[j + 2], rwA[j + 3], wt, pk[j]));
+            if (grpV) {                                  // v's rows: requested once q's are consumed (the register file holds one set)
+                const int chB = 2 * KD + h * DK + cc * 8;
+#pragma unroll
+                for (int d = 0; d < 7; d++) {
+                    const int tt = min(t0 + 4 * gi - 3 + d, S - 1);
+                    rwB[d] = *reinterpret_cast<const uint4*>(tt < 0 ? cs + (tt + 3) * CD + chB : proj + (size_t)tt * PW + chB);
+                }
+            }
+            rsqrt_rows<4>(ss, qk_eps(), rr, cc);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const double sq = conv8_silu_packed(L.tab, rw[part][j], rw[part][j + 1], rw[part][j + 2], rw[part][j + 3], wt, pk[j][part]);
-                if (part < 2) ss[2 * j + part] = (float)row16_sum_d(sq);
+                const int tl = 4 * gi + j, t = t0 + tl;
+                uint4 p = scale8_packed(pk[j], rr[j], sc);
+                if (t >= S) p = make_uint4(0, 0, 0, 0);
+                if (write_qkv && t < S) *reinterpret_cast<uint4*>(outA + ((size_t)t * HV + h) * DK + cc * 8) = p;
+                *reinterpret_cast<half8*>(&dst[tl * QS_LD + cc * 8]) = bf8_to_half8(p);
             }
-        }
-        rsqrt_rows<8>(ss, qk_eps(), rr, cc);
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int tl = 4 * gi + j, t = t0 + tl;
-            uint4 pq = scale8_packed(pk[j][0], rr[2 * j], scq), pkk = scale8_packed(pk[j][1], rr[2 * j + 1], sck), pv = pk[j][2];
-            if (t >= S) pq = pkk = pv = make_uint4(0, 0, 0, 0);
-            if (write_qkv && t < S) {
-                const size_t o = ((size_t)t * HV + h) * DK + cc * 8;
-                *reinterpret_cast<uint4*>(qi + o) = pq;
-                *reinterpret_cast<uint4*>(ki + o) = pkk;
-                *reinterpret_cast<uint4*>(vi + o) = pv;
-            }
-            stage_token(L, tl, cc, pq, pkk, pv);
         }
     }
     __syncthreads();
 
-    // ---- K K^T (lower tiles) -> L, and (Q K^T)^T -> Am, on MFMA.  Wave w: row of tiles ti = 3 - w of K K^T and the Am / Qh
-    // tiles of ct = w, plus the Kh tiles of mt = 2 w, 2 w + 1.  L stays in registers until every wave is done with Qs, whose
-    // LDS it then takes over.  G_ij = exp(Lc_i - Lc_j) = exp2(Lc2_i - Lc2_j).
-    f32x4 Lreg[4];
-    {
-        const int ti = 3 - w;
-        f32x4 lci, bei;                                        // Lc2 and beta of this lane's rows i = 16 ti + 4 g + r
-        lci = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * ti + 4 * g]);
-        bei = *reinterpret_cast<const f32x4*>(&L.beta[16 * ti + 4 * g]);
+    if (grpV) {
+        // ---- v: conv + SiLU, staged
+        if (!from_proj) {
 #pragma unroll
-        for (int tj = 0; tj < 4; tj++) {
-            Lreg[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (tj <= ti) {
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            for (int rr = 0; rr < 4; rr++) *reinterpret_cast<half8*>(&L.Vs[(rr * 16 + gi) * VS_LD + cc * 8]) = bf8_to_half8(rwB[rr]);
+        } else {
+            uint4 wt[4];
 #pragma unroll
-                for (int kb = 0; kb < 4; kb++) {
-                    const half8 a = *reinterpret_cast<const half8*>(&L.Ks[(16 * ti + n) * QS_LD + 32 * kb + 8 * g]);
-                    const half8 b = *reinterpret_cast<const half8*>(&L.Ks[(16 * tj + n) * QS_LD + 32 * kb + 8 * g]);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
-                }
-                const float lcj = L.Lc2[16 * tj + n];
+            for (int e = 0; e < 4; e++) wt[e] = *reinterpret_cast<const uint4*>(&L.taps[(2 * DK + cc * 8 + 2 * e) * 4]);
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const float v = bei[r] * __builtin_amdgcn_exp2f(lci[r] - lcj) * acc[r];
-                    Lreg[tj][r] = (tj < ti || 4 * g + r > n) ? v : 0.f;
-                }
+            for (int j = 0; j < 4; j++) {
+                const int tl = 4 * gi + j, t = t0 + tl;
+                uint4 p;
+                (void)conv8_silu_packed(L.tab, rwB[j], rwB[j + 1], rwB[j + 2], rwB[j + 3], wt, p);
+                if (t >= S) p = make_uint4(0, 0, 0, 0);
+                if (write_qkv && t < S) *reinterpret_cast<uint4*>(vi + ((size_t)t * HV + h) * DK + cc * 8) = p;
+                *reinterpret_cast<half8*>(&L.Vs[tl * VS_LD + cc * 8]) = bf8_to_half8(p);
             }
         }
-        const int ct = w, co = 16 * ct + n;                         // Am: rows c_out = 16 ct + n, k = c_in (permuted)
+        __syncthreads();
+        // ---- Am = lower_incl(G * Q K^T) transposed, rows c_out = 16 ct + n, k = c_in (permuted); G_ij = exp2(Lc2_i - Lc2_j)
+        const int ct = w, co = 16 * ct + n;
         const float lco = L.Lc2[co];
         for (int kb2 = 0; kb2 < 2; kb2++) {
             f32x4 part[2];
@@ -719,113 +816,47 @@ __global__ __launch_bounds__(256, 2) void gdn_phase_a_kernel(const bool from_pro
             for (int kb2 = 0; kb2 < 2; kb2++)
                 *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g);
         }
+        return;
     }
-    __syncthreads();
-    for (int i = tid; i < C * LS_LD / 4; i += 256) reinterpret_cast<f32x4*>(L.Ts)[i] = f32x4{0.f, 0.f, 0.f, 0.f};   // blocks above the diagonal stay zero
-    {
-        const int ti = 3 - w;
-#pragma unroll
-        for (int tj = 0; tj < 4; tj++)
-            if (tj <= ti) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) L.Ls[(16 * ti + 4 * g + r) * LS_LD + 16 * tj + n] = Lreg[tj][r];
-            }
-    }
-    __syncthreads();
 
-    // ---- T = (I + L)^-1 by blocks of 16 (exact fp32: forward substitution on the diagonal blocks, fp32 MFMA below them)
-    f32x4 TR[4];                                   // TR[d] = block (w + d, w) of T, accumulator layout
-    {
-        float x[16];
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            float a = (i == n) ? 1.f : 0.f;
-            const float* lr = &L.Ls[(16 * w + i) * LS_LD + 16 * w];
-#pragma unroll
-            for (int m = 0; m < i; m++) a -= lr[m] * x[m];
-            x[i] = a;
-        }
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            float v = 0.f;
-#pragma unroll
-            for (int i = 0; i < 16; i++) v = (i == 4 * g + r) ? x[i] : v;
-            TR[0][r] = v;
-            L.Ts[(16 * w + 4 * g + r) * LS_LD + 16 * w + n] = v;
-        }
+    // ---- group M: T = (I + L)^-1 by block rows, then Wn^T = K^T (-Tb gamma)^T and U = Tb V on fp16 MFMA; wavefront w owns the
+    // chunk rows of tile ct = w.  Both Tb operands hold Tb[16 ct + n][kperm(kb2, g, 0..7)]: as the A operand of U, and (columns
+    // scaled by -gamma) as the B operand of Wn^T.
+    __builtin_amdgcn_s_setprio(2);                       // few instructions, all of them on the critical path
+    half8 tbU[2], tbW[2];
+    switch (w) {
+        case 0: inverse_row<0>(L, n, g, tbU, tbW); break;
+        case 1: inverse_row<1>(L, n, g, tbU, tbW); break;
+        case 2: inverse_row<2>(L, n, g, tbU, tbW); break;
+        default: inverse_row<3>(L, n, g, tbU, tbW); break;
     }
-    __syncthreads();
+    const int ct = w, nkb = ct < 2 ? 1 : 2;              // Tb is lower triangular: columns past the row tile are zero
+    for (int kb = 0; kb < 4; kb++) {
+        f32x4 acc[2];
 #pragma unroll
-    for (int d = 1; d < 4; d++) {
-        if (w + d < 4) {
-            const int I = w + d;
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int e = 0; e < d; e++) {
-                const f32x4 a4 = *reinterpret_cast<const f32x4*>(&L.Ls[(16 * I + n) * LS_LD + 16 * (w + e) + 4 * g]);
-#pragma unroll
-                for (int kk = 0; kk < 4; kk++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[kk], TR[e][kk], acc, 0, 0, 0);
-            }
-            f32x4 res = {0.f, 0.f, 0.f, 0.f};
-            const f32x4 d4 = *reinterpret_cast<const f32x4*>(&L.Ts[(16 * I + n) * LS_LD + 16 * I + 4 * g]);
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) res = __builtin_amdgcn_mfma_f32_16x16x4f32(d4[kk], acc[kk], res, 0, 0, 0);
-            TR[d] = -res;
-#pragma unroll
-            for (int r = 0; r < 4; r++) L.Ts[(16 * I + 4 * g + r) * LS_LD + 16 * w + n] = TR[d][r];
-        }
-    }
-    __syncthreads();
-
-    // ---- Wn^T = K^T (-Tb gamma)^T and U = Tb V on fp16 MFMA; wave w owns the chunk rows of tile ct = w.  Both Tb operands hold
-    // Tb[16 ct + n][kperm(kb2, g, 0..7)]: as the A operand of U, and (columns scaled by -gamma) as the B operand of Wn^T.
-    {
-        const int ct = w, nkb = ct < 2 ? 1 : 2;                     // Tb is lower triangular: columns past the row tile are zero
-        half8 tbU[2], tbW[2];
-#pragma unroll
-        for (int kb2 = 0; kb2 < 2; kb2++) {
-            float u[8], v[8];
-#pragma unroll
-            for (int hf = 0; hf < 2; hf++) {
-                const int cp = 32 * kb2 + 16 * hf + 4 * g;
-                const f32x4 t4 = *reinterpret_cast<const f32x4*>(&L.Ts[(16 * ct + n) * LS_LD + cp]);
-                const f32x4 b4 = *reinterpret_cast<const f32x4*>(&L.beta[cp]);
-                const f32x4 g4 = *reinterpret_cast<const f32x4*>(&L.gam[cp]);
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    u[4 * hf + r] = t4[r] * b4[r];
-                    v[4 * hf + r] = -u[4 * hf + r] * g4[r];
-                }
-            }
-            tbU[kb2] = to_half8(u);
-            tbW[kb2] = to_half8(v);
-        }
-        for (int kb = 0; kb < 4; kb++) {
-            f32x4 acc[2];
-#pragma unroll
-            for (int hf = 0; hf < 2; hf++) {
-                const int mt = 2 * kb + hf;
-                acc[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int kb2 = 0; kb2 < 2; kb2++) {
-                    if (kb2 >= nkb) continue;
-                    acc[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g), tbW[kb2], acc[hf], 0, 0, 0);
-                }
-            }
-            *reinterpret_cast<half8*>(op + OP_W + (ct * 4 + kb) * 512 + lane * 8) = pack_half8(acc[0], acc[1]);
-        }
-        _Float16* up = U + rec * U_HALVES;
-        for (int sl = 0; sl < 8; sl++) {
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int hf = 0; hf < 2; hf++) {
+            const int mt = 2 * kb + hf;
+            acc[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kb2 = 0; kb2 < 2; kb2++) {
                 if (kb2 >= nkb) continue;
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tbU[kb2], tokens_operand(L.Vs, VS_LD, kb2, 16 * sl, n, g), acc, 0, 0, 0);
+                acc[hf] = __builtin_amdgcn_mfma_f32_16x16x32_f16(tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g), tbW[kb2], acc[hf], 0, 0, 0);
             }
-            half4 uh;
-            uh[0] = (_Float16)acc[0]; uh[1] = (_Float16)acc[1]; uh[2] = (_Float16)acc[2]; uh[3] = (_Float16)acc[3];
-            *reinterpret_cast<half4*>(up + ((sl * NCT + ct) * 64 + lane) * 4) = uh;
         }
+        *reinterpret_cast<half8*>(op + OP_W + (ct * 4 + kb) * 512 + lane * 8) = pack_half8(acc[0], acc[1]);
+    }
+    __syncthreads();                                     // v is staged
+    _Float16* up = U + rec * U_HALVES;
+    for (int sl = 0; sl < 8; sl++) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; kb2++) {
+            if (kb2 >= nkb) continue;
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tbU[kb2], tokens_operand(L.Vs, VS_LD, kb2, 16 * sl, n, g), acc, 0, 0, 0);
+        }
+        half4 uh;
+        uh[0] = (_Float16)acc[0]; uh[1] = (_Float16)acc[1]; uh[2] = (_Float16)acc[2]; uh[3] = (_Float16)acc[3];
+        *reinterpret_cast<half4*>(up + ((sl * NCT + ct) * 64 + lane) * 4) = uh;
     }
 }
 
@@ -897,7 +928,7 @@ int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v
     for (const void* p : {proj, q, k, v, (const void*)ops, (const void*)U, (const void*)gC})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     const int NC = (S + C - 1) / C;
-    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(256), 0, stream, false, false, (const bf16_t*)proj, (bf16_t*)q,
+    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(512), 0, stream, false, false, (const bf16_t*)proj, (bf16_t*)q,
                        (bf16_t*)k, (bf16_t*)v, (const bf16_t*)nullptr, (const bf16_t*)nullptr, (const bf16_t*)nullptr,
                        (bf16_t*)nullptr, A_log, dt_bias, (_Float16*)ops, (_Float16*)U, gC, S);
     QT_CHECK_LAUNCH();
@@ -916,7 +947,7 @@ int qt_gdn_phase_a_conv(const void* proj, const void* conv_state, const void* co
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if (conv_out == conv_state) return QT_ERR_UNSUPPORTED;          // the old window is still being read when the new one is written
     const int NC = (S + C - 1) / C;
-    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(256), 0, stream, true, q != nullptr, (const bf16_t*)proj, (bf16_t*)q,
+    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(512), 0, stream, true, q != nullptr, (const bf16_t*)proj, (bf16_t*)q,
                        (bf16_t*)k, (bf16_t*)v, (const bf16_t*)conv_state, (const bf16_t*)conv_w, (const bf16_t*)silu_table,
                        (bf16_t*)conv_out, A_log, dt_bias, (_Float16*)ops, (_Float16*)U, gC, S);
     QT_CHECK_LAUNCH();

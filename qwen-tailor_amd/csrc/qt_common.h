@@ -96,9 +96,9 @@ __device__ __forceinline__ float conv_silu(float w0, float w1, float w2, float x
 }
 
 // silu_bf16 is a bf16 -> bf16 map, so kernels that evaluate it many times per thread read it from a table in LDS:
-// 2 signs x 22 exponents (bf16 exponent fields 110..131, 2^-17 <= |x| < 2^5) x 128 mantissas = 5632 entries (11 KiB).
-// Inputs outside the range (about one in 10^5 for conv sums of unit-variance data) are evaluated directly.
-constexpr int SILU_TAB_LO = 110, SILU_TAB_N = 22 * 128, SILU_TAB_SIZE = 2 * SILU_TAB_N;
+// 2 signs x 24 exponents (bf16 exponent fields 110..133, 2^-17 <= |x| < 2^7) x 128 mantissas = 6144 entries (12 KiB).
+// Outside that range the map needs no exponential (silu_out_of_table).
+constexpr int SILU_TAB_LO = 110, SILU_TAB_N = 24 * 128, SILU_TAB_SIZE = 2 * SILU_TAB_N;
 __device__ __forceinline__ bf16_t silu_table_entry(int i) {
     const bf16_t xb = (bf16_t)(((i / SILU_TAB_N) << 15) | (SILU_TAB_LO * 128 + i % SILU_TAB_N));
     return f2bf(silu_bf16(bf2f(xb)));
@@ -112,11 +112,17 @@ __device__ __forceinline__ void silu_table_fill(bf16_t* tab, const bf16_t* __res
         for (int i = tid; i < SILU_TAB_SIZE; i += nthreads) tab[i] = silu_table_entry(i);
     }
 }
+// silu_bf16 outside the table's range.  Below 2^-17, exp(|x|) rounds to 1 in bf16 and the sigmoid is exactly 1/2.  From 2^7 on,
+// exp(|x|) overflows float: the sigmoid is 1 for x > 0 (the result is x) and +0 for x < 0 (the result is x * 0: -0, and NaN for
+// -inf).  NaN stays NaN.
+__device__ __forceinline__ float silu_out_of_table(float x) {
+    if (fabsf(x) < 1.0f) return BF(x * 0.5f);
+    return x > 0.0f ? x : x * 0.0f;
+}
 __device__ __forceinline__ float silu_lookup(const bf16_t* tab, bf16_t xb) {
     const unsigned idx = (xb & 0x7fffu) - SILU_TAB_LO * 128;                    // wraps for small |x|
     if (idx < (unsigned)SILU_TAB_N) return bf2f(tab[(xb >> 15) * SILU_TAB_N + idx]);
-    if ((xb & 0x7fffu) < SILU_TAB_LO * 128) return BF(bf2f(xb) * 0.5f);
-    return silu_bf16(bf2f(xb));
+    return silu_out_of_table(bf2f(xb));
 }
 // conv4 + silu through the table: taps in c (4 bf16), inputs oldest first
 __device__ __forceinline__ float conv_silu_tab(const bf16_t* tab, float w0, float w1, float w2, float x, uint2 c) {
@@ -127,18 +133,18 @@ __device__ __forceinline__ float conv_silu_tab(const bf16_t* tab, float w0, floa
     return silu_lookup(tab, f2bf(s));
 }
 // Branch-free form for hot loops: inputs outside the table return a placeholder and set `rare`; the caller then re-evaluates
-// that group of channels through conv8_silu_slow in one unlikely block (one branch per 8 channels instead of one per channel).
+// that group of channels in one unlikely block (one branch per 8 channels instead of one per channel).
 __device__ __forceinline__ float silu_lookup_fast(const bf16_t* tab, bf16_t xb, bool& rare) {
     const unsigned idx = (xb & 0x7fffu) - SILU_TAB_LO * 128;                      // wraps for small |x|
     const bool in_tab = idx < (unsigned)SILU_TAB_N;
     rare |= !in_tab;
     return bf2f(tab[(xb >> 15) * SILU_TAB_N + (in_tab ? idx : 0u)]);
 }
-__device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]);
+__device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]) {
+    f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
+    f[4] = lo_bf(w.z); f[5] = hi_bf(w.z); f[6] = lo_bf(w.w); f[7] = hi_bf(w.w);
+}
 // conv4 + silu of 8 consecutive channels of one token: rows x0..x3 (oldest first, 8 bf16 each), taps wt (4 bf16 per channel)
-struct F8 { float v[8]; };
-static __device__ __attribute__((always_inline)) inline F8 conv8_silu_slow(uint4 x0, uint4 x1, uint4 x2, uint4 x3, uint4 w0, uint4 w1, uint4 w2,
-                                                               uint4 w3);
 __device__ __forceinline__ void conv8_silu_tab(const bf16_t* tab, const uint4& x0, const uint4& x1, const uint4& x2,
                                                const uint4& x3, const uint4 (&wt)[4], float (&u)[8]) {
     float a[8], b[8], c[8], d[8];
@@ -158,32 +164,18 @@ __device__ __forceinline__ void conv8_silu_tab(const bf16_t* tab, const uint4& x
         u[e] = silu_lookup_fast(tab, f2bf(s), rare);
     }
     if (__builtin_expect(rare, 0)) {
-        const F8 r = conv8_silu_slow(x0, x1, x2, x3, wt[0], wt[1], wt[2], wt[3]);
 #pragma unroll
-        for (int e = 0; e < 8; e++) u[e] = r.v[e];
+        for (int e = 0; e < 8; e++) {
+            const uint4 ww = wt[e >> 1];
+            const uint32_t c0 = (e & 1) ? ww.z : ww.x, c1 = (e & 1) ? ww.w : ww.y;
+            float s = a[e] * lo_bf(c0);
+            s = s + b[e] * hi_bf(c0);
+            s = s + c[e] * lo_bf(c1);
+            s = s + d[e] * hi_bf(c1);
+            const bf16_t xb = f2bf(s);
+            if (((xb & 0x7fffu) - SILU_TAB_LO * 128) >= (unsigned)SILU_TAB_N) u[e] = silu_out_of_table(bf2f(xb));
+        }
     }
-}
-__device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]) {
-    f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
-    f[4] = lo_bf(w.z); f[5] = hi_bf(w.z); f[6] = lo_bf(w.w); f[7] = hi_bf(w.w);
-}
-
-static __device__ __attribute__((always_inline)) inline F8 conv8_silu_slow(uint4 x0, uint4 x1, uint4 x2, uint4 x3, uint4 w0, uint4 w1, uint4 w2,
-                                                               uint4 w3) {
-    float a[8], b[8], c[8], d[8];
-    unpack8(x0, a);
-    unpack8(x1, b);
-    unpack8(x2, c);
-    unpack8(x3, d);
-    const uint4 wt[4] = {w0, w1, w2, w3};
-    F8 r;
-#pragma unroll
-    for (int e = 0; e < 8; e += 2) {
-        const uint4 ww = wt[e >> 1];
-        r.v[e] = conv_silu(a[e], b[e], c[e], d[e], make_uint2(ww.x, ww.y));
-        r.v[e + 1] = conv_silu(a[e + 1], b[e + 1], c[e + 1], d[e + 1], make_uint2(ww.z, ww.w));
-    }
-    return r;
 }
 
 // conv4 + silu of 8 channels of one token, packed as bf16 pairs (the values are bf16-exact), and their exact sum of squares

@@ -182,3 +182,27 @@ def test_fused_conv_phase_a_equals_separate_kernels(qt, dev, T):
                        ("ops (no q, k, v stored)", ops2, ops0), ("U (no q, k, v stored)", U2, U0), ("gC (no q, k, v stored)", gC2, gC0)):
         check_tensors_equal(name, a, b)
     check_equal("conv tail", to_np(tail), np.concatenate([cs, proj[:, :CD]], axis=0)[-3:])
+
+
+def test_fused_conv_silu_exhaustive(qt, dev):
+    """every finite bf16 value as a conv sum (taps 0, 0, 0, 1) through the fused conv of phase A: the SiLU table and what
+    lies outside it, against the restatement of silu_bf16 (mslib.py:21-22)"""
+    f = (np.arange(65536, dtype=np.uint32) << 16).view(np.float32)
+    x = f[np.isfinite(f)]
+    S = 32
+    gen = torch.Generator().manual_seed(7)
+    proj = rand_bf(gen, (S, PW))
+    vals = np.resize(x, S * 2048).reshape(S, 2048)
+    proj[:, 4096:6144] = vals
+    cw, A_log, dtb, gw = layer_params(3)
+    cw[4096:6144] = (0.0, 0.0, 0.0, 1.0)
+    q, k, v, ops, U, gC = qt.gdn_nax.prep_a(to_dev(proj, dev, BF16), torch.zeros((3, CD), dtype=BF16, device=dev), to_dev(cw, dev, BF16),
+                                             to_dev(A_log, dev), to_dev(dtb, dev))
+    got, ref = to_np(v).reshape(S, 2048), O.silu_bf16(vals)
+    check_equal("silu of every finite bf16 value", got, ref)
+    nz = vals != 0                                                            # (a conv sum of zeros is +0 whatever the sign of x)
+    assert np.array_equal(np.signbit(got[nz]), np.signbit(ref[nz])), "sign of a zero result"
+    q2, k2, v2 = qt.prefill.conv_prep(to_dev(proj, dev, BF16), torch.zeros((3, CD), dtype=BF16, device=dev), to_dev(cw, dev, BF16))
+    check_tensors_equal("conv_prep v", v2, v)
+    check_tensors_equal("conv_prep q", q2, q)
+    check_tensors_equal("conv_prep k", k2, k)
