@@ -96,11 +96,13 @@ __device__ __forceinline__ float conv_silu(float w0, float w1, float w2, float x
 }
 
 // silu_bf16 is a bf16 -> bf16 map, so kernels that evaluate it many times per thread read it from a table in LDS:
-// 2 signs x 24 exponents (bf16 exponent fields 110..133, 2^-17 <= |x| < 2^7) x 128 mantissas = 6144 entries (12 KiB).
-// Outside that range the map needs no exponential (silu_out_of_table).
-constexpr int SILU_TAB_LO = 110, SILU_TAB_N = 24 * 128, SILU_TAB_SIZE = 2 * SILU_TAB_N;
+// 24 exponents (bf16 exponent fields 110..133, 2^-17 <= |x| < 2^7) x 128 mantissas x 2 signs = 6144 entries (12 KiB), the two
+// signs of a magnitude side by side: entry index = rotl16(x, 1) - 2 * (110 << 7).  Outside that range the map needs no
+// exponential (silu_out_of_table).  The table array has 8 more entries: index SILU_TAB_N2 is where out-of-range lookups land.
+constexpr int SILU_TAB_LO = 110, SILU_TAB_N2 = 2 * 24 * 128, SILU_TAB_SIZE = SILU_TAB_N2 + 8;
 __device__ __forceinline__ bf16_t silu_table_entry(int i) {
-    const bf16_t xb = (bf16_t)(((i / SILU_TAB_N) << 15) | (SILU_TAB_LO * 128 + i % SILU_TAB_N));
+    if (i >= SILU_TAB_N2) return 0;
+    const bf16_t xb = (bf16_t)(((i & 1) << 15) | (SILU_TAB_LO * 128 + (i >> 1)));
     return f2bf(silu_bf16(bf2f(xb)));
 }
 // fills `tab` (LDS) from a prebuilt copy in global memory, or computes it when there is none
@@ -119,82 +121,90 @@ __device__ __forceinline__ float silu_out_of_table(float x) {
     if (fabsf(x) < 1.0f) return BF(x * 0.5f);
     return x > 0.0f ? x : x * 0.0f;
 }
-__device__ __forceinline__ float silu_lookup(const bf16_t* tab, bf16_t xb) {
-    const unsigned idx = (xb & 0x7fffu) - SILU_TAB_LO * 128;                    // wraps for small |x|
-    if (idx < (unsigned)SILU_TAB_N) return bf2f(tab[(xb >> 15) * SILU_TAB_N + idx]);
-    return silu_out_of_table(bf2f(xb));
-}
-// conv4 + silu through the table: taps in c (4 bf16), inputs oldest first
-__device__ __forceinline__ float conv_silu_tab(const bf16_t* tab, float w0, float w1, float w2, float x, uint2 c) {
-    float s = w0 * lo_bf(c.x);
-    s = s + w1 * hi_bf(c.x);
-    s = s + w2 * lo_bf(c.y);
-    s = s + x * hi_bf(c.y);
-    return silu_lookup(tab, f2bf(s));
-}
-// Branch-free form for hot loops: inputs outside the table return a placeholder and set `rare`; the caller then re-evaluates
-// that group of channels in one unlikely block (one branch per 8 channels instead of one per channel).
-__device__ __forceinline__ float silu_lookup_fast(const bf16_t* tab, bf16_t xb, bool& rare) {
-    const unsigned idx = (xb & 0x7fffu) - SILU_TAB_LO * 128;                      // wraps for small |x|
-    const bool in_tab = idx < (unsigned)SILU_TAB_N;
-    rare |= !in_tab;
-    return bf2f(tab[(xb >> 15) * SILU_TAB_N + (in_tab ? idx : 0u)]);
-}
 __device__ __forceinline__ void unpack8(uint4 w, float (&f)[8]) {
     f[0] = lo_bf(w.x); f[1] = hi_bf(w.x); f[2] = lo_bf(w.y); f[3] = hi_bf(w.y);
     f[4] = lo_bf(w.z); f[5] = hi_bf(w.z); f[6] = lo_bf(w.w); f[7] = hi_bf(w.w);
 }
-// conv4 + silu of 8 consecutive channels of one token: rows x0..x3 (oldest first, 8 bf16 each), taps wt (4 bf16 per channel)
-__device__ __forceinline__ void conv8_silu_tab(const bf16_t* tab, const uint4& x0, const uint4& x1, const uint4& x2,
-                                               const uint4& x3, const uint4 (&wt)[4], float (&u)[8]) {
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// two floats rounded to bf16 (nearest even) by one v_cvt_pk_bf16_f32: a in the low half
+__device__ __forceinline__ uint32_t pack2_bf(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+// table index of both halves of a bf16 pair (packed 16-bit arithmetic): rotl16(x, 1) - 2 * (LO << 7), wrapping for small |x|
+__device__ __forceinline__ u16x2 silu_index2(uint32_t w) {
+    const u16x2 x = __builtin_bit_cast(u16x2, w);
+    return x * (unsigned short)2 + (x >> 15) - (unsigned short)(SILU_TAB_LO * 256);
+}
+// conv4 + silu of 8 consecutive channels of one token: rows x0..x3 (oldest first, 8 bf16 each), taps wt (4 bf16 per channel);
+// the results as four bf16 pairs (their values are what silu_bf16 returns).  An input outside the table reads the spare entry
+// and is re-evaluated in one unlikely block per 8 channels.
+__device__ __forceinline__ void conv8_silu_pairs(const bf16_t* tab, const uint4& x0, const uint4& x1, const uint4& x2,
+                                                 const uint4& x3, const uint4 (&wt)[4], uint32_t (&r)[4]) {
     float a[8], b[8], c[8], d[8];
     unpack8(x0, a);
     unpack8(x1, b);
     unpack8(x2, c);
     unpack8(x3, d);
-    bool rare = false;
+    float s[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         const uint4 ww = wt[e >> 1];
         const uint32_t c0 = (e & 1) ? ww.z : ww.x, c1 = (e & 1) ? ww.w : ww.y;
-        float s = a[e] * lo_bf(c0);
-        s = s + b[e] * hi_bf(c0);
-        s = s + c[e] * lo_bf(c1);
-        s = s + d[e] * hi_bf(c1);
-        u[e] = silu_lookup_fast(tab, f2bf(s), rare);
+        s[e] = a[e] * lo_bf(c0);
+        s[e] = s[e] + b[e] * hi_bf(c0);
+        s[e] = s[e] + c[e] * lo_bf(c1);
+        s[e] = s[e] + d[e] * hi_bf(c1);
     }
-    if (__builtin_expect(rare, 0)) {
+    uint32_t xb[4];
+    u16x2 worst = {0, 0};
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const uint4 ww = wt[e >> 1];
-            const uint32_t c0 = (e & 1) ? ww.z : ww.x, c1 = (e & 1) ? ww.w : ww.y;
-            float s = a[e] * lo_bf(c0);
-            s = s + b[e] * hi_bf(c0);
-            s = s + c[e] * lo_bf(c1);
-            s = s + d[e] * hi_bf(c1);
-            const bf16_t xb = f2bf(s);
-            if (((xb & 0x7fffu) - SILU_TAB_LO * 128) >= (unsigned)SILU_TAB_N) u[e] = silu_out_of_table(bf2f(xb));
+    for (int i = 0; i < 4; i++) {
+        xb[i] = pack2_bf(s[2 * i], s[2 * i + 1]);
+        const u16x2 idx = silu_index2(xb[i]);
+        worst = __builtin_elementwise_max(worst, idx);
+        const u16x2 off = __builtin_elementwise_min(idx, (u16x2){SILU_TAB_N2, SILU_TAB_N2}) << 1;     // byte offsets into the table
+        const char* tb = reinterpret_cast<const char*>(tab);
+        u16x2 v;
+        v.x = *reinterpret_cast<const bf16_t*>(tb + off.x);
+        v.y = *reinterpret_cast<const bf16_t*>(tb + off.y);
+        r[i] = __builtin_bit_cast(uint32_t, v);
+    }
+    if (__builtin_expect(max(worst.x, worst.y) >= SILU_TAB_N2, 0)) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const u16x2 idx = silu_index2(xb[i]);
+            if (idx.x >= SILU_TAB_N2) r[i] = (r[i] & 0xffff0000u) | f2bf(silu_out_of_table(lo_bf(xb[i])));
+            if (idx.y >= SILU_TAB_N2) r[i] = (r[i] & 0x0000ffffu) | ((uint32_t)f2bf(silu_out_of_table(hi_bf(xb[i]))) << 16);
         }
     }
 }
 
-// conv4 + silu of 8 channels of one token, packed as bf16 pairs (the values are bf16-exact), and their exact sum of squares
+// conv4 + silu of 8 channels of one token, packed as bf16 pairs, and their exact sum of squares
 __device__ __forceinline__ double conv8_silu_packed(const bf16_t* tab, const uint4& x0, const uint4& x1, const uint4& x2,
                                                     const uint4& x3, const uint4 (&wt)[4], uint4& packed) {
+    uint32_t r[4];
+    conv8_silu_pairs(tab, x0, x1, x2, x3, wt, r);
+    packed = make_uint4(r[0], r[1], r[2], r[3]);
     float u[8];
-    conv8_silu_tab(tab, x0, x1, x2, x3, wt, u);
+    unpack8(packed, u);
     double sq = 0.0;
 #pragma unroll
     for (int e = 0; e < 8; e++) sq += (double)u[e] * u[e];
-    packed = make_uint4(pack_bf(u[0], u[1]), pack_bf(u[2], u[3]), pack_bf(u[4], u[5]), pack_bf(u[6], u[7]));
     return sq;
 }
 // q/k normalization of 8 packed channels: BF(BF(u * r) * sc) (kernels.py:507-510)
 __device__ __forceinline__ uint4 scale8_packed(const uint4& u, float r, float sc) {
     float f[8];
     unpack8(u, f);
-    return make_uint4(pack_bf(BF(BF(f[0] * r) * sc), BF(BF(f[1] * r) * sc)), pack_bf(BF(BF(f[2] * r) * sc), BF(BF(f[3] * r) * sc)),
-                      pack_bf(BF(BF(f[4] * r) * sc), BF(BF(f[5] * r) * sc)), pack_bf(BF(BF(f[6] * r) * sc), BF(BF(f[7] * r) * sc)));
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t t = pack2_bf(f[2 * i] * r, f[2 * i + 1] * r);
+        o[i] = pack2_bf(lo_bf(t) * sc, hi_bf(t) * sc);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 constexpr float INV_SCALE = 0.08838834764831845f;                                // 128^-0.5, kernels.py:490
