@@ -462,7 +462,8 @@ __global__ __launch_bounds__(512) void gdn_phase_b_kernel(const _Float16* ops, c
 // A (chunk, head) costs about 10^5 vector-ALU instructions of conv + SiLU + normalisation and a chain of dependent matrix
 // steps (K K^T, the 64 x 64 triangular inverse, the products with it) that keeps no unit busy.  The two run side by side:
 // wavefronts 0..3 (group M) convolve k, then walk the matrix chain while wavefronts 4..7 (group V) convolve q and v and
-// form A = lower(G * Q K^T).  Three workgroup barriers: table and taps ready; k and q staged; v staged.
+// form A = lower(G * Q K^T).  One workgroup barrier (table, taps and gates ready); after it a consumer of k, q or v waits for
+// that part's four producers through a counter in LDS.
 //
 // q, k and v are converted to half precision ONCE, when they are staged into LDS, and every MFMA operand is then a plain
 // LDS read: row-major 16-byte reads for K K^T and Q K^T, the transposing load ds_read_b64_tr_b16 where the contraction runs
@@ -492,10 +493,24 @@ struct PhaseALds {                       // 76.6 KiB: two workgroups per CU
     __align__(16) _Float16 Vs[C * VS_LD];
     __align__(16) bf16_t tab[SILU_TAB_SIZE];     // fused conv only: the silu_bf16 table and this head's conv taps
     __align__(16) bf16_t taps[3 * DK * 4];
-    __align__(16) float Nd[4 * ND_BLK];          // diagonal blocks of L: [block][row][column]
-    __align__(16) float Td[4 * ND_BLK];          // their inverses, transposed: [block][column][row]
+    __align__(16) float Nd[4 * ND_BLK];          // diagonal blocks of L: [block][column][row]
+    __align__(16) float Td[4 * ND_BLK];          // their inverses: [block][column][row]
     float Lc2[C], beta[C], gam[C], dec[C];       // Lc2 = log2(e) * cumsum(log g)
+    int staged[4];                               // wavefronts that have staged their part of k, q, v (PA_K, PA_Q, PA_V)
 };
+constexpr int PA_K = 0, PA_Q = 1, PA_V = 2;
+
+// A wavefront announces that its LDS stores of a part are done; a consumer waits until all four producers have.  (The parts
+// are produced and consumed by different wavefronts at different times: a workgroup barrier would hold up seven wavefronts
+// for the slowest one three times per chunk.)
+__device__ __forceinline__ void part_staged(PhaseALds& L, int part, int lane) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if (lane == 0) __hip_atomic_fetch_add(&L.staged[part], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void await_part(PhaseALds& L, int part) {
+    while (__hip_atomic_load(&L.staged[part], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < 4) __builtin_amdgcn_s_sleep(1);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
 
 __device__ __forceinline__ half8 to_half8(const float (&v)[8]) {
     half8 h;
@@ -537,10 +552,10 @@ __device__ __forceinline__ f32x4 kk_block(const _Float16* Ks, int I, int J, int 
     return acc;
 }
 
-// The matrix chain of block row I (one wavefront of group M): returns Tb = T diag(beta) for rows 16 I + n as the two operand
-// forms of the products, tbU[kb2] = Tb[16 I + n][kperm(kb2, g, 0..7)] and tbW = the same with columns scaled by -gamma.
-template <int I>
-__device__ __forceinline__ void inverse_row(PhaseALds& L, int n, int g, half8 (&tbU)[2], half8 (&tbW)[2]) {
+// The matrix chain of block row I (one wavefront of group M; I is the same for the whole wavefront, so every test of it is a
+// scalar branch): returns Tb = T diag(beta) for rows 16 I + n as the two operand forms of the products,
+// tbU[kb2] = Tb[16 I + n][kperm(kb2, g, 0..7)] and tbW = the same with columns scaled by -gamma.
+__device__ __forceinline__ void inverse_row(PhaseALds& L, const int I, int n, int g, half8 (&tbU)[2], half8 (&tbW)[2]) {
     // diagonal blocks of L -> LDS (all four, in every wavefront)
 #pragma unroll
     for (int b = 0; b < 4; b++) {
@@ -548,63 +563,85 @@ __device__ __forceinline__ void inverse_row(PhaseALds& L, int n, int g, half8 (&
         const f32x4 lci = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * b + 4 * g]);
         const f32x4 bei = *reinterpret_cast<const f32x4*>(&L.beta[16 * b + 4 * g]);
         const float lcj = L.Lc2[16 * b + n];
+        f32x4 nd;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const float v = bei[r] * __builtin_amdgcn_exp2f(lci[r] - lcj) * acc[r];
-            L.Nd[b * ND_BLK + (4 * g + r) * ND_LD + n] = (4 * g + r > n) ? v : 0.f;
+            nd[r] = (4 * g + r > n) ? v : 0.f;
         }
+        *reinterpret_cast<f32x4*>(&L.Nd[b * ND_BLK + n * ND_LD + 4 * g]) = nd;
     }
-    // lane (n, g): column n of the inverse of diagonal block g, by forward substitution
+    // lane (n, g): column n of the inverse of diagonal block g, by forward substitution.  Column by column: once x[m] is known
+    // every later row takes its term, so one multiply-add per step is on the dependent path (the terms of a row are still
+    // added in ascending m).  The multiply-adds are written as fused ones: both input forms of the kernel then round alike.
     {
-        float x[16];
+        float a[16];
         const float* nb = &L.Nd[g * ND_BLK];
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            float a = (i == n) ? 1.f : 0.f;
+        for (int i = 0; i < 16; i++) a[i] = (i == n) ? 1.f : 0.f;
 #pragma unroll
-            for (int m = 0; m < i; m++) a -= nb[i * ND_LD + m] * x[m];
-            x[i] = a;
+        for (int m = 0; m < 15; m++) {
+            float col[16];
+#pragma unroll
+            for (int i4 = (m + 1) & ~3; i4 < 16; i4 += 4) {
+                const f32x4 v4 = *reinterpret_cast<const f32x4*>(nb + m * ND_LD + i4);
+                col[i4] = v4[0]; col[i4 + 1] = v4[1]; col[i4 + 2] = v4[2]; col[i4 + 3] = v4[3];
+            }
+#pragma unroll
+            for (int i = m + 1; i < 16; i++) a[i] = __builtin_fmaf(-col[i], a[m], a[i]);
+            if ((m & 3) == 3) __builtin_amdgcn_sched_barrier(0);     // at most four columns' worth of reads ahead
         }
         float* tb = &L.Td[g * ND_BLK + n * ND_LD];
 #pragma unroll
-        for (int i = 0; i < 16; i += 4) *reinterpret_cast<f32x4*>(tb + i) = f32x4{x[i], x[i + 1], x[i + 2], x[i + 3]};
+        for (int i = 0; i < 16; i += 4) *reinterpret_cast<f32x4*>(tb + i) = f32x4{a[i], a[i + 1], a[i + 2], a[i + 3]};
     }
-    __builtin_amdgcn_sched_barrier(0);                   // the substitution's sixteen values are dead before the blocks below are formed
-    // blocks of L below the diagonal that this row's recursion multiplies with: LB[J][w] = block (J, w), w < J <= I
-    f32x4 LB[4][4];
+    __builtin_amdgcn_sched_barrier(0);
+    // blocks of L below the diagonal that this row's recursion multiplies with: LB[J (J - 1) / 2 + w] = block (J, w), w < J <= I
+    f32x4 LB[6];
 #pragma unroll
-    for (int J = 1; J <= I; J++) {
-        const f32x4 lci = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * J + 4 * g]);
-        const f32x4 bei = *reinterpret_cast<const f32x4*>(&L.beta[16 * J + 4 * g]);
+    for (int J = 1; J < 4; J++) {
+        if (J <= I) {
+            const f32x4 lci = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * J + 4 * g]);
+            const f32x4 bei = *reinterpret_cast<const f32x4*>(&L.beta[16 * J + 4 * g]);
 #pragma unroll
-        for (int w = 0; w < J; w++) {
-            // (a zero offset passes through an empty asm: otherwise the rows of all four blocks stay in registers, 64 of the 128)
-            int zero = 0;
-            asm volatile("" : "+v"(zero));
-            const f32x4 acc = kk_block(L.Ks + zero, J, w, n, g);
-            const float lcj = L.Lc2[16 * w + n];
+            for (int w = 0; w < J; w++) {
+                const f32x4 acc = kk_block(L.Ks, J, w, n, g);
+                const float lcj = L.Lc2[16 * w + n];
 #pragma unroll
-            for (int r = 0; r < 4; r++) LB[J][w][r] = bei[r] * __builtin_amdgcn_exp2f(lci[r] - lcj) * acc[r];
+                for (int r = 0; r < 4; r++) LB[J * (J - 1) / 2 + w][r] = bei[r] * __builtin_amdgcn_exp2f(lci[r] - lcj) * acc[r];
+            }
         }
     }
     // column I of TT, upwards
     f32x4 TT[4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) TT[I][r] = L.Td[I * ND_BLK + (4 * g + r) * ND_LD + n];          // T_II[n][4 g + r]
+    for (int k = 0; k < 4; k++) {
+        TT[k] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (k == I) {
 #pragma unroll
-    for (int w = I - 1; w >= 0; w--) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int J = w + 1; J <= I; J++)
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(LB[J][w][kk], TT[J][kk], acc, 0, 0, 0);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&L.Td[w * ND_BLK + n * ND_LD + 4 * g]);   // T_ww[4 g + kk][n]
-        f32x4 res = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++) res = __builtin_amdgcn_mfma_f32_16x16x4f32(d4[kk], acc[kk], res, 0, 0, 0);
-        TT[w] = -res;
+            for (int r = 0; r < 4; r++) TT[k][r] = L.Td[k * ND_BLK + (4 * g + r) * ND_LD + n];     // T_II[n][4 g + r]
+        }
     }
-    // TT[w][r] = T[16 I + n][16 w + 4 g + r]
+#pragma unroll
+    for (int w = 2; w >= 0; w--) {
+        if (w < I) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int J = 3; J > w; J--) {                                // the block found last, TT[w + 1], enters last
+                if (J <= I) {
+#pragma unroll
+                    for (int kk = 0; kk < 4; kk++)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(LB[J * (J - 1) / 2 + w][kk], TT[J][kk], acc, 0, 0, 0);
+                }
+            }
+            const f32x4 d4 = *reinterpret_cast<const f32x4*>(&L.Td[w * ND_BLK + n * ND_LD + 4 * g]);   // T_ww[4 g + kk][n]
+            f32x4 res = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) res = __builtin_amdgcn_mfma_f32_16x16x4f32(d4[kk], acc[kk], res, 0, 0, 0);
+            TT[w] = -res;
+        }
+    }
+    // TT[w][r] = T[16 I + n][16 w + 4 g + r] (zero for w > I)
 #pragma unroll
     for (int kb2 = 0; kb2 < 2; kb2++) {
         float u[8], v[8];
@@ -615,8 +652,7 @@ __device__ __forceinline__ void inverse_row(PhaseALds& L, int n, int g, half8 (&
             const f32x4 g4 = *reinterpret_cast<const f32x4*>(&L.gam[cp]);
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const float t = (blk <= I) ? TT[blk <= I ? blk : 0][r] : 0.f;                   // blk is a constant after unrolling
-                u[4 * hf + r] = t * b4[r];
+                u[4 * hf + r] = TT[blk][r] * b4[r];
                 v[4 * hf + r] = -u[4 * hf + r] * g4[r];
             }
         }
@@ -629,10 +665,11 @@ __device__ __forceinline__ void inverse_row(PhaseALds& L, int n, int g, half8 (&
 // outputs).  from_proj = true: they are computed here from the projection rows (conv4 + SiLU + q/k norm with the arithmetic of
 // conv_prep_kernel, bit for bit; qwen35/prefill.py:96-134) and, with write_qkv, also stored; the workgroups of the last chunk
 // write the new conv window (the last three input rows, prefill.py:262-263) to conv_out if it is given.
-// proj [S,8224] supplies the gate inputs a, b in both forms.  The two forms are ONE kernel with uniform branches, not two
-// template instances: everything after the staging of q, k, v is then the same machine code, so both forms give the same bits
-// (two instances are scheduled and contracted independently by the compiler and differed in the last place now and then).
-__global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_proj, const bool write_qkv,
+// proj [S,8224] supplies the gate inputs a, b in both forms.  The two forms give the same bits: after the staging of q, k, v
+// every floating-point step is a single instruction chosen in the source (MFMA, multiplication, fused multiply-add), so the
+// compiler has nothing to contract differently in the two instances.
+template <bool from_proj>
+__global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool write_qkv,
                                                           const bf16_t* __restrict__ proj, bf16_t* qi, bf16_t* ki, bf16_t* vi,
                                                           const bf16_t* __restrict__ cs, const bf16_t* __restrict__ cw,
                                                           const bf16_t* __restrict__ silu_tab, bf16_t* __restrict__ conv_out,
@@ -656,14 +693,19 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
     // one register array per part for both forms.  !from_proj: rw[rr] = token rr * 16 + gi, a lane 8 consecutive columns;
     // from_proj: rw[d] = input row 4 gi - 3 + d of 8 channels of the part
     uint4 rwA[7], rwB[7];
+    // (wavefront 0 asks for its gate inputs first: loads return in order, so the gates are computed while the rows are in flight)
+    bf16_t ga_raw = 0, gb_raw = 0;
+    if (wv == 0 && t0 + lane < S) {
+        ga_raw = proj[(size_t)(t0 + lane) * PW + CD + KD + HV + h];
+        gb_raw = proj[(size_t)(t0 + lane) * PW + CD + KD + h];
+    }
     if (!from_proj) {
 #pragma unroll
         for (int rr = 0; rr < 4; rr++) {
             const int t = t0 + rr * 16 + gi;
             const size_t o = ((size_t)min(t, S - 1) * HV + h) * DK + cc * 8;
             rwA[rr] = *reinterpret_cast<const uint4*>(outA + o);
-            if (grpV) rwB[rr] = *reinterpret_cast<const uint4*>(vi + o);
-            if (t >= S) rwA[rr] = rwB[rr] = make_uint4(0, 0, 0, 0);
+            if (t >= S) rwA[rr] = make_uint4(0, 0, 0, 0);
         }
     } else {
         const int chA = partA * KD + h * DK + cc * 8;
@@ -690,8 +732,8 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
         const int t = t0 + lane;
         float lg = 0.f, be = 0.f;
         if (t < S) {
-            lg = log_decay(A_log[h], BF(bf2f(proj[(size_t)t * PW + CD + KD + HV + h]) + dt_bias[h]));
-            be = sigmoid_bf16(bf2f(proj[(size_t)t * PW + CD + KD + h]));
+            lg = log_decay(A_log[h], BF(bf2f(ga_raw) + dt_bias[h]));
+            be = sigmoid_bf16(bf2f(gb_raw));
         }
         float lc = lg;
 #pragma unroll
@@ -718,6 +760,7 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
         if (lane >= 60) gp[G_GC + lane - 60] = lane == 60 ? expf(tot) : 0.f;
     }
     if (from_proj) silu_table_fill(L.tab, silu_tab, tid, 512);
+    if (tid >= 508) L.staged[tid - 508] = 0;
     __syncthreads();
 
     // ---- k (group M) and q (group V): conv + SiLU + L2 norm, staged as half precision
@@ -726,6 +769,14 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
         if (!from_proj) {
 #pragma unroll
             for (int rr = 0; rr < 4; rr++) *reinterpret_cast<half8*>(&dst[(rr * 16 + gi) * QS_LD + cc * 8]) = bf8_to_half8(rwA[rr]);
+            if (grpV) {
+#pragma unroll
+                for (int rr = 0; rr < 4; rr++) {
+                    const int t = t0 + rr * 16 + gi;
+                    rwB[rr] = *reinterpret_cast<const uint4*>(vi + ((size_t)min(t, S - 1) * HV + h) * DK + cc * 8);
+                    if (t >= S) rwB[rr] = make_uint4(0, 0, 0, 0);
+                }
+            }
         } else {
             const float sc = grpV ? BF(INV_SCALE * INV_SCALE) : BF(INV_SCALE);
             uint4 wt[4], pk[4];
@@ -734,6 +785,7 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
             for (int e = 0; e < 4; e++) wt[e] = *reinterpret_cast<const uint4*>(&L.taps[(partA * DK + cc * 8 + 2 * e) * 4]);
 #pragma unroll
             for (int j = 0; j < 4; j++) ss[j] = (float)row16_sum_d(conv8_silu_packed(L.tab, rwA[j], rwA[j + 1], rwA[j + 2], rwA[j + 3], wt, pk[j]));
+            __builtin_amdgcn_sched_barrier(0);           // (the loads below must not be moved up: there is no room for them before)
             if (grpV) {                                  // v's rows: requested once q's are consumed (the register file holds one set)
                 const int chB = 2 * KD + h * DK + cc * 8;
 #pragma unroll
@@ -753,7 +805,7 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
             }
         }
     }
-    __syncthreads();
+    part_staged(L, grpV ? PA_Q : PA_K, lane);
 
     if (grpV) {
         // ---- v: conv + SiLU, staged
@@ -774,7 +826,9 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
                 *reinterpret_cast<half8*>(&L.Vs[tl * VS_LD + cc * 8]) = bf8_to_half8(p);
             }
         }
-        __syncthreads();
+        part_staged(L, PA_V, lane);
+        await_part(L, PA_Q);
+        await_part(L, PA_K);
         // ---- Am = lower_incl(G * Q K^T) transposed, rows c_out = 16 ct + n, k = c_in (permuted); G_ij = exp2(Lc2_i - Lc2_j)
         const int ct = w, co = 16 * ct + n;
         const float lco = L.Lc2[co];
@@ -810,26 +864,16 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
             qh[4] = hi[0]; qh[5] = hi[1]; qh[6] = hi[2]; qh[7] = hi[3];
             *reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8) = qh;
         }
-        // Kh = K^T (rows dk of tiles 2w, 2w+1), k index permuted
-        for (int mm = 0; mm < 2; mm++) {
-            const int mt = 2 * w + mm;
-            for (int kb2 = 0; kb2 < 2; kb2++)
-                *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g);
-        }
         return;
     }
 
     // ---- group M: T = (I + L)^-1 by block rows, then Wn^T = K^T (-Tb gamma)^T and U = Tb V on fp16 MFMA; wavefront w owns the
     // chunk rows of tile ct = w.  Both Tb operands hold Tb[16 ct + n][kperm(kb2, g, 0..7)]: as the A operand of U, and (columns
     // scaled by -gamma) as the B operand of Wn^T.
+    await_part(L, PA_K);
     __builtin_amdgcn_s_setprio(2);                       // few instructions, all of them on the critical path
     half8 tbU[2], tbW[2];
-    switch (w) {
-        case 0: inverse_row<0>(L, n, g, tbU, tbW); break;
-        case 1: inverse_row<1>(L, n, g, tbU, tbW); break;
-        case 2: inverse_row<2>(L, n, g, tbU, tbW); break;
-        default: inverse_row<3>(L, n, g, tbU, tbW); break;
-    }
+    inverse_row(L, w, n, g, tbU, tbW);
     const int ct = w, nkb = ct < 2 ? 1 : 2;              // Tb is lower triangular: columns past the row tile are zero
     for (int kb = 0; kb < 4; kb++) {
         f32x4 acc[2];
@@ -845,7 +889,14 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool from_pro
         }
         *reinterpret_cast<half8*>(op + OP_W + (ct * 4 + kb) * 512 + lane * 8) = pack_half8(acc[0], acc[1]);
     }
-    __syncthreads();                                     // v is staged
+    // Kh = K^T (rows dk of tiles 2w, 2w+1), k index permuted
+    for (int mm = 0; mm < 2; mm++) {
+        const int mt = 2 * w + mm;
+        for (int kb2 = 0; kb2 < 2; kb2++)
+            *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g);
+    }
+    __builtin_amdgcn_s_setprio(0);
+    await_part(L, PA_V);
     _Float16* up = U + rec * U_HALVES;
     for (int sl = 0; sl < 8; sl++) {
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -928,7 +979,7 @@ int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v
     for (const void* p : {proj, q, k, v, (const void*)ops, (const void*)U, (const void*)gC})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     const int NC = (S + C - 1) / C;
-    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(512), 0, stream, false, false, (const bf16_t*)proj, (bf16_t*)q,
+    hipLaunchKernelGGL(gdn_phase_a_kernel<false>, dim3(NC * HV), dim3(512), 0, stream, false, (const bf16_t*)proj, (bf16_t*)q,
                        (bf16_t*)k, (bf16_t*)v, (const bf16_t*)nullptr, (const bf16_t*)nullptr, (const bf16_t*)nullptr,
                        (bf16_t*)nullptr, A_log, dt_bias, (_Float16*)ops, (_Float16*)U, gC, S);
     QT_CHECK_LAUNCH();
@@ -947,7 +998,7 @@ int qt_gdn_phase_a_conv(const void* proj, const void* conv_state, const void* co
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     if (conv_out == conv_state) return QT_ERR_UNSUPPORTED;          // the old window is still being read when the new one is written
     const int NC = (S + C - 1) / C;
-    hipLaunchKernelGGL(gdn_phase_a_kernel, dim3(NC * HV), dim3(512), 0, stream, true, q != nullptr, (const bf16_t*)proj, (bf16_t*)q,
+    hipLaunchKernelGGL(gdn_phase_a_kernel<true>, dim3(NC * HV), dim3(512), 0, stream, q != nullptr, (const bf16_t*)proj, (bf16_t*)q,
                        (bf16_t*)k, (bf16_t*)v, (const bf16_t*)conv_state, (const bf16_t*)conv_w, (const bf16_t*)silu_table,
                        (bf16_t*)conv_out, A_log, dt_bias, (_Float16*)ops, (_Float16*)U, gC, S);
     QT_CHECK_LAUNCH();
