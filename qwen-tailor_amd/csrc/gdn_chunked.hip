@@ -487,13 +487,12 @@ constexpr int ND_LD = 20;            // row stride (floats) of a diagonal block
 constexpr int ND_BLK = 16 * ND_LD + 4;   // floats between diagonal blocks: the four lane groups read distinct banks
 constexpr float LOG2E = 1.4426950408889634f;
 
-struct PhaseALds {                       // 76.6 KiB: two workgroups per CU
+struct PhaseALds {                       // 73 KiB: two workgroups per CU
     __align__(16) _Float16 Ks[C * QS_LD];
     __align__(16) _Float16 Qs[C * QS_LD];
     __align__(16) _Float16 Vs[C * VS_LD];
     __align__(16) bf16_t tab[SILU_TAB_SIZE];     // fused conv only: the silu_bf16 table and this head's conv taps
     __align__(16) bf16_t taps[3 * DK * 4];
-    __align__(16) float Nd[4 * ND_BLK];          // diagonal blocks of L: [block][column][row]
     __align__(16) float Td[4 * ND_BLK];          // their inverses: [block][column][row]
     float Lc2[C], beta[C], gam[C], dec[C];       // Lc2 = log2(e) * cumsum(log g)
     int staged[4];                               // wavefronts that have staged their part of k, q, v (PA_K, PA_Q, PA_V)
@@ -552,45 +551,64 @@ __device__ __forceinline__ f32x4 kk_block(const _Float16* Ks, int I, int J, int 
     return acc;
 }
 
+// v_permlane32_swap: lanes 32..63 of x change places with lanes 0..31 of y; v_permlane16_swap: the odd 16-lane rows of x with
+// the even rows of y
+__device__ __forceinline__ void lanes32_swap(float& x, float& y) {
+    const auto t = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+    x = __uint_as_float(t[0]);
+    y = __uint_as_float(t[1]);
+}
+__device__ __forceinline__ void lanes16_swap(float& x, float& y) {
+    const auto t = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(y), false, false);
+    x = __uint_as_float(t[0]);
+    y = __uint_as_float(t[1]);
+}
+// steps M.. of the forward substitution: a[i] += (lane M's R value of row i) * a[M] for every row i > M
+template <int M>
+__device__ __forceinline__ void substitute_columns(const float (&R)[4][4], float (&a)[16]) {
+    if constexpr (M < 15) {
+#pragma unroll
+        for (int i = M + 1; i < 16; i++) a[i] = __builtin_fmaf(row16_bcast<M>(R[i >> 2][i & 3]), a[M], a[i]);
+        substitute_columns<M + 1>(R, a);
+    }
+}
+
 // The matrix chain of block row I (one wavefront of group M; I is the same for the whole wavefront, so every test of it is a
 // scalar branch): returns Tb = T diag(beta) for rows 16 I + n as the two operand forms of the products,
 // tbU[kb2] = Tb[16 I + n][kperm(kb2, g, 0..7)] and tbW = the same with columns scaled by -gamma.
 __device__ __forceinline__ void inverse_row(PhaseALds& L, const int I, int n, int g, half8 (&tbU)[2], half8 (&tbW)[2]) {
-    // diagonal blocks of L -> LDS (all four, in every wavefront)
+    // diagonal blocks of L, negated (all four, in every wavefront): R[b][r] = -L[16 b + 4 g + r][16 b + n]
+    float R[4][4];
 #pragma unroll
     for (int b = 0; b < 4; b++) {
         const f32x4 acc = kk_block(L.Ks, b, b, n, g);
         const f32x4 lci = *reinterpret_cast<const f32x4*>(&L.Lc2[16 * b + 4 * g]);
         const f32x4 bei = *reinterpret_cast<const f32x4*>(&L.beta[16 * b + 4 * g]);
         const float lcj = L.Lc2[16 * b + n];
-        f32x4 nd;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const float v = bei[r] * __builtin_amdgcn_exp2f(lci[r] - lcj) * acc[r];
-            nd[r] = (4 * g + r > n) ? v : 0.f;
+            R[b][r] = (4 * g + r > n) ? -v : 0.f;
         }
-        *reinterpret_cast<f32x4*>(&L.Nd[b * ND_BLK + n * ND_LD + 4 * g]) = nd;
     }
-    // lane (n, g): column n of the inverse of diagonal block g, by forward substitution.  Column by column: once x[m] is known
-    // every later row takes its term, so one multiply-add per step is on the dependent path (the terms of a row are still
-    // added in ascending m).  The multiply-adds are written as fused ones: both input forms of the kernel then round alike.
+    // 4 x 4 transpose over (register b, lane group g) with the VALU lane swaps: afterwards lane (n, g) holds column n of its own
+    // block g, R[j][r] = -L[16 g + 4 j + r][16 g + n]
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        lanes32_swap(R[0][r], R[2][r]);
+        lanes32_swap(R[1][r], R[3][r]);
+        lanes16_swap(R[0][r], R[1][r]);
+        lanes16_swap(R[2][r], R[3][r]);
+    }
+    // lane (n, g): column n of the inverse of diagonal block g, by forward substitution in registers.  Column by column: once
+    // x[m] is known every later row takes its term -L[i][m] x[m] (the factor is lane m's value, broadcast over the 16 lanes),
+    // so one multiply-add per step is on the dependent path; the terms of a row are still added in ascending m.  The
+    // multiply-adds are written as fused ones: both input forms of the kernel then round alike.
     {
         float a[16];
-        const float* nb = &L.Nd[g * ND_BLK];
 #pragma unroll
         for (int i = 0; i < 16; i++) a[i] = (i == n) ? 1.f : 0.f;
-#pragma unroll
-        for (int m = 0; m < 15; m++) {
-            float col[16];
-#pragma unroll
-            for (int i4 = (m + 1) & ~3; i4 < 16; i4 += 4) {
-                const f32x4 v4 = *reinterpret_cast<const f32x4*>(nb + m * ND_LD + i4);
-                col[i4] = v4[0]; col[i4 + 1] = v4[1]; col[i4 + 2] = v4[2]; col[i4 + 3] = v4[3];
-            }
-#pragma unroll
-            for (int i = m + 1; i < 16; i++) a[i] = __builtin_fmaf(-col[i], a[m], a[i]);
-            if ((m & 3) == 3) __builtin_amdgcn_sched_barrier(0);     // at most four columns' worth of reads ahead
-        }
+        substitute_columns<0>(R, a);
         float* tb = &L.Td[g * ND_BLK + n * ND_LD];
 #pragma unroll
         for (int i = 0; i < 16; i += 4) *reinterpret_cast<f32x4*>(tb + i) = f32x4{a[i], a[i + 1], a[i + 2], a[i + 3]};
