@@ -72,20 +72,21 @@ __device__ __forceinline__ half8 pack_half8(const f32x4& a, const f32x4& b) {
 // its rows of D (scaled by dec for the update, and plain for the outputs) and reads both k-blocks (barrier E2).  The fifth
 // wavefront copies S^T and the plain D from LDS to `snap`: the MFMA wavefronts issue loads only, which keeps their vmcnt
 // waits partial (a store in flight next to loads forces every wait to zero on this target).
-constexpr int PB_DEP = 4;                        // chunks of operands in flight per MFMA wavefront
 constexpr int SNAP_S = 4 * 512;                  // halves: S^T as B operand, [kb 4][lane 64][8]
 constexpr int SNAP_D = 2 * 512;                  // halves: D as B operand, [kb2 2][lane 64][8]
 constexpr int SNAP_HALVES = SNAP_S + SNAP_D;     // 6 KiB per (chunk, head, slice)
 constexpr int KORD[4] = {0, 2, 1, 3};            // order in which a step consumes its Kh tiles (two independent accumulators)
 constexpr int N_CHAIN = HV * 8;                  // chain workgroups
+constexpr int PF_AHEAD = 10;                     // chunks between the L2 prefetch and the chain
+constexpr int PF_SLOTS = 8;                      // prefetch loads in flight
 constexpr int PUB_LAG = 8;                       // a chunk is published when at most this many newer chunks' stores are in flight
 constexpr int FLAG_STRIDE = 64;                  // ints between progress words: every word has a 256-byte stretch of its own
 constexpr int FLAG_WORDS = (N_CHAIN + 1) * FLAG_STRIDE;   // flag area at the head of `snap` (33 KiB): progress [128] | done count, error
-constexpr int FLAG_DONE = N_CHAIN * FLAG_STRIDE, FLAG_ERR = FLAG_DONE + 1;
+constexpr int FLAG_DONE = N_CHAIN * FLAG_STRIDE, FLAG_ERR = FLAG_DONE + 1, FLAG_NEXT = FLAG_DONE + 2;   // FLAG_NEXT: head of the item queue
 constexpr int FLAG_HALVES = FLAG_WORDS * 2;
 constexpr int SPIN_LIMIT = 1 << 21;              // polls (about a second) before a consumer gives up
-constexpr int UNITS_PER_HEAD = 16;               // output units (half workgroups) per head: unit r takes chunks r, r + 16, ...
-constexpr int FUSED_MIN_CHUNKS = 64;             // from 4096 tokens on the one-launch form wins (measured: 2048 tokens 37 / 35 us, 8192 134 / 155 us)
+constexpr int MAX_OUT_WGS = 256;                 // output workgroups of the one-launch form: what fits beside the chain workgroups
+constexpr int FUSED_MIN_CHUNKS = 64;              // from 4096 tokens on the one-launch form wins (measured: 2048 tokens 37 / 35 us, 8192 134 / 155 us)
 typedef unsigned long long u64;
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -121,13 +122,16 @@ struct ChainLds {
 };
 
 // blk = (head, slice) index of this workgroup; wavefronts 0..3 compute, wavefront 4 writes snapshots and publishes progress
-template <bool PUBLISH>
+// PB_DEP = chunks of operands in flight per MFMA wavefront (4 in the two-launch form; 3 in the one-launch form, whose
+// wavefronts share their SIMDs with output wavefronts and have 168 registers each)
+template <bool PUBLISH, int PB_DEP>
 __device__ __forceinline__ void chain_role(ChainLds& L, int blk, const _Float16* ops, const _Float16* U, const float* gates,
                                            const float* st_in, float* st_out, _Float16* snaps, int* flags, int NC) {
     // heads that share an XCD's L2 keep their 8 slices there: workgroup id = xcd + 8 k, head = xcd + 8 (k / 8), slice = k % 8
     const int xcd = blk & 7, kq = blk >> 3;
     const int h = xcd + 8 * (kq >> 3), sl = kq & 7;
-    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    // (the wavefront number as a scalar: the roles are then separated by real branches, which the barriers inside them need)
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const half8* sbx = reinterpret_cast<const half8*>(L.sb_x) + lane;
     const half8* dbx = reinterpret_cast<const half8*>(L.db_x) + lane;
     const half8* dnx = reinterpret_cast<const half8*>(L.dn_x) + lane;
@@ -163,7 +167,42 @@ __device__ __forceinline__ void chain_role(ChainLds& L, int blk, const _Float16*
         }
         return;
     }
-    if (w > 4) return;
+    if (w == 5) {
+        // sixth wavefront: brings the operands of chunk c + PF_AHEAD into this XCD's L2 (this slice's eighth of the head's Wn
+        // and Kh tiles, and its own U tiles: 48 lines of 128 bytes, one load per step, never waited for).  The operand FIFO
+        // of the MFMA wavefronts covers a few steps; a load that goes to HBM while other workgroups stream takes longer.
+        const char* wk = reinterpret_cast<const char*>(ops + (size_t)h * OP_HALVES);
+        const char* up = reinterpret_cast<const char*>(U + (size_t)h * U_HALVES + (size_t)sl * NCT * 256);
+        const size_t ostb = (size_t)HV * OP_HALVES * 2, ustb = (size_t)HV * U_HALVES * 2;
+        // lanes 0..15: lines sl * 16 .. + 15 of the 128 lines of Wn; 16..31: the same of Kh; 32..47: the 16 lines of the U slice
+        const int part = lane >> 4, li = lane & 15;
+        const size_t off = part == 0 ? (size_t)OP_W * 2 + (sl * 16 + li) * 128 : (size_t)OP_K * 2 + (sl * 16 + li) * 128;
+        // PF_SLOTS loads in flight, each into a register of its own that is read (an empty asm) before it is loaded again, one
+        // round later: the compiler counts the loads, and the wait it puts before that read names a load of many steps ago
+        unsigned pf[PF_SLOTS];
+#pragma unroll
+        for (int j = 0; j < PF_SLOTS; j++) pf[j] = 0;
+        for (int c0 = 0; c0 < NC; c0 += PF_SLOTS) {
+#pragma unroll
+            for (int j = 0; j < PF_SLOTS; j++) {
+                const int c = c0 + j;
+                if (c < NC) {                                                   // uniform: every wavefront meets 2 NC barriers
+                    __builtin_amdgcn_s_barrier();
+                    const int cp = c + PF_AHEAD;
+                    asm volatile("" ::"v"(pf[j]));
+                    if (cp < NC && lane < 48) {
+                        const char* a = part < 2 ? wk + cp * ostb + off : up + cp * ustb + li * 128;
+                        pf[j] = *reinterpret_cast<const unsigned*>(a);
+                    }
+                    __builtin_amdgcn_s_barrier();
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < PF_SLOTS; j++) asm volatile("" ::"v"(pf[j]));
+        return;
+    }
+    if (w > 5) return;
 
     f32x4 ST[2];
     {
@@ -260,41 +299,90 @@ __device__ __forceinline__ void chain_role(ChainLds& L, int blk, const _Float16*
         __builtin_amdgcn_sched_barrier(0);
     };
     int c = 0;
-    for (; c + PB_DEP <= NC; c += PB_DEP) {
-        step(std::integral_constant<int, 0>{}, c);
-        step(std::integral_constant<int, 1>{}, c + 1);
-        step(std::integral_constant<int, 2>{}, c + 2);
-        step(std::integral_constant<int, 3>{}, c + 3);
+    if constexpr (PB_DEP == 4) {
+        for (; c + 4 <= NC; c += 4) {
+            step(std::integral_constant<int, 0>{}, c);
+            step(std::integral_constant<int, 1>{}, c + 1);
+            step(std::integral_constant<int, 2>{}, c + 2);
+            step(std::integral_constant<int, 3>{}, c + 3);
+        }
+        if (c < NC) step(std::integral_constant<int, 0>{}, c);
+        if (c + 1 < NC) step(std::integral_constant<int, 1>{}, c + 1);
+        if (c + 2 < NC) step(std::integral_constant<int, 2>{}, c + 2);
+    } else {
+        static_assert(PB_DEP == 3 || PB_DEP == 4, "the chain loop is unrolled by hand");
+        for (; c + 3 <= NC; c += 3) {
+            step(std::integral_constant<int, 0>{}, c);
+            step(std::integral_constant<int, 1>{}, c + 1);
+            step(std::integral_constant<int, 2>{}, c + 2);
+        }
+        if (c < NC) step(std::integral_constant<int, 0>{}, c);
+        if (c + 1 < NC) step(std::integral_constant<int, 1>{}, c + 1);
     }
-    if (c < NC) step(std::integral_constant<int, 0>{}, c);
-    if (c + 1 < NC) step(std::integral_constant<int, 1>{}, c + 1);
-    if (c + 2 < NC) step(std::integral_constant<int, 2>{}, c + 2);
     {
         float* sp = st_out + ((size_t)h * DV + sl * 16 + n) * DK + w * 32 + 4 * g;
         *reinterpret_cast<f32x4*>(sp) = ST[0];
         *reinterpret_cast<f32x4*>(sp + 16) = ST[1];
     }
 }
-static_assert(PB_DEP == 4, "the chain loop is unrolled by hand for four FIFO entries");
 
-// Output role: Y_c = gamma_c * (Qh_c S_c^T) + Am_c D_c for one (chunk, head) at a time per unit of 4 wavefronts (a workgroup
-// holds two units); wavefront w of the unit covers the dv slices 2w and 2w+1.  The 64 x 128 tile goes through LDS as bf16 and
-// leaves either as y [S,16,128] or, with NORM, straight through the gated RMSNorm (same arithmetic as the stand-alone kernel:
-// 16 lanes per row, 8 columns each; batch.py:338-343).  Both units of a workgroup run the same number of rounds, so that they
-// meet at the same workgroup barriers.
+// The gated RMSNorm of one 64 x 128 output tile in LDS.  A function of its own, called, not inlined: inlined into the item
+// loop of the one-launch kernel, the constants of its rare exact path (a double-precision exponential) are hoisted out of
+// the loop and kept in registers through the MFMA phase, which has none to spare.
 constexpr int YS_LD = DV + 8;
+typedef const __attribute__((address_space(3))) bf16_t* lds_bf16_ptr;
+__device__ __attribute__((noinline)) void gated_norm_tile(lds_bf16_ptr ys, int tid, int c, int h, bf16_t* __restrict__ y,
+                                                           const bf16_t* __restrict__ proj, const float* __restrict__ gw, float eps, int S) {
+    const int cc = tid & 15;
+    float gwv[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) gwv[j] = gw[cc * 8 + j];
+    // the four rows of this 16-lane group: all sums of squares first, then one reciprocal square root per lane
+    uint4 yv4[4];
+    float ss4[4], inv4[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int row = it * 16 + (tid >> 4);
+        const u32x4 yw = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(&ys[row * YS_LD + cc * 8]);
+        yv4[it] = make_uint4(yw[0], yw[1], yw[2], yw[3]);
+        float yy[8];
+        unpack8(yv4[it], yy);
+        double ss = 0.0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
+        ss4[it] = (float)row16_sum_d(ss);
+    }
+    rsqrt_rows<4>(ss4, eps, inv4, cc);
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int row = it * 16 + (tid >> 4);
+        const int t = c * C + row;
+        if (t >= S) continue;                                       // whole 16-lane groups leave together
+        const uint4 zv = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
+        float yy[8], zz[8];
+        unpack8(yv4[it], yy);
+        unpack8(zv, zz);
+        uint32_t o[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv4[it]));
+        reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV)[cc] =
+            make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
+    }
+}
+
+// Output role: Y_c = gamma_c * (Qh_c S_c^T) + Am_c D_c for one (chunk, head) by 4 wavefronts; wavefront w covers the dv slices 2w
+// and 2w+1.  The 64 x 128 tile goes through LDS as bf16 and leaves either as y [S,16,128] or, with NORM, straight through the
+// gated RMSNorm (same arithmetic as the stand-alone kernel: 16 lanes per row, 8 columns each; batch.py:338-343).
+// With WAIT the item's snapshots come from a chain that runs in the same launch: `seq` counts the items of this workgroup.
 template <bool NORM, bool WAIT>
-__device__ __forceinline__ void output_role(bf16_t* ys, volatile int* ready, int unit, int units_per_head, const _Float16* __restrict__ ops,
+__device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int seq, int c, int h, const _Float16* __restrict__ ops,
                                             const _Float16* snaps, int* flags, const float* __restrict__ gates,
                                             bf16_t* __restrict__ y, const bf16_t* __restrict__ proj, const float* __restrict__ gw,
-                                            float eps, int S, int NC) {
-    const int h = unit % HV, r0 = unit / HV;
+                                            float eps, int S) {
     const int tid = threadIdx.x & 255, w = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
-    const int rounds = (NC + units_per_head - 1) / units_per_head;
-    for (int rd = 0; rd < rounds; rd++) {
-        const int c = r0 + rd * units_per_head;
-        const bool active = c < NC;                                             // uniform over the unit
-        if (active) {
+    {
+        constexpr bool active = true;
+        {
             const size_t rec = (size_t)c * HV + h;
             const half8* op = reinterpret_cast<const half8*>(ops + rec * OP_HALVES) + lane;
             half8 Sb[2][4], Db[2][2], Qt[16], At[8];
@@ -324,9 +412,9 @@ __device__ __forceinline__ void output_role(bf16_t* ys, volatile int* ready, int
                     }
                     __builtin_amdgcn_s_sleep(32);
                 }
-                if (lane == 0) *ready = c + 1;
+                if (lane == 0) *ready = seq + 1;
             } else {
-                while (*ready <= c) __builtin_amdgcn_s_sleep(2);
+                while (*ready <= seq) __builtin_amdgcn_s_sleep(2);
                 asm volatile("" ::: "memory");
             }
             const _Float16* sp = snaps + (rec * 8 + 2 * w) * SNAP_HALVES + lane * 8;
@@ -370,40 +458,7 @@ __device__ __forceinline__ void output_role(bf16_t* ys, volatile int* ready, int
                     for (int i = 0; i < 4; i++) dst[i] = src[i];
                 }
             } else {
-                const int cc = tid & 15;
-                float gwv[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) gwv[j] = gw[cc * 8 + j];
-                // the four rows of this 16-lane group: all sums of squares first, then one reciprocal square root per lane
-                uint4 yv4[4];
-                float ss4[4], inv4[4];
-#pragma unroll
-                for (int it = 0; it < 4; it++) {
-                    const int row = it * 16 + (tid >> 4);
-                    yv4[it] = *reinterpret_cast<const uint4*>(&ys[row * YS_LD + cc * 8]);
-                    float yy[8];
-                    unpack8(yv4[it], yy);
-                    double ss = 0.0;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
-                    ss4[it] = (float)row16_sum_d(ss);
-                }
-                rsqrt_rows<4>(ss4, eps, inv4, cc);
-#pragma unroll
-                for (int it = 0; it < 4; it++) {
-                    const int row = it * 16 + (tid >> 4);
-                    const int t = c * C + row;
-                    if (t >= S) continue;                                       // whole 16-lane groups leave together
-                    const uint4 zv = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
-                    float yy[8], zz[8];
-                    unpack8(yv4[it], yy);
-                    unpack8(zv, zz);
-                    uint32_t o[8];
-#pragma unroll
-                    for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv4[it]));
-                    reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV)[cc] =
-                        make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
-                }
+                gated_norm_tile((lds_bf16_ptr)ys, tid, c, h, y, proj, gw, eps, S);
             }
         }
         __syncthreads();                                                        // ys is reused by the next round
@@ -411,10 +466,10 @@ __device__ __forceinline__ void output_role(bf16_t* ys, volatile int* ready, int
 }
 
 // the two-launch form: 128 chain workgroups of 320 threads, then one output workgroup of 256 threads per (chunk, head)
-__global__ __launch_bounds__(320) void gdn_chain_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
+__global__ __launch_bounds__(384) void gdn_chain_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
                                                         float* st_out, _Float16* snap, int NC) {
     __shared__ ChainLds chain_lds;
-    chain_role<false>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snap + FLAG_HALVES, nullptr, NC);
+    chain_role<false, 4>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snap + FLAG_HALVES, nullptr, NC);
 }
 template <bool NORM>
 __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restrict__ ops, const _Float16* __restrict__ snap,
@@ -422,37 +477,46 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
                                                          const bf16_t* __restrict__ proj, const float* __restrict__ gw, float eps,
                                                          int S, int NC) {
     __shared__ __align__(16) bf16_t ys[C * YS_LD];
-    // unit = blockIdx = chunk * HV + head, one round: output_role's unit u takes chunk u / HV + round * units_per_head
-    output_role<NORM, false>(ys, nullptr, blockIdx.x, NC, ops, snap + FLAG_HALVES, nullptr, gates, y, proj, gw, eps, S, NC);
+    output_item<NORM, false>(ys, nullptr, 0, blockIdx.x / HV, blockIdx.x % HV, ops, snap + FLAG_HALVES, nullptr, gates, y, proj, gw, eps, S);
 }
 
-// the one-launch form: grid = N_CHAIN + output workgroups (two units each), 512 threads: one workgroup per CU, all resident
+// the one-launch form: N_CHAIN chain workgroups, then output workgroups (4 wavefronts at work) that take (chunk, head) items
+// from a queue in chunk order.  320 threads and at most 168 registers: a CU holds a chain workgroup and an output workgroup,
+// or three output workgroups.  The chain workgroups have the lowest indices, so they are resident before any output
+// workgroup starts, and they wait for nothing: an output workgroup's wait for its item always ends.
 template <bool NORM>
-__global__ __launch_bounds__(512) void gdn_phase_b_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
-                                                          float* st_out, _Float16* snap, bf16_t* y, const bf16_t* proj,
-                                                          const float* gw, float eps, int S, int NC, int units_per_head) {
+__global__ __launch_bounds__(384, 3) void gdn_phase_b_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
+                                                             float* st_out, _Float16* snap, bf16_t* y, const bf16_t* proj,
+                                                             const float* gw, float eps, int S, int NC) {
     __shared__ ChainLds chain_lds;
-    __shared__ __align__(16) bf16_t ys[2][C * YS_LD];
-    __shared__ int ready[2];                                                    // chunks seen complete by each unit's polling wavefront
+    __shared__ __align__(16) bf16_t ys[C * YS_LD];
+    __shared__ int ready, item_s, last;
     int* flags = reinterpret_cast<int*>(snap);
     _Float16* snaps = snap + FLAG_HALVES;
     if (blockIdx.x < N_CHAIN) {
-        chain_role<true>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snaps, flags, NC);
+        chain_role<true, 3>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snaps, flags, NC);
         return;
     }
-    if (threadIdx.x < 2) ready[threadIdx.x] = 0;
-    __syncthreads();
-    const int unit = (blockIdx.x - N_CHAIN) * 2 + (threadIdx.x >> 8);
-    output_role<NORM, true>(ys[threadIdx.x >> 8], ready + (threadIdx.x >> 8), unit, units_per_head, ops, snaps, flags, gates, y, proj, gw,
-                            eps, S, NC);
-    // the last output workgroup to finish leaves the flag area zero for the next launch: by then every chunk has been
-    // consumed, so every chain workgroup has made its last store to it
-    __shared__ int last;
+    if (threadIdx.x >= 256) return;                                             // (a wavefront that has ended is no party to the barriers)
+    if (threadIdx.x == 0) ready = 0;
+    const int total = NC * HV;
+    for (int seq = 0;; seq++) {
+        if (threadIdx.x == 0) item_s = atomicAdd(flags + FLAG_NEXT, 1);
+        __syncthreads();
+        const int item = item_s;
+        if (item >= total) break;
+        output_item<NORM, true>(ys, &ready, seq, item / HV, item % HV, ops, snaps, flags, gates, y, proj, gw, eps, S);
+    }
+    // the last output workgroup to finish leaves the flag area zero for the next launch: by then every item has been
+    // taken and computed, so every chain workgroup has made its last store to it
     if (threadIdx.x == 0) last = atomicAdd(flags + FLAG_DONE, 1) == (int)gridDim.x - N_CHAIN - 1;
     __syncthreads();
     if (last) {
         if (threadIdx.x < N_CHAIN) __hip_atomic_store(flags + threadIdx.x * FLAG_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (threadIdx.x == 0) __hip_atomic_store(flags + FLAG_DONE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) {
+            __hip_atomic_store(flags + FLAG_DONE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(flags + FLAG_NEXT, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 
@@ -953,17 +1017,15 @@ static int phase_b_launch(const void* ops, const void* U, const float* gC, void*
         return QT_OK;
     }
     if (NC >= FUSED_MIN_CHUNKS) {
-        // one launch: unit r of a head takes chunks r, r + UNITS_PER_HEAD, ...; two units per output workgroup
-        const dim3 grid(N_CHAIN + HV * UNITS_PER_HEAD / 2), block(512);
+        const dim3 grid(N_CHAIN + min(MAX_OUT_WGS, NC * HV)), block(384);
         if (norm)
             hipLaunchKernelGGL(gdn_phase_b_kernel<true>, grid, block, 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
-                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S, NC, UNITS_PER_HEAD);
+                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S, NC);
         else
             hipLaunchKernelGGL(gdn_phase_b_kernel<false>, grid, block, 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
-                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S, NC,
-                               UNITS_PER_HEAD);
+                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S, NC);
     } else {
-        hipLaunchKernelGGL(gdn_chain_kernel, dim3(N_CHAIN), dim3(320), 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
+        hipLaunchKernelGGL(gdn_chain_kernel, dim3(N_CHAIN), dim3(384), 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
                            state_out, (_Float16*)snap, NC);
         QT_CHECK_LAUNCH();
         if (norm)
