@@ -391,9 +391,9 @@ __device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int
             for (int i = 0; i < 16; i++) Qt[i] = op[(OP_Q / 8) + i * 64];
 #pragma unroll
             for (int i = 0; i < 8; i++) At[i] = op[(OP_A / 8) + i * 64];
-            f32x4 gam[NCT];                                                     // gamma of this lane's four rows of every row tile
+            float gam[NCT];                                                     // gamma of this lane's token of every row tile
 #pragma unroll
-            for (int ct = 0; ct < NCT; ct++) gam[ct] = *reinterpret_cast<const f32x4*>(gates + rec * GATE_FLOATS + G_GAM + 16 * ct + 4 * g);
+            for (int ct = 0; ct < NCT; ct++) gam[ct] = gates[rec * GATE_FLOATS + G_GAM + 16 * ct + n];
             // wait until the chain has published chunk c for all eight slices of the head: the unit's first wavefront polls (lanes
             // 0..7, one progress word each, about once a microsecond: thousands of pollers on one memory line would hold up the
             // chain's own progress stores) and passes the news on through LDS, where the other three wavefronts wait
@@ -427,23 +427,26 @@ __device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int
             }
 #pragma unroll
             for (int s = 0; s < 2; s++) {
+                // the products are taken transposed (the snapshot as the A operand, the Qh / Am tile as the B operand: the same
+                // registers either way), so that a lane holds four consecutive columns of one token: Y[ct][r] = y[token 16 ct + n][dv
+                // 16 (2 w + s) + 4 g + r], eight bytes of a row of the LDS tile
                 f32x4 Y[NCT];
 #pragma unroll
                 for (int ct = 0; ct < NCT; ct++) Y[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kb = 0; kb < 4; kb++)
 #pragma unroll
-                    for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Qt[ct * 4 + kb], Sb[s][kb], Y[ct], 0, 0, 0);
+                    for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Sb[s][kb], Qt[ct * 4 + kb], Y[ct], 0, 0, 0);
 #pragma unroll
                 for (int ct = 0; ct < NCT; ct++) Y[ct] *= gam[ct];
 #pragma unroll
                 for (int kb2 = 0; kb2 < 2; kb2++)
 #pragma unroll
-                    for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(At[ct * 2 + kb2], Db[s][kb2], Y[ct], 0, 0, 0);
+                    for (int ct = 0; ct < NCT; ct++) Y[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Db[s][kb2], At[ct * 2 + kb2], Y[ct], 0, 0, 0);
 #pragma unroll
                 for (int ct = 0; ct < NCT; ct++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) ys[(ct * 16 + 4 * g + r) * YS_LD + (2 * w + s) * 16 + n] = f2bf(Y[ct][r]);
+                    *reinterpret_cast<uint2*>(&ys[(ct * 16 + n) * YS_LD + (2 * w + s) * 16 + 4 * g]) =
+                        make_uint2(pack2_bf(Y[ct][0], Y[ct][1]), pack2_bf(Y[ct][2], Y[ct][3]));
             }
         }
         __syncthreads();

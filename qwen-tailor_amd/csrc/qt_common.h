@@ -79,9 +79,19 @@ __device__ __forceinline__ float decay_gate(float A_log, float av) { return expf
 // z * sigmoid(z) * n rounded to bf16 once (kernels.py:134-137): z/(1+exp32(-z)) * n.  The fast path uses the hardware
 // reciprocal and float exp (a few ulp off in total); a result within 16 float ulp of a bf16 rounding boundary, or a large |z|,
 // takes the exact path (IEEE divide, double-precision exp).
+// exp(-z) for |z| <= 80: the steps of the library's float exp (-z log2(e) as a two-term product, the fraction through
+// v_exp_f32, the integer part applied by ldexp; <= 1 ulp) without its overflow and underflow selects
+__device__ __forceinline__ float exp_neg_in_range(float z) {
+    const float c_hi = -1.44269502f, c_lo = -1.92596299e-08f;                    // -log2(e) = c_hi + c_lo
+    const float ph = z * c_hi;
+    float pl = __builtin_fmaf(z, c_hi, -ph);
+    pl = __builtin_fmaf(z, c_lo, pl);
+    const float ip = __builtin_rintf(ph);
+    return __builtin_ldexpf(__builtin_amdgcn_exp2f((ph - ip) + pl), (int)ip);
+}
 __device__ __forceinline__ bf16_t gated_out(float z, float n) {
-    float o = z * __builtin_amdgcn_rcpf(1.0f + expf(-z)) * n;
-    if (__builtin_expect(near_bf16_tie(o, 16) || fabsf(z) > 80.0f, 0)) o = __fdiv_rn(z, 1.0f + exp32(-z)) * n;
+    float o = z * __builtin_amdgcn_rcpf(1.0f + exp_neg_in_range(z)) * n;
+    if (__builtin_expect(near_bf16_tie(o, 16) || !(fabsf(z) <= 80.0f), 0)) o = __fdiv_rn(z, 1.0f + exp32(-z)) * n;
     return f2bf(o);
 }
 
