@@ -73,8 +73,11 @@ __host__ __device__ inline long parts_upto(long n, long c) {      // sum over j 
     const long k = n / c;
     return c * (k * (k + 1) / 2) + (n - k * c) * (k + 1);
 }
-// floats of one part's O, [4 heads][RB rows][256], and of its m, l, [4 heads][m | l][RB rows] (RB = rows of a block: 16 or 32)
+// elements of one part's O, [4 heads][RB rows][256] in half precision (each row divided by its row sum, so that the values are
+// weighted means of V), and floats of its m, l, [4 heads][m | l][RB rows] (RB = rows of a block: 16 or 32)
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 constexpr int part_o_floats(int RB) { return 4 * RB * AD; }
+constexpr long part_bytes(int RB) { return (long)part_o_floats(RB) * 2 + (long)(4 * 2 * RB) * 4; }
 constexpr int part_ml_floats(int RB) { return 4 * 2 * RB; }
 
 // NH = heads per wavefront: 2 (32 query rows per workgroup, as described above) for long sequences; 1 (16 rows per workgroup,
@@ -84,7 +87,7 @@ template <int NH>
 __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
                                                            const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
                                                            int q_pos0, long q_head_stride, long kv_head_stride, int tmax,
-                                                           float* __restrict__ part_o, float* __restrict__ part_ml) {
+                                                           _Float16* __restrict__ part_o, float* __restrict__ part_ml) {
     // four separate arrays, not [2][TILE]: the compiler tracks outstanding direct-to-LDS loads per LDS variable, so a read of
     // one buffer does not wait for the loads in flight to the others
     __shared__ __align__(1024) bf16_t k_s0[TILE];
@@ -427,14 +430,15 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
 #pragma unroll
         for (int hh = 0; hh < NH; hh++) {
             const int hq = (NH == 2 ? 2 * (w & 1) : w) + hh;     // head within the KV group
-            float* po = part_o + (slot * 4 + hq) * (RB * AD);
+            _Float16* po = part_o + (slot * 4 + hq) * (RB * AD);
             float* pml = part_ml + (slot * 4 + hq) * (2 * RB);
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int lr = lr0 + 4 * g + r;
                 const bool seen = q_pos0 + rb * RB + lr >= first_key;
+                const float inv = seen ? 1.0f / Lsum[hh][r] : 0.f;
 #pragma unroll
-                for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n] = seen ? O[hh][j][r] : 0.f;
+                for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n] = (_Float16)(seen ? O[hh][j][r] * inv : 0.f);
                 if (n == 0) pml[RB + lr] = seen ? Lsum[hh][r] : 0.f;
             }
             if (g == 0) pml[lr0 + n] = my_last >= first_key ? m_run[hh] : NEG;
@@ -458,10 +462,10 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
 }
 
 // Combines the parts of the row blocks that were split: grid = (split blocks, KV heads, 4 heads of the group x 16-row halves of
-// a block); thread (row, 16-column group) of 16 x 256 outputs.  out = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p, parts in order; a
+// a block); thread (row, 16-column group) of 16 x 256 outputs.  out = sum_p w_p O_p / sum_p w_p, w_p = 2^(m_p - m) l_p, parts in order; a
 // thread's loads of O do not depend on the factors, so all parts are in flight together.
 template <int RB>
-__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const _Float16* __restrict__ part_o, const float* __restrict__ part_ml,
                                                                  bf16_t* __restrict__ out, int S, int q_pos0, int tmax, long slots_per_kv,
                                                                  long q_head_stride) {
     constexpr int PO = part_o_floats(RB), PML = part_ml_floats(RB);
@@ -473,7 +477,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
     {
         const int lr = 16 * (blockIdx.z % (RB / 16)) + (threadIdx.x >> 4);
         if (rb * RB + lr >= S) return;
-        const float* po = part_o + (slot0 * 4 + hq) * (RB * AD) + lr * AD + cg * 16;
+        const _Float16* po = part_o + (slot0 * 4 + hq) * (RB * AD) + lr * AD + cg * 16;
         const float* pml = part_ml + (slot0 * 4 + hq) * (2 * RB) + lr;
         float m = NEG;
         for (int pp = 0; pp < np; pp++) m = fmaxf(m, pml[(size_t)pp * PML]);
@@ -483,13 +487,15 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
         for (int i = 0; i < 4; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 2
         for (int pp = 0; pp < np; pp++) {
-            f32x4 o[4];
+            half8 oh[2];
 #pragma unroll
-            for (int i = 0; i < 4; i++) o[i] = reinterpret_cast<const f32x4*>(po + (size_t)pp * PO)[i];
-            const float f = __builtin_amdgcn_exp2f(pml[(size_t)pp * PML] - m);
-            l += f * pml[(size_t)pp * PML + RB];
+            for (int i = 0; i < 2; i++) oh[i] = reinterpret_cast<const half8*>(po + (size_t)pp * PO)[i];
+            const float f = __builtin_amdgcn_exp2f(pml[(size_t)pp * PML] - m) * pml[(size_t)pp * PML + RB];
+            l += f;
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[i] += f * o[i];
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[i][e] += f * (float)oh[i >> 1][4 * (i & 1) + e];
         }
         const float inv = 1.0f / l;
         uint32_t pk[8];
@@ -522,7 +528,7 @@ struct KeySplit {
     int tmax = 0;
     long parts = 0;
     int split_blocks = 0;
-    long bytes() const { return parts * AKV * (long)(part_o_floats(16 * nh) + part_ml_floats(16 * nh)) * 4; }
+    long bytes() const { return parts * AKV * part_bytes(16 * nh); }
 };
 KeySplit plan_split_nh(int S, int L, int q_pos0, int nh, int min_gain) {
     KeySplit ks;
@@ -586,8 +592,8 @@ long qt_gqa_prefill_workspace_bytes_for(int S, int L, int q_pos0) {
 long qt_gqa_prefill_workspace_bytes(int L) {
     if (L < 0) return -1;
     const long cus = cu_count(), nb16 = std::min((long)(L + 15) / 16, cus / AKV), nb32 = std::min((long)(L + 31) / 32, cus / AKV);
-    const long b16 = (cus + AKV * (2 * nb16 + 2)) * (long)(part_o_floats(16) + part_ml_floats(16)) * 4;
-    const long b32 = (cus + AKV * (2 * nb32 + 2)) * (long)(part_o_floats(32) + part_ml_floats(32)) * 4;
+    const long b16 = (cus + AKV * (2 * nb16 + 2)) * part_bytes(16);
+    const long b32 = (cus + AKV * (2 * nb32 + 2)) * part_bytes(32);
     return std::max(b16, b32);
 }
 
@@ -609,8 +615,8 @@ int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out
     }
     const int RB = 16 * ks.nh;
     const dim3 grid((ks.tmax ? (unsigned)ks.parts : (unsigned)((S + RB - 1) / RB)) * AKV);
-    float* part_o = ks.tmax ? (float*)workspace : nullptr;
-    float* part_ml = ks.tmax ? part_o + (size_t)ks.parts * AKV * part_o_floats(RB) : nullptr;
+    _Float16* part_o = ks.tmax ? (_Float16*)workspace : nullptr;
+    float* part_ml = ks.tmax ? reinterpret_cast<float*>(part_o + (size_t)ks.parts * AKV * part_o_floats(RB)) : nullptr;
     if (ks.nh == 2)
         hipLaunchKernelGGL(attn_prefill_kernel<2>, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
                            (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
