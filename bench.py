@@ -27,7 +27,9 @@ DECODE_TRAFFIC_B64 = int((34563.5 * 1.9993 + 68142.9) * 1024)
 DECODE_TRAFFIC_SOURCE = ("profiles/gdn_decode_wide_kernel_B64.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gdn_decode_wide_kernel<4> at "
                          "B=64 (a recorded measurement of that kernel, not of this run)")
 # same for the three kernels of the T = 2048 prefill (profiles/gdn_prefill_T2048.md)
-PREFILL_TRAFFIC_T2048 = int(((17328.8 + 16941.0 + 23758.5) * 1.9993 + 49204 + 25600 + 8192) * 1024)
+PREFILL_TRAFFIC_T2048 = int(((16715.9 + 12942.5 + 23841.5) * 1.9993 + 37172 + 25600 + 8192) * 1024)
+PREFILL_TRAFFIC_SOURCE = ("profiles/gdn_prefill_T2048.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gdn_phase_a_kernel, gdn_chain_kernel and "
+                          "gdn_output_kernel at T=2048 (a recorded measurement of those kernels, not of this run)")
 
 
 def decode_bytes(B):
@@ -406,6 +408,8 @@ def profile_leg(torch, qt, dev, args):
     elif leg == "prefill":
         for _ in range(3):
             bench_prefill_once(torch, qt, dev, 2048)
+    elif leg == "prefill_long":
+        bench_prefill_once(torch, qt, dev, 8192)
     elif leg == "verify":
         bench_verify_gdn(torch, qt, dev)
     elif leg == "attn_decode":
@@ -452,7 +456,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the B sweep and the single-pool run")
     ap.add_argument("--only", default="", help="profile helper: run only one leg a few times and exit "
-                                               "(decode | copy | prefill | verify | attn_decode | attn_verify | attn_prefill | attn_prefill_long | "
+                                               "(decode | copy | prefill | prefill_long | verify | attn_decode | attn_verify | attn_prefill | attn_prefill_long | "
                                                "projections | state_admission | prefix_cache | attn_glue)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -568,7 +572,8 @@ def main():
                             "config": {"workload": "configs[2]: conv + chunked GDN (chunk 64) + gated RMSNorm, B=1, T=2048, 16 heads, "
                                                    "nonzero initial state"},
                             "roofline": {"bound": "mfma", "achieved": p2k["mfma_tflops"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                         "frac": p2k["mfma_frac"], "traffic": PREFILL_TRAFFIC_T2048}}
+                                         "frac": p2k["mfma_frac"], "traffic": PREFILL_TRAFFIC_T2048,
+                                         "traffic_source": PREFILL_TRAFFIC_SOURCE}}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B)
     print(json.dumps(out))

@@ -77,7 +77,7 @@ constexpr int SNAP_D = 2 * 512;                  // halves: D as B operand, [kb2
 constexpr int SNAP_HALVES = SNAP_S + SNAP_D;     // 6 KiB per (chunk, head, slice)
 constexpr int KORD[4] = {0, 2, 1, 3};            // order in which a step consumes its Kh tiles (two independent accumulators)
 constexpr int N_CHAIN = HV * 8;                  // chain workgroups
-constexpr int PF_AHEAD = 10;                     // chunks between the L2 prefetch and the chain
+constexpr int PF_AHEAD = 16;                     // chunks between the L2 prefetch and the chain
 constexpr int PF_SLOTS = 8;                      // prefetch loads in flight
 constexpr int PUB_LAG = 8;                       // a chunk is published when at most this many newer chunks' stores are in flight
 constexpr int FLAG_STRIDE = 64;                  // ints between progress words: every word has a 256-byte stretch of its own
@@ -85,7 +85,7 @@ constexpr int FLAG_WORDS = (N_CHAIN + 1) * FLAG_STRIDE;   // flag area at the he
 constexpr int FLAG_DONE = N_CHAIN * FLAG_STRIDE, FLAG_ERR = FLAG_DONE + 1, FLAG_NEXT = FLAG_DONE + 2;   // FLAG_NEXT: head of the item queue
 constexpr int FLAG_HALVES = FLAG_WORDS * 2;
 constexpr int SPIN_LIMIT = 1 << 21;              // polls (about a second) before a consumer gives up
-constexpr int MAX_OUT_WGS = 256;                 // output workgroups of the one-launch form: what fits beside the chain workgroups
+constexpr int MAX_OUT_WGS = 384;                 // output workgroups of the one-launch form: what fits beside the chain workgroups
 constexpr int FUSED_MIN_CHUNKS = 64;              // from 4096 tokens on the one-launch form wins (measured: 2048 tokens 37 / 35 us, 8192 134 / 155 us)
 typedef unsigned long long u64;
 

@@ -89,7 +89,7 @@ def test_prefill_attention_split_plan_on_the_host():
     assert need(-1, 8, 0) == -1 and need(8, 0, 0) == -1 and bound(-1) == -1
     assert need(4096, 4096, 0) == 0 and need(8192, 8192, 0) == 0          # a workgroup per CU or more: not split
     assert need(0, 64, 64) == 0 and need(5, 5, 0) == 0                    # nothing to split
-    part = 4 * (16 * 256 + 2 * 16) * 4                                    # bytes of one part: O, m, l of 16 rows x 4 heads
+    part = 4 * (16 * 256 * 2 + 2 * 16 * 4)                                # bytes of one part: O (half precision), m, l (float) of 16 rows x 4 heads
     for S, P0 in ((64, 8000), (16, 32000), (1024, 0), (1536, 1000), (300, 4001), (1, 4095), (2048, 0), (2048, 6000)):
         n = need(S, S + P0, P0)
         size = part * (2 if S >= 1472 else 1)                             # from about 1500 rows on the row blocks are 32 rows
