@@ -102,15 +102,15 @@ int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_ne
 
 /* Chunked (chunk = 64) GatedDeltaNet prefill, two phases (qwen35/gdn_nax.py:394-426: prep_a / gdn_chunked's phase A, phase_b).
  * Phase A is parallel over (chunk, head): it takes q, k, v [S,16,128] bf16 (qt_gdn_conv_prep's outputs) and the gate inputs in
- * proj [S,8224], and computes the gates, K K^T / Q K^T on bf16 MFMA, the 64 x 64 unit-lower-triangular inverse in fp32 and the
+ * proj [S,8224], and computes the gates, K K^T / Q K^T on fp16 MFMA, the 64 x 64 unit-lower-triangular inverse in fp32 and the
  * state-independent MFMA operands of phase B.  It fills three caller-owned buffers of qt_gdn_chunk_{ops,u,gc}_bytes(S) bytes, all
  * 16-byte aligned: `ops` and `U` (half-precision operand tiles) and `gC` (f32: per (chunk, head) the 64 per-token decay
  * factors gamma and dec and the chunk's total decay, which phase B applies to accumulator rows).
  * Intermediate operands are half precision (fp16: 11 significant bits, largest finite value 65504): conv outputs |v| and
  * states |S| beyond that are not representable and are not supported; values below 6e-5 lose precision gracefully.
- * Phase B: state_in / state_out [16,128,128] f32, y [S,16,128] bf16.  One launch with two kinds of workgroups: 128 run the
- * serial state chain over the chunks and leave the per-chunk B operands in `snap`; the others compute the outputs of a
- * chunk as soon as the chain has published it.  `snap`: qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned; its
+ * Phase B: state_in / state_out [16,128,128] f32, y [S,16,128] bf16.  128 workgroups run the serial state chain over the chunks
+ * and leave the per-chunk B operands in `snap`; others compute the outputs of a chunk from them: as a second launch up to 4095
+ * tokens, from 4096 on in the same launch, as soon as the chain has published the chunk.  `snap`: qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned; its
  * first 33 KiB (qt_gdn_chunk_snap_bytes(0) bytes) are the progress words of the launch and MUST BE ZERO when a launch starts.  A launch leaves them zero, so
  * the caller zeroes them once; launches that use the same `snap` must not overlap.
  * qt_gdn_phase_b_norm is the same with prefill.gated_norm (qwen35/prefill.py:241-244) fused into the output kernel: it
