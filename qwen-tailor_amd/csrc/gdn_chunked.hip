@@ -326,12 +326,21 @@ __device__ __forceinline__ void chain_role(ChainLds& L, int blk, const _Float16*
     }
 }
 
-// The gated RMSNorm of one 64 x 128 output tile in LDS.  A function of its own, called, not inlined: inlined into the item
-// loop of the one-launch kernel, the constants of its rare exact path (a double-precision exponential) are hoisted out of
-// the loop and kept in registers through the MFMA phase, which has none to spare.
+// gated_out (qt_common.h) with its exact path as a called function: inlined 32 times, that path (an IEEE division and a
+// double-precision exponential) is most of the norm's code, and every wavefront runs it a few times per tile.  The
+// instruction cache is shared by two CUs: a chain workgroup's three-step loop has to stay in it while its neighbour's
+// output workgroups run this code.
+__device__ __attribute__((noinline)) float gated_out_exact(float z, float n) { return __fdiv_rn(z, 1.0f + exp32(-z)) * n; }
+__device__ __forceinline__ bf16_t gated_out_small(float z, float n) {
+    float o = z * __builtin_amdgcn_rcpf(1.0f + exp_neg_in_range(z)) * n;
+    if (__builtin_expect(near_bf16_tie(o, 16) || !(fabsf(z) <= 80.0f), 0)) o = gated_out_exact(z, n);
+    return f2bf(o);
+}
+
+// The gated RMSNorm of one 64 x 128 output tile in LDS.
 constexpr int YS_LD = DV + 8;
 typedef const __attribute__((address_space(3))) bf16_t* lds_bf16_ptr;
-__device__ __attribute__((noinline)) void gated_norm_tile(lds_bf16_ptr ys, int tid, int c, int h, bf16_t* __restrict__ y,
+__device__ __forceinline__ void gated_norm_tile(lds_bf16_ptr ys, int tid, int c, int h, bf16_t* __restrict__ y,
                                                            const bf16_t* __restrict__ proj, const float* __restrict__ gw, float eps, int S) {
     const int cc = tid & 15;
     float gwv[8];
@@ -352,21 +361,28 @@ __device__ __attribute__((noinline)) void gated_norm_tile(lds_bf16_ptr ys, int t
         for (int j = 0; j < 4; j++) ss += (double)yy[2 * j] * yy[2 * j] + (double)yy[2 * j + 1] * yy[2 * j + 1];
         ss4[it] = (float)row16_sum_d(ss);
     }
+    // every z row is requested before the first result is stored: a wavefront's loads and stores share one counter, so a load
+    // issued behind a store is waited for together with it, and a store takes microseconds to complete
+    uint4 zv4[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int t = min(c * C + it * 16 + (tid >> 4), S - 1);
+        zv4[it] = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
+    }
     rsqrt_rows<4>(ss4, eps, inv4, cc);
 #pragma unroll
     for (int it = 0; it < 4; it++) {
         const int row = it * 16 + (tid >> 4);
         const int t = c * C + row;
         if (t >= S) continue;                                       // whole 16-lane groups leave together
-        const uint4 zv = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
         float yy[8], zz[8];
         unpack8(yv4[it], yy);
-        unpack8(zv, zz);
+        unpack8(zv4[it], zz);
         uint32_t o[8];
 #pragma unroll
-        for (int j = 0; j < 8; j++) o[j] = gated_out(zz[j], gwv[j] * (yy[j] * inv4[it]));
-        reinterpret_cast<uint4*>(y + ((size_t)t * HV + h) * DV)[cc] =
-            make_uint4(o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16));
+        for (int j = 0; j < 8; j++) o[j] = gated_out_small(zz[j], gwv[j] * (yy[j] * inv4[it]));
+        const u32x4 ov = {o[0] | (o[1] << 16), o[2] | (o[3] << 16), o[4] | (o[5] << 16), o[6] | (o[7] << 16)};
+        __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(y + ((size_t)t * HV + h) * DV) + cc);   // written once, read by a later kernel
     }
 }
 
