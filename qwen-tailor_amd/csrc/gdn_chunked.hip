@@ -332,8 +332,8 @@ __device__ __forceinline__ void chain_role(ChainLds& L, int blk, const _Float16*
 // output workgroups run this code.
 __device__ __attribute__((noinline)) float gated_out_exact(float z, float n) { return __fdiv_rn(z, 1.0f + exp32(-z)) * n; }
 __device__ __forceinline__ bf16_t gated_out_small(float z, float n) {
-    float o = z * __builtin_amdgcn_rcpf(1.0f + exp_neg_in_range(z)) * n;
-    if (__builtin_expect(near_bf16_tie(o, 16) || !(fabsf(z) <= 80.0f), 0)) o = gated_out_exact(z, n);
+    float o;
+    if (__builtin_expect(!gated_out_fast(z, n, o), 0)) o = gated_out_exact(z, n);
     return f2bf(o);
 }
 

@@ -76,22 +76,23 @@ __device__ __forceinline__ float softplus_bf16(float x) {                       
 // float exp and does not round it; here both exps are float with <= 1 ulp error.
 __device__ __forceinline__ float log_decay(float A_log, float av) { return -expf(A_log) * softplus_bf16(av); }
 __device__ __forceinline__ float decay_gate(float A_log, float av) { return expf(log_decay(A_log, av)); }
-// z * sigmoid(z) * n rounded to bf16 once (kernels.py:134-137): z/(1+exp32(-z)) * n.  The fast path uses the hardware
-// reciprocal and float exp (a few ulp off in total); a result within 16 float ulp of a bf16 rounding boundary, or a large |z|,
-// takes the exact path (IEEE divide, double-precision exp).
-// exp(-z) for |z| <= 80: the steps of the library's float exp (-z log2(e) as a two-term product, the fraction through
-// v_exp_f32, the integer part applied by ldexp; <= 1 ulp) without its overflow and underflow selects
-__device__ __forceinline__ float exp_neg_in_range(float z) {
-    const float c_hi = -1.44269502f, c_lo = -1.92596299e-08f;                    // -log2(e) = c_hi + c_lo
-    const float ph = z * c_hi;
-    float pl = __builtin_fmaf(z, c_hi, -ph);
-    pl = __builtin_fmaf(z, c_lo, pl);
-    const float ip = __builtin_rintf(ph);
-    return __builtin_ldexpf(__builtin_amdgcn_exp2f((ph - ip) + pl), (int)ip);
+// exp(-z) for a bf16 value z, |z| <= 16, in four instructions.  -log2(e) = c1 + c2 with c1 of 16 significant bits, so the
+// product z c1 is exact in float; exp(-z) = 2^(z c1) (1 + z c2 ln 2 + ...), the second-order term below 1e-8.  v_exp_f32 is
+// good to 1 ulp, the multiply-add adds half of one.
+__device__ __forceinline__ float exp_neg_bf16(float z) {
+    const float e0 = __builtin_amdgcn_exp2f(z * -1.44268798828125f);
+    return __builtin_fmaf(e0, z * -4.888495152129525e-06f, e0);
+}
+// z * sigmoid(z) * n rounded to bf16 once (kernels.py:134-137): z/(1+exp32(-z)) * n, z a bf16 value.  The fast path uses the
+// hardware reciprocal and the exponential above (a few ulp off in total); a result within 16 float ulp of a bf16 rounding
+// boundary, or |z| > 16, takes the exact path (IEEE divide, double-precision exp).
+__device__ __forceinline__ bool gated_out_fast(float z, float n, float& o) {
+    o = z * __builtin_amdgcn_rcpf(1.0f + exp_neg_bf16(z)) * n;
+    return !(near_bf16_tie(o, 16) || !(fabsf(z) <= 16.0f));
 }
 __device__ __forceinline__ bf16_t gated_out(float z, float n) {
-    float o = z * __builtin_amdgcn_rcpf(1.0f + exp_neg_in_range(z)) * n;
-    if (__builtin_expect(near_bf16_tie(o, 16) || !(fabsf(z) <= 80.0f), 0)) o = __fdiv_rn(z, 1.0f + exp32(-z)) * n;
+    float o;
+    if (__builtin_expect(!gated_out_fast(z, n, o), 0)) o = __fdiv_rn(z, 1.0f + exp32(-z)) * n;
     return f2bf(o);
 }
 
