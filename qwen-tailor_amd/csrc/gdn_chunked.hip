@@ -340,6 +340,14 @@ __device__ __forceinline__ bf16_t gated_out_small(float z, float n) {
 // The gated RMSNorm of one 64 x 128 output tile in LDS.
 constexpr int YS_LD = DV + 8;
 typedef const __attribute__((address_space(3))) bf16_t* lds_bf16_ptr;
+// a load of data that nothing reads again.  In the one-launch form (STREAM) it is marked nontemporal: there the output
+// workgroups stream beside the chain, whose operands wait in the L2 for their step, and must not push them out.  In the
+// two-launch form the same mark costs time (the records are still in the L2 from the kernel that wrote them).
+template <bool STREAM, typename T>
+__device__ __forceinline__ T load_once(const T* p) {
+    return STREAM ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool STREAM>
 __device__ __forceinline__ void gated_norm_tile(lds_bf16_ptr ys, int tid, int c, int h, bf16_t* __restrict__ y,
                                                            const bf16_t* __restrict__ proj, const float* __restrict__ gw, float eps, int S) {
     const int cc = tid & 15;
@@ -367,7 +375,8 @@ __device__ __forceinline__ void gated_norm_tile(lds_bf16_ptr ys, int tid, int c,
 #pragma unroll
     for (int it = 0; it < 4; it++) {
         const int t = min(c * C + it * 16 + (tid >> 4), S - 1);
-        zv4[it] = reinterpret_cast<const uint4*>(proj + (size_t)t * PW + CD + h * DV)[cc];
+        const u32x4 zw = load_once<STREAM>(reinterpret_cast<const u32x4*>(proj + (size_t)t * PW + CD + h * DV) + cc);
+        zv4[it] = make_uint4(zw[0], zw[1], zw[2], zw[3]);
     }
     rsqrt_rows<4>(ss4, eps, inv4, cc);
 #pragma unroll
@@ -404,9 +413,9 @@ __device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int
             half8 Sb[2][4], Db[2][2], Qt[16], At[8];
             // what does not depend on the chain is requested before the wait
 #pragma unroll
-            for (int i = 0; i < 16; i++) Qt[i] = op[(OP_Q / 8) + i * 64];
+            for (int i = 0; i < 16; i++) Qt[i] = load_once<WAIT>(&op[(OP_Q / 8) + i * 64]);
 #pragma unroll
-            for (int i = 0; i < 8; i++) At[i] = op[(OP_A / 8) + i * 64];
+            for (int i = 0; i < 8; i++) At[i] = load_once<WAIT>(&op[(OP_A / 8) + i * 64]);
             float gam[NCT];                                                     // gamma of this lane's token of every row tile
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) gam[ct] = gates[rec * GATE_FLOATS + G_GAM + 16 * ct + n];
@@ -477,7 +486,7 @@ __device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int
                     for (int i = 0; i < 4; i++) dst[i] = src[i];
                 }
             } else {
-                gated_norm_tile((lds_bf16_ptr)ys, tid, c, h, y, proj, gw, eps, S);
+                gated_norm_tile<WAIT>((lds_bf16_ptr)ys, tid, c, h, y, proj, gw, eps, S);
             }
         }
         __syncthreads();                                                        // ys is reused by the next round
