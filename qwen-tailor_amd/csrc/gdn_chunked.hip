@@ -963,7 +963,7 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool write_qk
                     }
                 }
             }
-            *reinterpret_cast<half8*>(op + OP_A + (ct * 2 + kb2) * 512 + lane * 8) = pack_half8(part[0], part[1]);
+            __builtin_nontemporal_store(pack_half8(part[0], part[1]), reinterpret_cast<half8*>(op + OP_A + (ct * 2 + kb2) * 512 + lane * 8));
         }
         // Qh = Q (rows of tile ct), k index permuted: two 8-byte pieces of the row
         for (int kb = 0; kb < 4; kb++) {
@@ -972,7 +972,7 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool write_qk
             half8 qh;
             qh[0] = lo[0]; qh[1] = lo[1]; qh[2] = lo[2]; qh[3] = lo[3];
             qh[4] = hi[0]; qh[5] = hi[1]; qh[6] = hi[2]; qh[7] = hi[3];
-            *reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8) = qh;
+            __builtin_nontemporal_store(qh, reinterpret_cast<half8*>(op + OP_Q + (ct * 4 + kb) * 512 + lane * 8));
         }
         return;
     }
