@@ -939,6 +939,12 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool write_qk
         part_staged(L, PA_V, lane);
         await_part(L, PA_Q);
         await_part(L, PA_K);
+        // Kh = K^T (rows dk of tiles 2w, 2w+1), k index permuted: group V has the time for it (group M ends last)
+        for (int mm = 0; mm < 2; mm++) {
+            const int mt = 2 * w + mm;
+            for (int kb2 = 0; kb2 < 2; kb2++)
+                *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g);
+        }
         // ---- Am = lower_incl(G * Q K^T) transposed, rows c_out = 16 ct + n, k = c_in (permuted); G_ij = exp2(Lc2_i - Lc2_j)
         const int ct = w, co = 16 * ct + n;
         const float lco = L.Lc2[co];
@@ -998,12 +1004,6 @@ __global__ __launch_bounds__(512, 4) void gdn_phase_a_kernel(const bool write_qk
             }
         }
         *reinterpret_cast<half8*>(op + OP_W + (ct * 4 + kb) * 512 + lane * 8) = pack_half8(acc[0], acc[1]);
-    }
-    // Kh = K^T (rows dk of tiles 2w, 2w+1), k index permuted
-    for (int mm = 0; mm < 2; mm++) {
-        const int mt = 2 * w + mm;
-        for (int kb2 = 0; kb2 < 2; kb2++)
-            *reinterpret_cast<half8*>(op + OP_K + (mt * 2 + kb2) * 512 + lane * 8) = tokens_operand(L.Ks, QS_LD, kb2, 16 * mt, n, g);
     }
     __builtin_amdgcn_s_setprio(0);
     await_part(L, PA_V);
