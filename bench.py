@@ -27,7 +27,7 @@ DECODE_TRAFFIC_B64 = int((34563.5 * 1.9993 + 68142.9) * 1024)
 DECODE_TRAFFIC_SOURCE = ("profiles/gdn_decode_wide_kernel_B64.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gdn_decode_wide_kernel<4> at "
                          "B=64 (a recorded measurement of that kernel, not of this run)")
 # same for the three kernels of the T = 2048 prefill (profiles/gdn_prefill_T2048.md)
-PREFILL_TRAFFIC_T2048 = int(((16715.9 + 12942.5 + 23841.5) * 1.9993 + 37172 + 25600 + 8192) * 1024)
+PREFILL_TRAFFIC_T2048 = int(((16710.2 + 13618.8 + 23732.0) * 1.9993 + 37172 + 25600 + 8192) * 1024)
 PREFILL_TRAFFIC_SOURCE = ("profiles/gdn_prefill_T2048.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gdn_phase_a_kernel, gdn_chain_kernel and "
                           "gdn_output_kernel at T=2048 (a recorded measurement of those kernels, not of this run)")
 
