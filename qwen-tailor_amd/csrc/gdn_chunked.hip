@@ -59,10 +59,10 @@ __device__ __forceinline__ half8 pack_half8(const f32x4& a, const f32x4& b) {
 // snapshots and progress words cross CUs (and XCDs, whose L2s are not coherent with each other) inside one launch, so they
 // are written and read with device-scope accesses that go to memory; everything else uses plain accesses.  The writer never
 // waits for its newest stores: it publishes chunk c - PUB_LAG once at most the stores of the PUB_LAG newest chunks are still
-// in flight (stores of one wavefront complete in order).  Every workgroup of that launch is resident at once (512 threads,
-// one workgroup per CU, at most 256 of them), so a consumer's producer is always running; a consumer that does not see its
-// snapshot within SPIN_LIMIT polls gives up, sets the error word and computes on what is there, so that every wavefront
-// ends.  The last output workgroup to finish clears the progress words: the flag area is zero before and after every launch
+// in flight (stores of one wavefront complete in order).  The chain workgroups have the lowest indices, so all of them are
+// running before the first output workgroup starts, and they wait for nothing: a consumer's producer is always running,
+// whether or not every output workgroup is resident.  A consumer that does not see its snapshot within SPIN_LIMIT polls
+// gives up, sets the error word and computes on what is there, so that every wavefront ends.  The last output workgroup to finish clears the progress words: the flag area is zero before and after every launch
 // (the caller zeroes it once).
 //
 // Chain role: 5 wavefronts per (head, 16-wide dv slice).  MFMA wavefront w owns rows 16w..16w+15 of D (the chunk's tokens) and
@@ -509,9 +509,12 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
 }
 
 // the one-launch form: N_CHAIN chain workgroups, then output workgroups (4 wavefronts at work) that take (chunk, head) items
-// from a queue in chunk order.  320 threads and at most 168 registers: a CU holds a chain workgroup and an output workgroup,
-// or three output workgroups.  The chain workgroups have the lowest indices, so they are resident before any output
-// workgroup starts, and they wait for nothing: an output workgroup's wait for its item always ends.
+// from a queue in chunk order.  384 threads and at most 168 registers, i.e. three wavefronts per SIMD.  Measured placement
+// (hardware ids recorded by every workgroup): a CU with a chain workgroup (two wavefronts on two of its SIMDs) takes no output
+// workgroup, whose six wavefronts would need the same SIMDs when it starts; every other CU holds two.  So 256 output
+// workgroups run beside the chain and the rest start as chain workgroups end, on the items still in the queue.  The chain
+// workgroups have the lowest indices, so they are resident before any output workgroup starts, and they wait for nothing:
+// an output workgroup's wait for its item always ends.
 template <bool NORM>
 __global__ __launch_bounds__(384, 3) void gdn_phase_b_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
                                                              float* st_out, _Float16* snap, bf16_t* y, const bf16_t* proj,
