@@ -112,7 +112,10 @@ int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_ne
  * and leave the per-chunk B operands in `snap`; others compute the outputs of a chunk from them: as a second launch up to 4095
  * tokens, from 4096 on in the same launch, as soon as the chain has published the chunk.  `snap`: qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned; its
  * first 33 KiB (qt_gdn_chunk_snap_bytes(0) bytes) are the progress words of the launch and MUST BE ZERO when a launch starts.  A launch leaves them zero, so
- * the caller zeroes them once; launches that use the same `snap` must not overlap.
+ * the caller zeroes them once; launches that use the same `snap` must not overlap.  (The one word a launch may leave set is
+ * the int32 at byte 32772: an output workgroup of the one-launch form that has polled for its chunk for about a second gives
+ * up, sets it to 1 and finishes on what is there, so that every launch ends.  It cannot happen while the chain workgroups run,
+ * and nothing reads the word back; a caller that wants the assurance checks it after synchronising and zeroes it again.)
  * qt_gdn_phase_b_norm is the same with prefill.gated_norm (qwen35/prefill.py:241-244) fused into the output kernel: it
  * writes out [S,2048] bf16 = gated RMSNorm of y with z = proj[:,6144:8192] and weight gw [128] f32 instead of y. */
 long qt_gdn_chunk_ops_bytes(int S);

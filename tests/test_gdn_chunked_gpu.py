@@ -150,6 +150,10 @@ def test_config2_long_prefill(qt, dev, T):
     for lo in range(0, T, 1024):                                              # no stretch of the sequence is worse than the bound
         check_rel(f"tokens {lo}.. output rel-L2", got[lo:lo + 1024], ref[lo:lo + 1024], 2e-3, rel_l2)
     check_equal("conv tail", to_np(conv4)[0], otail)
+    # the launches left their progress words, queue head and done count zero, and no output workgroup gave up its wait
+    flag_halves = qt._lib.lib().qt_gdn_chunk_snap_bytes(0) // 2
+    for snap in qt.gdn_nax._SNAP.values():
+        assert int(snap[:flag_halves].view(torch.int32).ne(0).sum().item()) == 0
     print(f"T={T}: state L2 {e1:.2e} max {e2:.2e}, out {e3:.2e}")
 
 
