@@ -422,6 +422,13 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             if (t + 1 < tb) tile(t + 1, std::integral_constant<int, 1>{});
         }
     }
+    // The lane's coordinates for the epilogue are taken again here, from the lane number the hardware counts: kept from the
+    // prologue they would live through the tile loop, in two registers more than the wavefront has (the kernel then spills
+    // them, and a kernel that uses scratch memory at all starts its wavefronts more slowly).
+    int zero = 0;
+    asm volatile("" : "+v"(zero));                               // (keeps the count below the loop)
+    const int lane_e = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));
+    const int n_e = lane_e & 15, g_e = lane_e >> 4, my_last_e = q_pos0 + r0 + n_e;
     if (nparts > 1) {
         // One part of several: leave O, m, l of this wavefront's heads as they are.  A row that sees no key of this part (its
         // last key lies before the part's first) has exponentiated masked scores against a masked maximum: it is written as
@@ -434,26 +441,26 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             float* pml = part_ml + (slot * 4 + hq) * (2 * RB);
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const int lr = lr0 + 4 * g + r;
+                const int lr = lr0 + 4 * g_e + r;
                 const bool seen = q_pos0 + rb * RB + lr >= first_key;
                 const float inv = seen ? 1.0f / Lsum[hh][r] : 0.f;
 #pragma unroll
-                for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n] = (_Float16)(seen ? O[hh][j][r] * inv : 0.f);
-                if (n == 0) pml[RB + lr] = seen ? Lsum[hh][r] : 0.f;
+                for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n_e] = (_Float16)(seen ? O[hh][j][r] * inv : 0.f);
+                if (n_e == 0) pml[RB + lr] = seen ? Lsum[hh][r] : 0.f;
             }
-            if (g == 0) pml[lr0 + n] = my_last >= first_key ? m_run[hh] : NEG;
+            if (g_e == 0) pml[lr0 + n_e] = my_last_e >= first_key ? m_run[hh] : NEG;
         }
         return;
     }
-    // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n, and of the row sums (any column)
+    // ---- normalise and store: lane (n_e, g_e) holds rows 4g .. 4g+3 of column 16 j + n_e, and of the row sums (any column)
 #pragma unroll
     for (int hh = 0; hh < NH; hh++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int orow = r0 + 4 * g + r;
+            const int orow = r0 + 4 * g_e + r;
             if (orow < S) {
                 const float inv = 1.0f / Lsum[hh][r];
-                bf16_t* dst = out + (size_t)(h0 + hh) * q_head_stride + (size_t)orow * AD + n;
+                bf16_t* dst = out + (size_t)(h0 + hh) * q_head_stride + (size_t)orow * AD + n_e;
 #pragma unroll
                 for (int j = 0; j < 16; j++) dst[16 * j] = f2bf(O[hh][j][r] * inv);
             }
