@@ -109,8 +109,8 @@ int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_ne
  * Intermediate operands are half precision (fp16: 11 significant bits, largest finite value 65504): conv outputs |v| and
  * states |S| beyond that are not representable and are not supported; values below 6e-5 lose precision gracefully.
  * Phase B: state_in / state_out [16,128,128] f32, y [S,16,128] bf16.  128 workgroups run the serial state chain over the chunks
- * and leave the per-chunk B operands in `snap`; others compute the outputs of a chunk from them: as a second launch up to 4095
- * tokens, from 4096 on in the same launch, as soon as the chain has published the chunk.  `snap`: qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned; its
+ * and leave the per-chunk B operands in `snap`; others compute the outputs of a chunk from them: as a second launch up to 63
+ * chunks (4032 tokens), from 64 chunks on in the same launch, as soon as the chain has published the chunk.  `snap`: qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned; its
  * first 33 KiB (qt_gdn_chunk_snap_bytes(0) bytes) are the progress words of the launch and MUST BE ZERO when a launch starts.  A launch leaves them zero, so
  * the caller zeroes them once; launches that use the same `snap` must not overlap.  (The one word a launch may leave set is
  * the int32 at byte 32772: an output workgroup of the one-launch form that has polled for its chunk for about a second gives

@@ -125,11 +125,12 @@ def test_config2_chunked_prefill(qt, dev, T):
     check_equal("gdn_core conv tail", to_np(conv4)[0], otail)
 
 
-@pytest.mark.parametrize("T", [8192, 8131, 4100])
+@pytest.mark.parametrize("T", [8192, 8131, 4100, 4033, 4032])
 def test_config2_long_prefill(qt, dev, T):
     """config 2's longest sweep point (T = 8192: a chain of 128 chunks, each step rounding its operands to half precision), the
-    same with a partial last chunk, and 65 chunks (the output units of the one-launch form of phase B, which these lengths
-    take, then run different numbers of rounds), from a nonzero state, through the layer core (reference entry
+    same with a partial last chunk, 65 chunks (the output units of the one-launch form of phase B, which these lengths
+    take, then run different numbers of rounds), and the two lengths either side of the switch between the forms (64 chunks,
+    the last one of a single token: one launch; 63 chunks: two), from a nonzero state, through the layer core (reference entry
     qwen35/gdn_nax.py:413-426).  Run twice on the same buffers: the second launch finds the progress words the first one left.
     The per-head errors are checked too: a head whose state decays fast must not hide behind the slow ones."""
     proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(2002 + T, T)
