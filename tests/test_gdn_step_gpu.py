@@ -171,7 +171,7 @@ def _solo(qt, dev, proj, cs, cw, A_log, dtb, ss, sel, **kw):
                                to_dev(dtb, dev), to_dev(ss, dev), torch.tensor([sel], dtype=torch.int32, device=dev), **kw)
 
 
-@pytest.mark.parametrize("M", [1, 3, 4])
+@pytest.mark.parametrize("M", [1, 3, 4, 8, 16])                             # (16: the most the entry point takes)
 def test_deltanet_solo_vs_oracle_and_chaining(qt, dev, M):
     gen = torch.Generator().manual_seed(300 + M)
     cw, A_log, dtb, gw = layer_params(6)
@@ -305,8 +305,9 @@ def test_deltanet_b_out_of_range_slot_is_skipped(qt, dev):
 
 
 def test_deltanet_bm_layout_of_reference_test(qt, dev):
-    """reference tests/batch_spec.py:40-67: 4 sequences, ragged entries / start snapshots / conv buffers, M = 3; and config 4's M = 4"""
-    for M, seed in ((3, 0), (4, 1004)):
+    """reference tests/batch_spec.py:40-67: 4 sequences, ragged entries / start snapshots / conv buffers, M = 3; config 4's M = 4;
+    and M = 8, beyond what the reference's scheduler drafts"""
+    for M, seed in ((3, 0), (4, 1004), (8, 1008)):
         rng = np.random.default_rng(seed)
         cw, A_log, dtb, gw = layer_params(11)
         NS, B = 6, 4
