@@ -89,14 +89,16 @@ def test_attn_b_out_of_range_rows_are_skipped(qt, dev):
         qt.batch.attn_b(q, kn, kn, Kp, Vp, torch.tensor([0], dtype=torch.int32, device=dev), torch.tensor([0], dtype=torch.int32, device=dev), M=5)
 
 
-@pytest.mark.parametrize("B,M", [(64, 1), (64, 4), (40, 1), (40, 3), (130, 2)])
-def test_attn_b_many_sequences(qt, dev, B, M):
+@pytest.mark.parametrize("B,M,Lmax", [(64, 1, 640), (64, 4, 640), (40, 1, 640), (40, 3, 640), (130, 2, 640), (300, 4, 200),
+                                      (1024, 1, 96)])
+def test_attn_b_many_sequences(qt, dev, B, M, Lmax):
     """more (sequence, KV head) segments than one 64-lane scan step of the segment table holds (B > 32), many segments per
-    workgroup, and more segments than workgroups' worth of tiles: ragged positions including 0, 1 and the last position that
-    fits, a few rows with an out-of-range slot or a full sequence (skipped: their outputs are not defined and not compared),
-    every other row against the oracle row by row, the pools bit-exact outside the appended rows"""
+    workgroup, and more segments than workgroups' worth of tiles, up to the 1024 sequences (2048 segments) the entry point
+    takes: ragged positions including 0, 1 and the last position that fits, a few rows with an out-of-range slot or a full
+    sequence (skipped: their outputs are not defined and not compared), every other row against the oracle row by row, the
+    pools bit-exact outside the appended rows"""
     rng = np.random.default_rng(100 * B + M)
-    S, Lmax = B + 3, 640
+    S = B + 3
     slots = rng.permutation(S)[:B].astype(np.int32)
     pos = rng.integers(0, Lmax - M, B).astype(np.int32)
     pos[:6] = [0, 1, Lmax - M, 15, 16, 17]
