@@ -52,7 +52,9 @@ def _close(name, got, want, ulps, inner=None):
     # wide outputs with K = 1024: rows in LDS from 4 to 64 rows (every count of 16-row blocks, partial blocks, feature counts
     # that leave the last workgroup partly or wholly past N); more than 64 rows keep the rows in registers
     (4, 8224, 1024, "none"), (17, 4096, 1024, "add"), (33, 7168, 1024, "swiglu"), (48, 4100, 1024, "none"), (63, 5120, 1024, "add"),
-    (100, 8224, 1024, "none"), (3, 8224, 1024, "none")])
+    (100, 8224, 1024, "none"), (3, 8224, 1024, "none"),
+    # ... with each epilogue, and more row blocks than one pass of 64 rows
+    (100, 4096, 1024, "add"), (70, 7168, 1024, "swiglu"), (200, 5120, 1024, "none")])
 def test_fused_gemv_vs_oracle(qt, dev, M, N, K, epi):
     g = torch.Generator().manual_seed(M * 7 + N * 3 + K)
     W = rand_bf(g, (N, K), K ** -0.5)
