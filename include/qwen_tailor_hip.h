@@ -8,7 +8,9 @@
  * Conventions: every pointer is a device pointer unless said otherwise; bf16 tensors are passed as raw 16-bit words
  * (const void*), state is float; tensors are contiguous in the layouts of the reference; index arrays are int32 on the
  * device; `stream` is a hipStream_t (passed as void* so that this header needs no HIP include).  No entry point
- * allocates, synchronises or keeps global state; all work is enqueued on `stream`.  Return value: 0 on success, or
+ * allocates or synchronises; all work is enqueued on `stream`.  What the library keeps per process: the CU count of each
+ * device (asked once, cached), the static scratch array of qt_gqa_attn_decode_static with its per-device address, and the
+ * poll limit set by qt_gdn_phase_b_poll_limit.  Return value: 0 on success, or
  *   -1 bad dimension, -2 misaligned pointer, -3 null pointer, -4 unsupported shape, -5 launch failure,
  *   -6 workspace too small, -7 size beyond the maximum of the allocation-free entry point.
  * Rows whose slot index lies outside the pool (or whose position would overflow it) are skipped by the kernels: nothing
@@ -75,14 +77,16 @@ int qt_gdn_conv_prep(const void* proj, const void* conv_state, const void* conv_
 int qt_gated_rmsnorm(const void* y, const void* proj, const float* gw, void* out, long rows, float eps, qt_stream_t stream);
 
 /* gated_delta_update's recurrence kernel (qwen35/gated_delta.py:143-174) with g (f32) and beta (bf16) [B,T,Hv] given:
- * q, k [B,T,Hk,128], v, y [B,T,Hv,Dv] bf16, state [B,Hv,Dv,128] f32.  Dk must be 128 and Dv a multiple of 16, otherwise -4
- * (the reference raises ValueError, gated_delta.py:164-166). */
+ * q, k [B,T,Hk,128], v, y [B,T,Hv,Dv] bf16, state [B,Hv,Dv,128] f32.  Dk must be 128 and Dv a multiple of 8, otherwise -4
+ * (where the reference raises ValueError, gated_delta.py:164-166). */
 int qt_gdn_recurrent(const void* q, const void* k, const void* v, const float* g, const void* beta, const float* state_in,
                      float* state_out, void* y, int B, int T, int Hk, int Hv, int Dk, int Dv, qt_stream_t stream);
 
 /* batch.attn_b (qwen35/batch.py:230-237): ragged decode / verify attention, 8 query heads on 2 KV heads, head dim 256.
  * q [B*M,8,256], k_new / v_new [B*M,2,256], pools Kp / Vp [n_slots,2,Lmax,256] bf16 (rows pos[b]..pos[b]+M-1 are appended),
- * out [B*M,8,256].  1 <= M <= 4, B <= 1024.  The batch's 16-key tiles are spread evenly over one workgroup per CU (split-K
+ * out [B*M,8,256].  1 <= M <= 16 (the limit of qt_gdn_verify_step; the reference kernel is generic in M), B <= 1024.  Up to
+ * four tokens per sequence share one pass over the pool; more run as passes of four (rows 4p .. 4p+3 at pos[b] + 4p), each a
+ * pair of launches.  The batch's 16-key tiles are spread evenly over one workgroup per CU (split-K
  * over a flat tile space, so ragged lengths balance); CH = smallest number of pool keys one workgroup takes (multiple of 16).
  * Workspace of at least qt_gqa_attn_workspace_bytes(B, M, Lmax, CH) bytes, 16-byte aligned, owned by the caller. */
 long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH);
@@ -111,17 +115,25 @@ int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_ne
  * Phase B: state_in / state_out [16,128,128] f32, y [S,16,128] bf16.  128 workgroups run the serial state chain over the chunks
  * and leave the per-chunk B operands in `snap`; others compute the outputs of a chunk from them: as a second launch up to 63
  * chunks (4032 tokens), from 64 chunks on in the same launch, as soon as the chain has published the chunk.  `snap`: qt_gdn_chunk_snap_bytes(S) bytes, caller-owned, 16-byte aligned; its
- * first 33 KiB (qt_gdn_chunk_snap_bytes(0) bytes) are the progress words of the launch and MUST BE ZERO when a launch starts.  A launch leaves them zero, so
- * the caller zeroes them once; launches that use the same `snap` must not overlap.  (The one word a launch may leave set is
- * the int32 at byte 32772: an output workgroup of the one-launch form that has polled for its chunk for about a second gives
- * up, sets it to 1 and finishes on what is there, so that every launch ends.  It cannot happen while the chain workgroups run,
- * and nothing reads the word back; a caller that wants the assurance checks it after synchronising and zeroes it again.)
+ * first 33 KiB (qt_gdn_chunk_snap_bytes(0) bytes) are the flag area of the launch and MUST BE ZERO when a launch starts (memory that
+ * was merely allocated will not do: the one-launch form reads its queue head and progress words from it).  A launch leaves
+ * them zero, so the caller zeroes them once; launches that use the same `snap` must not overlap.  The one word a launch may
+ * leave set is the STATUS WORD, the int32 at byte qt_gdn_chunk_status_offset() (32772) of `snap`; no launch clears it, the
+ * caller reads it after (or asynchronously behind) the launch and resets it:
+ *   bit 0: an output workgroup of the one-launch form polled for its chunk longer than the poll limit (about a second) and
+ *          gave up; its rows of y were NOT written.  It cannot happen while the chain workgroups run undisturbed.
+ *   bit 1: the final state holds a value that is not finite: an operand left the half-precision range (above) and y is not
+ *          to be trusted either.
+ * qt_gdn_phase_b_poll_limit(polls) sets the poll limit of later launches (0 = the default); it exists so that the give-up
+ * path can be exercised from the host with a tiny limit.
  * qt_gdn_phase_b_norm is the same with prefill.gated_norm (qwen35/prefill.py:241-244) fused into the output kernel: it
  * writes out [S,2048] bf16 = gated RMSNorm of y with z = proj[:,6144:8192] and weight gw [128] f32 instead of y. */
 long qt_gdn_chunk_ops_bytes(int S);
 long qt_gdn_chunk_u_bytes(int S);
 long qt_gdn_chunk_gc_bytes(int S);
 long qt_gdn_chunk_snap_bytes(int S);
+long qt_gdn_chunk_status_offset(void);
+int qt_gdn_phase_b_poll_limit(int polls);
 int qt_gdn_phase_a(const void* proj, const void* q, const void* k, const void* v, const float* A_log, const float* dt_bias,
                    void* ops, void* U, float* gC, int S, qt_stream_t stream);
 /* qt_gdn_phase_a with qt_gdn_conv_prep fused in (the reference's fused prep kernel, qwen35/gdn_nax.py:394-401 prep_a, with the

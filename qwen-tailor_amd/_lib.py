@@ -30,6 +30,7 @@ _SIGS = {
     "qt_gqa_attn_decode": [_vp] * 9 + [_l, _i, _i, _i, _i, _i, _vp],
     "qt_gqa_attn_decode_static": [_vp] * 8 + [_i, _i, _i, _i, _i, _vp],
     "qt_gdn_phase_b": [_vp] * 7 + [_i, _vp],
+    "qt_gdn_phase_b_poll_limit": [_i],
     "qt_gdn_phase_b_norm": [_vp] * 8 + [_f, _vp, _i, _vp],
     "qt_gqa_prefill_causal": [_vp] * 5 + [_l, _i, _i, _i, _l, _l, _vp],
     "qt_gdn_phase_a": [_vp] * 9 + [_i, _vp],
@@ -55,6 +56,7 @@ def lib():
             fn = getattr(L, name)
             fn.argtypes, fn.restype = args, ctypes.c_int
         L.qt_gqa_attn_workspace_bytes.argtypes, L.qt_gqa_attn_workspace_bytes.restype = [_i] * 4, ctypes.c_long
+        L.qt_gdn_chunk_status_offset.argtypes, L.qt_gdn_chunk_status_offset.restype = [], ctypes.c_long
         for name in ("qt_gdn_chunk_ops_bytes", "qt_gdn_chunk_u_bytes", "qt_gdn_chunk_gc_bytes", "qt_gdn_chunk_snap_bytes",
                      "qt_gqa_prefill_workspace_bytes"):
             getattr(L, name).argtypes, getattr(L, name).restype = [_i], ctypes.c_long
@@ -92,6 +94,24 @@ def silu_table(dev):
 
 def stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+_WORKSPACES = {}         # (purpose, device index, stream handle) -> uint8 tensor
+_RETIRED = []            # outgrown buffers: kept for the life of the process, a captured HIP graph may still hold their address
+
+
+def workspace(purpose, dev, nbytes, first_bytes=0):
+    """Scratch memory for a kernel's partial results (the C ABI never allocates): one uint8 buffer per (purpose, device, stream),
+    because launches on different streams may overlap.  A buffer that is outgrown is replaced but never freed: a HIP graph
+    captured earlier replays with the old address.  first_bytes: size of the first allocation, so that growth is rare."""
+    key = (purpose, dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    buf = _WORKSPACES.get(key)
+    if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _RETIRED.append(buf)
+        buf = torch.empty(max(nbytes, first_bytes), dtype=torch.uint8, device=dev)
+        _WORKSPACES[key] = buf
+    return buf
 
 
 def ptr(t):

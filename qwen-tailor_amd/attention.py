@@ -34,7 +34,7 @@ def scaled_dot_product_attention(q, k, v, *, scale: float, mask="causal"):
     out = torch.empty_like(q)
     # launches that would leave half of the CUs idle are split along the keys; their parts meet in a workspace
     nws = L.lib().qt_gqa_prefill_workspace_bytes_for(S, Lk, Lk - S)
-    ws = torch.empty(nws, dtype=torch.uint8, device=q.device) if nws > 0 else None
+    ws = L.workspace("prefill_attention", q.device, nws) if nws > 0 else None      # cached per (device, stream)
     L.call("qt_gqa_prefill_causal", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(ws), max(nws, 0),
            S, Lk, Lk - S, S * 256, k.stride(1), L.stream())
     return out

@@ -35,23 +35,13 @@ def deltanet_b(proj, conv_pool, conv_w, A_log, dt_bias, ssm_pool, slots, pos, ro
     return y
 
 
-_WORKSPACE = {}          # (device index, stream handle) -> uint8 tensor
-_RETIRED = []            # outgrown buffers: kept for the life of the process, a captured HIP graph may still hold their address
-_WS_MIN = 32 << 20       # first allocation: enough for 256 sequences x 4 rows, so that growth is rare
+_WS_MIN = 32 << 20       # first allocation of the attention scratch: enough for 256 sequences x 4 rows, so that growth is rare
 
 
 def _workspace(dev, nbytes):
-    """Split-K scratch of the attention kernel (the C ABI never allocates): one buffer per (device, stream), because launches
-    on different streams may overlap.  A buffer that is outgrown is replaced but never freed: a HIP graph captured earlier
-    replays with the old address.  Callers that manage memory themselves pass `workspace=` to attn_b instead."""
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
-    buf = _WORKSPACE.get(key)
-    if buf is None or buf.numel() < nbytes:
-        if buf is not None:
-            _RETIRED.append(buf)
-        buf = torch.empty(max(nbytes, _WS_MIN), dtype=torch.uint8, device=dev)
-        _WORKSPACE[key] = buf
-    return buf
+    """Split-K scratch of the attention kernel, cached per (device, stream) (see _lib.workspace).  Callers that manage memory
+    themselves pass `workspace=` to attn_b instead."""
+    return L.workspace("attn_b", dev, nbytes, _WS_MIN)
 
 
 def deltanet_b_gnorm(proj, conv_pool, conv_w, A_log, dt_bias, ssm_pool, slots, pos, gw, eps=1e-6):
@@ -81,12 +71,13 @@ def split_size(Lmax: int, B: int = 16) -> int:
 def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None, workspace=None):
     """q [R,H,D], k / v [R,KV,D] (normed + roped), pools [S+1,KV,Lmax,D]; R = B*M rows (row b*M+j = position pos[b]+j of slot
     slots[b]; slots / pos int32 [B]).  Returns o [R,H,D] bf16 and appends k / v at pos[b]+j (in place)
-    (qwen35/batch.py:230-237).  workspace: optional uint8 device tensor of at least qt_gqa_attn_workspace_bytes(B, M, Lmax, split)
+    (qwen35/batch.py:230-237).  M up to 16 (the limit of batch_spec.deltanet_bm); more than four tokens per sequence run as
+    passes of four, each reading the pool once.  workspace: optional uint8 device tensor of at least qt_gqa_attn_workspace_bytes(B, M, Lmax, split)
     bytes for the split-K partial results (default: a buffer cached per device and stream)."""
     q = L.dev(q, BF16, "q", (None, 8, 256))
     R = q.shape[0]
-    if M < 1 or M > 4 or R % M:
-        raise ValueError(f"attn_b: M = {M} (1..4) must divide the number of rows ({R})")
+    if M < 1 or M > 16 or R % M:
+        raise ValueError(f"attn_b: M = {M} (1..16, as deltanet_bm) must divide the number of rows ({R})")
     B = R // M
     k, v = L.dev(k, BF16, "k", (R, 2, 256)), L.dev(v, BF16, "v", (R, 2, 256))
     Kp = L.dev(Kp, BF16, "Kp", (None, 2, None, 256))

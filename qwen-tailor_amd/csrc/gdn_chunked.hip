@@ -62,8 +62,12 @@ __device__ __forceinline__ half8 pack_half8(const f32x4& a, const f32x4& b) {
 // in flight (stores of one wavefront complete in order).  The chain workgroups have the lowest indices, so all of them are
 // running before the first output workgroup starts, and they wait for nothing: a consumer's producer is always running,
 // whether or not every output workgroup is resident.  A consumer that does not see its snapshot within SPIN_LIMIT polls
-// gives up, sets the error word and computes on what is there, so that every wavefront ends.  The last output workgroup to finish clears the progress words: the flag area is zero before and after every launch
-// (the caller zeroes it once).
+// gives up: it sets bit 0 of the status word and leaves the item's output rows unwritten, so that every wavefront ends.
+// Every workgroup of either role counts itself done when it has made its last store to the flag area (a chain workgroup
+// after its final progress store has been acknowledged), and the last one to do so clears the progress words, the done
+// count and the queue head: they are zero before and after every launch (the caller zeroes them once).  The status word
+// is never cleared by a launch: it is the caller's to read and reset.  Bit 1 of it is set by a chain workgroup whose final
+// state slice holds a value that is not finite: a half-precision operand (the state, D, U or a conv output) has overflowed.
 //
 // Chain role: 5 wavefronts per (head, 16-wide dv slice).  MFMA wavefront w owns rows 16w..16w+15 of D (the chunk's tokens) and
 // rows 32w..32w+31 of S^T (dk): per chunk it pulls only its 8 operand tiles (8 KiB) and keeps PB_DEP chunks of them in flight
@@ -82,7 +86,8 @@ constexpr int PF_SLOTS = 8;                      // prefetch loads in flight
 constexpr int PUB_LAG = 8;                       // a chunk is published when at most this many newer chunks' stores are in flight
 constexpr int FLAG_STRIDE = 64;                  // ints between progress words: every word has a 256-byte stretch of its own
 constexpr int FLAG_WORDS = (N_CHAIN + 1) * FLAG_STRIDE;   // flag area at the head of `snap` (33 KiB): progress [128] | done count, error
-constexpr int FLAG_DONE = N_CHAIN * FLAG_STRIDE, FLAG_ERR = FLAG_DONE + 1, FLAG_NEXT = FLAG_DONE + 2;   // FLAG_NEXT: head of the item queue
+constexpr int FLAG_DONE = N_CHAIN * FLAG_STRIDE, FLAG_ERR = FLAG_DONE + 1, FLAG_NEXT = FLAG_DONE + 2;   // FLAG_ERR: the status word; FLAG_NEXT: head of the item queue
+constexpr int ERR_GAVE_UP = 1, ERR_NOT_FINITE = 2;
 constexpr int FLAG_HALVES = FLAG_WORDS * 2;
 constexpr int SPIN_LIMIT = 1 << 21;              // polls (about a second) before a consumer gives up
 constexpr int MAX_OUT_WGS = 512;                 // output workgroups of the one-launch form: two for every CU (measured: 384 +2 us, 640 +4 us at 8192 tokens)
@@ -113,6 +118,15 @@ __device__ __forceinline__ half8 load_coherent(const _Float16* p) {
 template <bool COHERENT>
 __device__ __forceinline__ half8 load_snap(const _Float16* p) {
     return COHERENT ? load_coherent(p) : *reinterpret_cast<const half8*>(p);
+}
+
+// the last workgroup of a one-launch phase B leaves the progress words, the done count and the queue head zero (not the status word)
+__device__ __forceinline__ void clear_flags(int* flags, int tid, int nthreads) {
+    for (int i = tid; i < N_CHAIN; i += nthreads) __hip_atomic_store(flags + i * FLAG_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) {
+        __hip_atomic_store(flags + FLAG_DONE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(flags + FLAG_NEXT, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 struct ChainLds {
@@ -164,6 +178,10 @@ __device__ __forceinline__ void chain_role(ChainLds& L, int blk, const _Float16*
         if (PUBLISH) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (lane == 0) __hip_atomic_store(flag, NC, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                    // the progress store is acknowledged before this workgroup counts as done
+            int last = 0;
+            if (lane == 0) last = atomicAdd(flags + FLAG_DONE, 1) == (int)gridDim.x - 1;
+            if (__builtin_amdgcn_readfirstlane(last)) clear_flags(flags, lane, 64);
         }
         return;
     }
@@ -323,6 +341,11 @@ __device__ __forceinline__ void chain_role(ChainLds& L, int blk, const _Float16*
         float* sp = st_out + ((size_t)h * DV + sl * 16 + n) * DK + w * 32 + 4 * g;
         *reinterpret_cast<f32x4*>(sp) = ST[0];
         *reinterpret_cast<f32x4*>(sp + 16) = ST[1];
+        // an overflow of a half-precision operand anywhere in the chain (state, D, U, conv outputs) ends here as inf or NaN
+        bool bad = false;
+#pragma unroll
+        for (int i = 0; i < 4; i++) bad |= !(fabsf(ST[0][i]) <= 3.0e38f) | !(fabsf(ST[1][i]) <= 3.0e38f);
+        if (__any(bad) && lane == 0) atomicOr(flags + FLAG_ERR, ERR_NOT_FINITE);
     }
 }
 
@@ -400,7 +423,7 @@ __device__ __forceinline__ void gated_norm_tile(lds_bf16_ptr ys, int tid, int c,
 // gated RMSNorm (same arithmetic as the stand-alone kernel: 16 lanes per row, 8 columns each; batch.py:338-343).
 // With WAIT the item's snapshots come from a chain that runs in the same launch: `seq` counts the items of this workgroup.
 template <bool NORM, bool WAIT>
-__device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int seq, int c, int h, const _Float16* __restrict__ ops,
+__device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int seq, int spin_limit, int c, int h, const _Float16* __restrict__ ops,
                                             const _Float16* snaps, int* flags, const float* __restrict__ gates,
                                             bf16_t* __restrict__ y, const bf16_t* __restrict__ proj, const float* __restrict__ gw,
                                             float eps, int S) {
@@ -422,25 +445,33 @@ __device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int
             // wait until the chain has published chunk c for all eight slices of the head: the unit's first wavefront polls (lanes
             // 0..7, one progress word each, about once a microsecond: thousands of pollers on one memory line would hold up the
             // chain's own progress stores) and passes the news on through LDS, where the other three wavefronts wait
+            // `ready` = 2 * (items this workgroup has been let into) + (1 if the last one was given up)
             if (!WAIT) {
             } else if (w == 0) {
                 const int* fp = flags + (h * 8 + (lane & 7)) * FLAG_STRIDE;
                 int spins = 0;
+                bool gave_up = false;
                 while (true) {
                     int v = c + 1;
                     if (lane < 8) v = __hip_atomic_load(fp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     asm volatile("" ::: "memory");                              // the snapshot loads stay behind the poll
                     if (__all(v > c)) break;
-                    if (++spins > SPIN_LIMIT) {
-                        if (lane == 0) __hip_atomic_store(flags + FLAG_ERR, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (++spins > spin_limit) {
+                        gave_up = true;
                         break;
                     }
                     __builtin_amdgcn_s_sleep(32);
                 }
-                if (lane == 0) *ready = seq + 1;
+                if (lane == 0) {
+                    if (gave_up) atomicOr(flags + FLAG_ERR, ERR_GAVE_UP);
+                    *ready = 2 * (seq + 1) + (gave_up ? 1 : 0);
+                }
+                if (gave_up) return;                                            // (all four wavefronts leave here: no barrier is skipped by some only)
             } else {
-                while (*ready <= seq) __builtin_amdgcn_s_sleep(2);
+                int rv;
+                while (((rv = *ready) >> 1) <= seq) __builtin_amdgcn_s_sleep(2);
                 asm volatile("" ::: "memory");
+                if (rv & 1) return;                                             // given up: the item's rows stay unwritten
             }
             const _Float16* sp = snaps + (rec * 8 + 2 * w) * SNAP_HALVES + lane * 8;
 #pragma unroll
@@ -497,7 +528,7 @@ __device__ __forceinline__ void output_item(bf16_t* ys, volatile int* ready, int
 __global__ __launch_bounds__(384) void gdn_chain_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
                                                         float* st_out, _Float16* snap, int NC) {
     __shared__ ChainLds chain_lds;
-    chain_role<false, 4>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snap + FLAG_HALVES, nullptr, NC);
+    chain_role<false, 4>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snap + FLAG_HALVES, reinterpret_cast<int*>(snap), NC);
 }
 template <bool NORM>
 __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restrict__ ops, const _Float16* __restrict__ snap,
@@ -505,7 +536,7 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
                                                          const bf16_t* __restrict__ proj, const float* __restrict__ gw, float eps,
                                                          int S, int NC) {
     __shared__ __align__(16) bf16_t ys[C * YS_LD];
-    output_item<NORM, false>(ys, nullptr, 0, blockIdx.x / HV, blockIdx.x % HV, ops, snap + FLAG_HALVES, nullptr, gates, y, proj, gw, eps, S);
+    output_item<NORM, false>(ys, nullptr, 0, 0, blockIdx.x / HV, blockIdx.x % HV, ops, snap + FLAG_HALVES, nullptr, gates, y, proj, gw, eps, S);
 }
 
 // the one-launch form: N_CHAIN chain workgroups, then output workgroups (4 wavefronts at work) that take (chunk, head) items
@@ -518,7 +549,7 @@ __global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restr
 template <bool NORM>
 __global__ __launch_bounds__(384, 3) void gdn_phase_b_kernel(const _Float16* ops, const _Float16* U, const float* gates, const float* st_in,
                                                              float* st_out, _Float16* snap, bf16_t* y, const bf16_t* proj,
-                                                             const float* gw, float eps, int S, int NC) {
+                                                             const float* gw, float eps, int S, int NC, int spin_limit) {
     __shared__ ChainLds chain_lds;
     __shared__ __align__(16) bf16_t ys[C * YS_LD];
     __shared__ int ready, item_s, last;
@@ -536,19 +567,13 @@ __global__ __launch_bounds__(384, 3) void gdn_phase_b_kernel(const _Float16* ops
         __syncthreads();
         const int item = item_s;
         if (item >= total) break;
-        output_item<NORM, true>(ys, &ready, seq, item / HV, item % HV, ops, snaps, flags, gates, y, proj, gw, eps, S);
+        output_item<NORM, true>(ys, &ready, seq, spin_limit, item / HV, item % HV, ops, snaps, flags, gates, y, proj, gw, eps, S);
     }
-    // the last output workgroup to finish leaves the flag area zero for the next launch: by then every item has been
-    // taken and computed, so every chain workgroup has made its last store to it
-    if (threadIdx.x == 0) last = atomicAdd(flags + FLAG_DONE, 1) == (int)gridDim.x - N_CHAIN - 1;
+    // a workgroup counts itself done when it has taken its last item; the last workgroup of the launch (of either role)
+    // leaves the flag area zero for the next launch
+    if (threadIdx.x == 0) last = atomicAdd(flags + FLAG_DONE, 1) == (int)gridDim.x - 1;
     __syncthreads();
-    if (last) {
-        if (threadIdx.x < N_CHAIN) __hip_atomic_store(flags + threadIdx.x * FLAG_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (threadIdx.x == 0) {
-            __hip_atomic_store(flags + FLAG_DONE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(flags + FLAG_NEXT, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+    if (last) clear_flags(flags, threadIdx.x, 256);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -1033,6 +1058,9 @@ long qt_gdn_chunk_ops_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C)
 long qt_gdn_chunk_u_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * U_HALVES * 2; }
 long qt_gdn_chunk_gc_bytes(int S) { return S < 0 ? -1 : (long)((S + C - 1) / C) * HV * GATE_FLOATS * 4; }
 
+// polls before an output workgroup of the one-launch form gives up on its chunk (0 = the default, about a second)
+static std::atomic<int> poll_limit{0};
+
 static int phase_b_launch(const void* ops, const void* U, const float* gC, void* snap, const float* state_in, float* state_out,
                           void* y, const void* proj, const float* gw, float eps, bool norm, int S, hipStream_t stream) {
     if (!ops || !U || !gC || !snap || !state_in || !state_out || !y) return QT_ERR_NULL;
@@ -1049,12 +1077,13 @@ static int phase_b_launch(const void* ops, const void* U, const float* gC, void*
     }
     if (NC >= FUSED_MIN_CHUNKS) {
         const dim3 grid(N_CHAIN + min(MAX_OUT_WGS, NC * HV)), block(384);
+        const int pl = poll_limit.load(std::memory_order_relaxed), spin = pl > 0 ? pl : SPIN_LIMIT;
         if (norm)
             hipLaunchKernelGGL(gdn_phase_b_kernel<true>, grid, block, 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
-                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S, NC);
+                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)proj, gw, eps, S, NC, spin);
         else
             hipLaunchKernelGGL(gdn_phase_b_kernel<false>, grid, block, 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
-                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S, NC);
+                               state_out, (_Float16*)snap, (bf16_t*)y, (const bf16_t*)nullptr, (const float*)nullptr, 0.f, S, NC, spin);
     } else {
         hipLaunchKernelGGL(gdn_chain_kernel, dim3(N_CHAIN), dim3(384), 0, stream, (const _Float16*)ops, (const _Float16*)U, gC, state_in,
                            state_out, (_Float16*)snap, NC);
@@ -1069,6 +1098,13 @@ static int phase_b_launch(const void* ops, const void* U, const float* gC, void*
     QT_CHECK_LAUNCH();
     return QT_OK;
 }
+
+int qt_gdn_phase_b_poll_limit(int polls) {
+    if (polls < 0) return QT_ERR_DIM;
+    poll_limit.store(polls, std::memory_order_relaxed);
+    return QT_OK;
+}
+long qt_gdn_chunk_status_offset(void) { return (long)FLAG_ERR * 4; }
 
 long qt_gdn_chunk_snap_bytes(int S) { return S < 0 ? -1 : (long)FLAG_WORDS * 4 + (long)((S + C - 1) / C) * HV * 8 * SNAP_HALVES * 2; }
 

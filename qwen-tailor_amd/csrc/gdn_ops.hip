@@ -143,16 +143,19 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(const bf16_t* __restric
 // gated_delta_update's kernel (qwen35/gated_delta.py:33-137): T sequential tokens with q, k, v, g, beta given.
 // One workgroup of 256 threads per (batch, value head, 16-row block); a 16-lane group owns one value row, a lane 8 of its
 // 128 columns; no LDS, no barriers.  q, k [B,T,Hk,128], v, y [B,T,Hv,Dv], g f32 / beta bf16 [B,T,Hv], state [B,Hv,Dv,128].
+// Dv is a multiple of 8 (gated_delta.py:164-166): the last block of a Dv that is no multiple of 16 has eight idle row groups,
+// which work on a copy of the last row and store nothing.
 __global__ __launch_bounds__(256) void recurrent_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                         const bf16_t* __restrict__ v, const float* __restrict__ g,
                                                         const bf16_t* __restrict__ beta, const float* st_in,
                                                         float* st_out, bf16_t* __restrict__ y, int T, int Hk, int Hv,
                                                         int Dv) {
-    const int nblk = Dv / 16;
+    const int nblk = (Dv + 15) / 16;
     const int blk = blockIdx.x % nblk, n = blockIdx.x / nblk;             // n = b*Hv + hv
     const int b = n / Hv, hv = n % Hv, hk = hv / (Hv / Hk);              // gated_delta.py:43-46
     const int tid = threadIdx.x, c = tid & 15;
-    const int row = blk * 16 + (tid >> 4);
+    const bool live = blk * 16 + (tid >> 4) < Dv;                         // whole 16-lane groups are live or idle together
+    const int row = min(blk * 16 + (tid >> 4), Dv - 1);
     const size_t so = ((size_t)n * Dv + row) * DK;
     float sv[8];
     {
@@ -172,7 +175,7 @@ __global__ __launch_bounds__(256) void recurrent_kernel(const bf16_t* __restrict
         const float k8[8] = {lo_bf(ka.x), hi_bf(ka.x), lo_bf(ka.y), hi_bf(ka.y), lo_bf(kb.x), hi_bf(kb.x), lo_bf(kb.y), hi_bf(kb.y)};
         const float kq = dot8_row16(k8, q8);
         const float yv = gdn_row_step(sv, k8, q8, bf2f(*vp), *gp, bf2f(*bp), kq);
-        if (c == 0) *yp = f2bf(yv);
+        if (c == 0 && live) *yp = f2bf(yv);
         qp += (size_t)Hk * DK;
         kp += (size_t)Hk * DK;
         vp += (size_t)Hv * Dv;
@@ -180,6 +183,7 @@ __global__ __launch_bounds__(256) void recurrent_kernel(const bf16_t* __restrict
         gp += Hv;
         bp += Hv;
     }
+    if (!live) return;
     reinterpret_cast<float4*>(st_out + so)[c] = make_float4(sv[0], sv[1], sv[2], sv[3]);
     reinterpret_cast<float4*>(st_out + so)[16 + c] = make_float4(sv[4], sv[5], sv[6], sv[7]);
 }
@@ -256,11 +260,11 @@ int qt_gated_rmsnorm(const void* y, const void* proj, const float* gw, void* out
 int qt_gdn_recurrent(const void* q, const void* k, const void* v, const float* g, const void* beta, const float* state_in,
                      float* state_out, void* y, int B, int T, int Hk, int Hv, int Dk, int Dv, hipStream_t stream) {
     if (!q || !k || !v || !g || !beta || !state_in || !state_out || !y) return QT_ERR_NULL;
-    if (Dk != DK || Dv <= 0 || Dv % 16 || Hk <= 0 || Hv <= 0 || Hv % Hk) return QT_ERR_UNSUPPORTED;   // gated_delta.py:164-166
+    if (Dk != DK || Dv <= 0 || Dv % 8 || Hk <= 0 || Hv <= 0 || Hv % Hk) return QT_ERR_UNSUPPORTED;   // gated_delta.py:164-166
     if (B < 0 || T < 0) return QT_ERR_DIM;
     if (B == 0) return QT_OK;
     if (!al(q, 8) || !al(k, 8) || !al(state_in, 16) || !al(state_out, 16)) return QT_ERR_ALIGN;
-    hipLaunchKernelGGL(recurrent_kernel, dim3((unsigned)(B * Hv * (Dv / 16))), dim3(256), 0, stream, (const bf16_t*)q,
+    hipLaunchKernelGGL(recurrent_kernel, dim3((unsigned)(B * Hv * ((Dv + 15) / 16))), dim3(256), 0, stream, (const bf16_t*)q,
                        (const bf16_t*)k, (const bf16_t*)v, g, (const bf16_t*)beta, state_in, state_out, (bf16_t*)y, T, Hk, Hv, Dv);
     QT_CHECK_LAUNCH();
     return QT_OK;

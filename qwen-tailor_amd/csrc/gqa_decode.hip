@@ -21,6 +21,9 @@
 // Each wavefront keeps its own online-softmax state (m, l, O); the 4 wavefronts of a workgroup are merged through LDS and
 // the workgroup writes one unnormalised partial (m, l, O) per row and segment; a second kernel merges the partials
 // (batch.py:203-221).
+// A kernel instance holds at most four query tokens per sequence (16 rows = one MFMA tile).  More tokens per sequence (M up
+// to 16) run as passes of up to four: pass j0 = 0, 4, 8, 12 takes rows j0 .. j0+3 of every sequence at position pos[b] + j0 and
+// finds the rows that the earlier passes appended among its pool keys (the passes are launches on one stream, in order).
 #include "qt_common.h"
 
 using namespace qt;
@@ -111,12 +114,12 @@ constexpr int VISIT_TILES = 5;
 // is out of range own no tiles (they are skipped by both kernels).  Every thread of the workgroup must call it.
 template <int M>
 __device__ __forceinline__ int build_segments(int* seg_start, const int* __restrict__ slots, const int* __restrict__ pos, int nseg,
-                                              int Lmax, int n_slots) {
+                                              int Lmax, int n_slots, int Mtot, int j0) {
     const int tid = threadIdx.x, lane = tid & 63;
     for (int sg = tid; sg < nseg; sg += 256) {
         const int b = sg / AKV, slot = slots[b], p0 = pos[b];
-        const bool ok = (unsigned)slot < (unsigned)n_slots && p0 >= 0 && p0 + M <= Lmax;
-        seg_start[sg + 1] = ok ? max(1, (p0 + 15) >> 4) + VISIT_TILES : 0;
+        const bool ok = (unsigned)slot < (unsigned)n_slots && p0 >= 0 && p0 + Mtot <= Lmax;    // all of the sequence's rows fit, or none is taken
+        seg_start[sg + 1] = ok ? max(1, (p0 + j0 + 15) >> 4) + VISIT_TILES : 0;
     }
     if (tid == 0) seg_start[0] = 0;
     __syncthreads();
@@ -147,7 +150,9 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
                                                            const bf16_t* __restrict__ v_new, bf16_t* Kp, bf16_t* Vp,
                                                            const int* __restrict__ slots, const int* __restrict__ pos,
                                                            float* __restrict__ part_o, float* __restrict__ part_ml,
-                                                           int* __restrict__ seg_tab, int B, int Lmax, int min_tiles, int n_slots) {
+                                                           int* __restrict__ seg_tab, int B, int Lmax, int min_tiles, int n_slots,
+                                                           int Mtot, int j0) {
+    // M = tokens of this pass (rows j0 .. j0 + M - 1 of each sequence's Mtot rows)
     constexpr int R = 4 * M;
     __shared__ int seg_start[MAX_SEG + 1];
     // one V tile and one K tile per wavefront, in one array: at the end the same memory holds the four wavefronts' scaled O
@@ -159,7 +164,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     float* const mo = reinterpret_cast<float*>(tile_s);
 
     const int nseg = B * AKV;
-    const int total = build_segments<M>(seg_start, slots, pos, nseg, Lmax, n_slots);
+    const int total = build_segments<M>(seg_start, slots, pos, nseg, Lmax, n_slots, Mtot, j0);
     if (blockIdx.x == 0)                                         // the merge kernel reads the table instead of building it again
         for (int i = threadIdx.x; i <= nseg; i += 256) seg_tab[i] = seg_start[i];
     const int per = tiles_per_wg(total, gridDim.x, min_tiles);
@@ -178,7 +183,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     const int ss = seg_start[sg], se = seg_start[sg + 1];
     if (se == ss) continue;                                      // a skipped row
     const int kvh = sg % AKV, b = sg / AKV;
-    const int slot = slots[b], p0 = pos[b];
+    const int slot = slots[b], p0 = pos[b] + j0;                 // the pass's rows start at p0; the keys below it are in the pool
     const bool first = wt0 <= ss;                                // this workgroup holds the segment's first tile
     const int lo = max(0, max(wt0, ss) - ss - VISIT_TILES) * 16, hi = min(max(0, min(wt1, se) - ss - VISIT_TILES) * 16, p0);
     const size_t pslot = (size_t)blockIdx.x + sg;
@@ -187,7 +192,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     bf16x8 bq[8];
     {
         const bool real = n < R;
-        const bf16_t* qr = q + ((size_t)(b * M + (real ? n / GQA : 0)) * AH + kvh * GQA + (n % GQA)) * AD;
+        const bf16_t* qr = q + ((size_t)(b * Mtot + j0 + (real ? n / GQA : 0)) * AH + kvh * GQA + (n % GQA)) * AD;
 #pragma unroll
         for (int kb = 0; kb < 8; kb++) {
             u32x4 v = reinterpret_cast<const u32x4*>(qr)[kb * 4 + g];
@@ -253,8 +258,8 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     if (first && w == 3) {
         // The M new keys of this sequence, straight from the inputs (batch.py:143-145), with the causal rule among them:
         // key i is visible to query token j only if i <= j.  Not pipelined: it runs once per sequence.
-        const bf16_t* kn = k_new + ((size_t)b * M * AKV + kvh) * AD;
-        const bf16_t* vn = v_new + ((size_t)b * M * AKV + kvh) * AD;
+        const bf16_t* kn = k_new + ((size_t)(b * Mtot + j0) * AKV + kvh) * AD;
+        const bf16_t* vn = v_new + ((size_t)(b * Mtot + j0) * AKV + kvh) * AD;
         const size_t stride = (size_t)AKV * AD;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         {
@@ -281,8 +286,8 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     if (first && w == 0) {
         // append (batch.py:196-201): row j of this sequence goes to pool position p0 + j
         for (int j = 0; j < M; j++) {
-            const uint2 kk = reinterpret_cast<const uint2*>(k_new + ((size_t)(b * M + j) * AKV + kvh) * AD)[lane];
-            const uint2 vv2 = reinterpret_cast<const uint2*>(v_new + ((size_t)(b * M + j) * AKV + kvh) * AD)[lane];
+            const uint2 kk = reinterpret_cast<const uint2*>(k_new + ((size_t)(b * Mtot + j0 + j) * AKV + kvh) * AD)[lane];
+            const uint2 vv2 = reinterpret_cast<const uint2*>(v_new + ((size_t)(b * Mtot + j0 + j) * AKV + kvh) * AD)[lane];
             reinterpret_cast<uint2*>(Kp + pbase + (size_t)(p0 + j) * AD)[lane] = kk;
             reinterpret_cast<uint2*>(Vp + pbase + (size_t)(p0 + j) * AD)[lane] = vv2;
         }
@@ -336,7 +341,7 @@ constexpr int MAX_SPLITS = 4096;
 template <int M>
 __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                          const int* __restrict__ seg_tab, bf16_t* __restrict__ out, int B, int nwg,
-                                                         int min_tiles) {
+                                                         int min_tiles, int Mtot, int j0) {
     constexpr int R = 4 * M;
     __shared__ float fs_s[MAX_SPLITS];
     __shared__ float red_m[4], red_l[4];
@@ -381,7 +386,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
     const int d = tid;
     const float a = (acc_s[0][d] + acc_s[1][d]) + (acc_s[2][d] + acc_s[3][d]);
     const float ov = l == 0.f ? a : a / l;                                           // batch.py:216
-    out[((size_t)(b * M + r / GQA) * AH + kvh * GQA + (r % GQA)) * AD + d] = f2bf(ov);
+    out[((size_t)(b * Mtot + j0 + r / GQA) * AH + kvh * GQA + (r % GQA)) * AD + d] = f2bf(ov);
 }
 
 }  // namespace
@@ -389,6 +394,8 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
 extern "C" {
 
 constexpr int MAX_WG = 1024;           // upper bound of the partial kernel's grid (one workgroup per CU)
+constexpr int MAX_PASS_M = 4;          // query tokens per sequence in one pass (16 rows: one MFMA tile)
+constexpr int MAX_M = 16;              // query tokens per sequence in one call (as many as the verify step of the recurrent layers takes)
 
 static int partial_grid() {            // one workgroup per CU of the current device: measured faster than two (the stream is
                                        // bandwidth-bound with 64 KiB in flight per CU; a second workgroup only adds queueing)
@@ -402,7 +409,8 @@ constexpr long SEG_TAB_BYTES = ((MAX_SEG + 1) * 4 + 15) / 16 * 16;   // the segm
 // written against the fixed-split form and does not change the size
 long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH) {
     if (B < 0 || M < 1 || Lmax < 1 || CH < 16) return -1;
-    return ((long)MAX_WG + (long)B * AKV) * (4 * M) * (AD + 2) * 4 + SEG_TAB_BYTES;
+    const int mp = M < MAX_PASS_M ? M : MAX_PASS_M;                // the passes of a call with more tokens reuse one pass's space
+    return ((long)MAX_WG + (long)B * AKV) * (4 * mp) * (AD + 2) * 4 + SEG_TAB_BYTES;
 }
 
 // Both entry points: checks, grid size and the two launches.  The partial results of at most `slot_cap` slots
@@ -414,20 +422,23 @@ static int attn_launch(const void* q, const void* k_new, const void* v_new, void
     const long max_tiles = (long)B * AKV * ((Lmax + 15) / 16);
     const long want = (max_tiles + min_tiles - 1) / min_tiles;
     const int nwg = (int)(want < max_grid ? want : max_grid);
-    const dim3 g1((unsigned)nwg), g2((unsigned)(B * AKV * 4 * M));
+    const dim3 g1((unsigned)nwg);
 #define QT_ATTN_LAUNCH(MM)                                                                                                \
     hipLaunchKernelGGL(attn_partial_kernel<MM>, g1, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)k_new,         \
                        (const bf16_t*)v_new, (bf16_t*)Kp, (bf16_t*)Vp, slots, pos, part_o, part_ml, seg_tab, B, Lmax, min_tiles,    \
-                       n_slots);                                                                                          \
-    hipLaunchKernelGGL(attn_merge_kernel<MM>, g2, dim3(256), 0, stream, part_o, part_ml, seg_tab, (bf16_t*)out, B, nwg, min_tiles);
-    switch (M) {
-        case 1: QT_ATTN_LAUNCH(1) break;
-        case 2: QT_ATTN_LAUNCH(2) break;
-        case 3: QT_ATTN_LAUNCH(3) break;
-        default: QT_ATTN_LAUNCH(4) break;
+                       n_slots, M, j0);                                                                                   \
+    hipLaunchKernelGGL(attn_merge_kernel<MM>, dim3((unsigned)(B * AKV * 4 * MM)), dim3(256), 0, stream, part_o, part_ml, seg_tab,   \
+                       (bf16_t*)out, B, nwg, min_tiles, M, j0);
+    for (int j0 = 0; j0 < M; j0 += MAX_PASS_M) {                 // passes of up to four tokens per sequence
+        switch (M - j0 < MAX_PASS_M ? M - j0 : MAX_PASS_M) {
+            case 1: QT_ATTN_LAUNCH(1) break;
+            case 2: QT_ATTN_LAUNCH(2) break;
+            case 3: QT_ATTN_LAUNCH(3) break;
+            default: QT_ATTN_LAUNCH(4) break;
+        }
+        QT_CHECK_LAUNCH();
     }
 #undef QT_ATTN_LAUNCH
-    QT_CHECK_LAUNCH();
     return QT_OK;
 }
 
@@ -435,7 +446,7 @@ static int attn_check(const void* q, const void* k_new, const void* v_new, const
                       const int32_t* pos, const void* out, int B, int M, int Lmax, int n_slots, int CH) {
     if (!q || !k_new || !v_new || !Kp || !Vp || !slots || !pos || !out) return QT_ERR_NULL;
     if (B < 0 || Lmax < 1 || n_slots < 1 || CH < 16 || CH % 16) return QT_ERR_DIM;
-    if (M < 1 || M > 4 || B * AKV > MAX_SEG) return QT_ERR_UNSUPPORTED;
+    if (M < 1 || M > MAX_M || B * AKV > MAX_SEG) return QT_ERR_UNSUPPORTED;
     for (const void* p : {q, k_new, v_new, Kp, Vp})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
     return QT_OK;
@@ -450,9 +461,10 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
     if (reinterpret_cast<uintptr_t>(workspace) & 15u) return QT_ERR_ALIGN;
     if (workspace_bytes < qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)) return -6;
     const size_t cap = (size_t)MAX_WG + (size_t)B * AKV;
+    const int mp = M < MAX_PASS_M ? M : MAX_PASS_M;
     float* part_o = (float*)workspace;
-    float* part_ml = part_o + cap * (4 * M) * AD;
-    int* seg_tab = reinterpret_cast<int*>(part_ml + cap * (4 * M) * 2);
+    float* part_ml = part_o + cap * (4 * mp) * AD;
+    int* seg_tab = reinterpret_cast<int*>(part_ml + cap * (4 * mp) * 2);
     return attn_launch(q, k_new, v_new, Kp, Vp, slots, pos, out, part_o, part_ml, seg_tab, partial_grid(), B, M, Lmax, n_slots, CH,
                        stream);
 }
@@ -488,9 +500,10 @@ int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_ne
     unsigned char* base = nullptr;
     if (const int rc = scratch_address(&base)) return rc;
     // Nothing in the array has to start at zero: every partial slot and table entry a launch reads was written by that launch.
+    const int mp = M < MAX_PASS_M ? M : MAX_PASS_M;
     float* part_o = reinterpret_cast<float*>(base);
-    float* part_ml = part_o + ST_CAP * (4 * M) * AD;
-    int* seg_tab = reinterpret_cast<int*>(part_ml + ST_CAP * (4 * M) * 2);
+    float* part_ml = part_o + ST_CAP * (4 * mp) * AD;
+    int* seg_tab = reinterpret_cast<int*>(part_ml + ST_CAP * (4 * mp) * 2);
     const int grid = partial_grid() < ST_MAX_WG ? partial_grid() : ST_MAX_WG;
     return attn_launch(q, k_new, v_new, Kp, Vp, slots, pos, out, part_o, part_ml, seg_tab, grid, B, M, Lmax, n_slots, CH, stream);
 }

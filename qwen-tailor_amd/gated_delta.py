@@ -66,7 +66,7 @@ def gated_delta_update(q, k, v, a, b, A_log, dt_bias, state: Optional[torch.Tens
         state = torch.zeros((B, Hv, Dv, Dk), dtype=torch.float32, device=q.device)
     if Dk != 128 or Dv % 8 or state.dtype != torch.float32:
         raise ValueError(f"only the scalar-gate, Dk=128, fp32-state case is supported (Dk={Dk}, Dv={Dv}, state {state.dtype})")
-    if Dv % 16 or Hv % Hk:
+    if Hv % Hk:
         raise ValueError(f"unsupported head layout (Hk={Hk}, Hv={Hv}, Dv={Dv})")
     q, k, v = L.dev(q, BF16, "q", (B, T, Hk, Dk)), L.dev(k, BF16, "k"), L.dev(v, BF16, "v", (B, T, Hv, Dv))
     state = L.dev(state, torch.float32, "state", (B, Hv, Dv, Dk))

@@ -68,19 +68,78 @@ def gdn_chunked(q, k, v, proj, A_log, dt_bias, state, relaxed=True, flags=DEFAUL
 
 _SNAP = {}            # (device index, stream handle) -> float16 tensor: flag area + chain snapshots
 _SNAP_RETIRED = []    # outgrown buffers stay alive: a captured HIP graph may hold their address
+_STATUS = {}          # (device index, stream handle) -> pinned int32[1]: the last copy of the buffer's status word
+
+GAVE_UP, NOT_FINITE = 1, 2        # bits of the status word
+
+
+class ChunkedPrefillError(RuntimeError):
+    """A chunked-prefill launch on this stream reported a failure in its status word: its results are not to be used."""
+
+
+def _key(dev):
+    return (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
 
 
 def _snap_buffer(dev, nbytes):
-    """The buffer between phase B's chain and output workgroups, cached per (device, stream): its first KiB is the flag
+    """The buffer between phase B's chain and output workgroups, cached per (device, stream): its first 33 KiB are the flag
     area, which has to be zero before a launch and is left zero by it, so the buffer is zero-filled once, when it is made."""
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    key = _key(dev)
     buf = _SNAP.get(key)
     if buf is None or buf.numel() * 2 < nbytes:
         if buf is not None:
+            _raise_if_failed(key, buf, sync=True)          # the old buffer's word is looked at one last time
             _SNAP_RETIRED.append(buf)
         buf = torch.zeros(max(nbytes // 2, 8), dtype=torch.float16, device=dev)
         _SNAP[key] = buf
+        _STATUS[key] = torch.zeros(1, dtype=torch.int32, pin_memory=True)
     return buf
+
+
+def _status_word(buf):
+    off = L.lib().qt_gdn_chunk_status_offset() // 4
+    return buf.view(torch.int32)[off:off + 1]
+
+
+def _describe(v):
+    what = []
+    if v & GAVE_UP:
+        what.append("an output workgroup waited for its chunk for too long and gave up (its rows were not written)")
+    if v & NOT_FINITE:
+        what.append("the final state is not finite: a half-precision operand overflowed (|state|, |v| or an intermediate above 65504)")
+    return "; ".join(what) or f"status {v}"
+
+
+def _raise_if_failed(key, buf, sync=False):
+    """Looks at the status word of the launches made so far with `buf`.  Without `sync` it reads the host copy that the last
+    launch's asynchronous read-back has left (no wait: a launch still in flight is judged at the next call); with `sync` it
+    waits for the stream first.  A set word is cleared on the device and raised as ChunkedPrefillError."""
+    pin = _STATUS[key]
+    if sync and not torch.cuda.is_current_stream_capturing():
+        torch.cuda.current_stream(buf.device).synchronize()
+        pin.copy_(_status_word(buf))
+    v = int(pin[0])
+    if v:
+        torch.cuda.current_stream(buf.device).synchronize()     # error path only: no read-back may land after the reset
+        _status_word(buf).zero_()
+        pin.zero_()
+        raise ChunkedPrefillError("chunked prefill: " + _describe(v))
+
+
+def _read_back_status(key, buf):
+    """Enqueues the copy of the status word to pinned host memory behind the launch (skipped under graph capture)."""
+    if not torch.cuda.is_current_stream_capturing():
+        _STATUS[key].copy_(_status_word(buf), non_blocking=True)
+
+
+def check_status(device=None, sync=True):
+    """Raises ChunkedPrefillError if a chunked-prefill launch on the current stream of `device` has failed (see
+    _raise_if_failed).  phase_b / phase_b_norm call this without waiting before every launch, so a failure surfaces at the
+    next call at the latest; a caller that needs the answer for the launches already made calls it with sync=True."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    key = _key(dev)
+    if key in _SNAP:
+        _raise_if_failed(key, _SNAP[key], sync=sync)
 
 
 def _phase_b_args(S, Tb, Am, gv, state):
@@ -91,6 +150,7 @@ def _phase_b_args(S, Tb, Am, gv, state):
         raise ValueError("phase_b: the phase A records are too small for this many tokens")
     state = L.dev(state, torch.float32, "state").reshape(1, HV, DV, DK)
     snap = _snap_buffer(state.device, lib.qt_gdn_chunk_snap_bytes(S))
+    _raise_if_failed(_key(state.device), snap)              # the previous launch with this buffer, if its word has arrived
     return ops, U, gC, snap, state, torch.empty_like(state)
 
 
@@ -101,6 +161,7 @@ def phase_b(q, k, v, Tb, Am, gv, state, relaxed=True, flags=DEFAULT_FLAGS, tg=No
     ops, U, gC, snap, state, out = _phase_b_args(S, Tb, Am, gv, state)
     y = torch.empty((S, HV, DV), dtype=BF16, device=state.device)
     L.call("qt_gdn_phase_b", L.ptr(ops), L.ptr(U), L.ptr(gC), L.ptr(snap), L.ptr(state), L.ptr(out), L.ptr(y), S, L.stream())
+    _read_back_status(_key(state.device), snap)
     return y, out
 
 
@@ -114,4 +175,5 @@ def phase_b_norm(proj, Tb, Am, gv, state, gw, eps=1e-6):
     out = torch.empty((S, HV * DV), dtype=BF16, device=state.device)
     L.call("qt_gdn_phase_b_norm", L.ptr(ops), L.ptr(U), L.ptr(gC), L.ptr(snap), L.ptr(state), L.ptr(new_state), L.ptr(proj),
            L.ptr(gw), float(eps), L.ptr(out), S, L.stream())
+    _read_back_status(_key(state.device), snap)
     return out, new_state

@@ -211,3 +211,105 @@ def test_fused_conv_silu_exhaustive(qt, dev):
     check_tensors_equal("conv_prep v", v2, v)
     check_tensors_equal("conv_prep q", q2, q)
     check_tensors_equal("conv_prep k", k2, k)
+
+
+def _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0):
+    return qt.prefill.gdn_core(to_dev(proj, dev, BF16), to_dev(cs[None], dev, BF16), to_dev(S0[None], dev), to_dev(cw, dev, BF16),
+                               to_dev(A_log, dev), to_dev(dtb, dev), to_dev(gw, dev))
+
+
+@pytest.mark.parametrize("T", [300, 4100])
+def test_chunked_prefill_at_the_edge_of_the_half_precision_range(qt, dev, T):
+    """the documented operand range (|v|, |S| up to 65504): a state of N(0, 1e4) (largest element ~4.8e4) and conv outputs of a few
+    thousand keep the 2e-3 tolerance, in both launch forms of phase B, and leave the status word clear"""
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(900 + T, T, state_scale=1.0e4)
+    proj[:, 4096:6144] = bf(proj[:, 4096:6144] * 2000.0)
+    assert np.abs(S0).max() < 6.0e4
+    o4, conv4, s4 = _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0)
+    qt.gdn_nax.check_status(dev, sync=True)
+    oo, oy, otail, os_ = O.prefill_gdn(proj, cs, cw, A_log, dtb, S0, gw)
+    assert 1.0e3 < np.abs(oy).max() < 6.0e4
+    check_rel("final state rel-L2", to_np(s4)[0], os_, 2e-3, rel_l2)
+    check_rel("final state max", to_np(s4)[0], os_, 2e-3, rel_max)
+    check_rel("gated output rel-L2", to_np(o4), oo, 2e-3, rel_l2)
+
+
+@pytest.mark.parametrize("T", [300, 4100])
+def test_status_word_reports_operands_beyond_half_precision(qt, dev, T):
+    """a state beyond 65504 cannot be carried by the half-precision operands: the launch ends normally, bit 1 of the status
+    word is set, and the wrapper raises at the next call (or at check_status) instead of handing out the rows; the word is
+    reset by the raise, so the launch after it runs clean"""
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(950 + T, T, state_scale=1.0e6)
+    _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0)
+    with pytest.raises(qt.gdn_nax.ChunkedPrefillError, match="not finite"):
+        qt.gdn_nax.check_status(dev, sync=True)
+    qt.gdn_nax.check_status(dev, sync=True)                                   # reset
+    _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0)
+    torch.cuda.synchronize()                                                  # the read-back behind the launch has landed:
+    with pytest.raises(qt.gdn_nax.ChunkedPrefillError):                       # the next call sees it without waiting
+        _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0 * 1e-8)
+    o4, conv4, s4 = _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0 * 1e-8)
+    qt.gdn_nax.check_status(dev, sync=True)
+    oo, oy, otail, os_ = O.prefill_gdn(proj, cs, cw, A_log, dtb, S0 * 1e-8, gw)
+    check_rel("gated output after the reset", to_np(o4), oo, 2e-3, rel_l2)
+
+
+def test_give_up_path_ends_the_launch_and_leaves_the_flags_clean(qt, dev):
+    """the bounded wait of the one-launch form, forced from the host with a poll limit of one: output workgroups give up on chunks
+    the chain has not published yet, leave those rows unwritten and set bit 0 of the status word; every workgroup ends, the
+    last one to finish (a chain workgroup here: the output workgroups are done long before it) clears the progress words, and
+    the next launch on the same buffer, with the default limit, gives the bits of an undisturbed one"""
+    T = 8192
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(2002 + T, T)
+    want, _, s_want = _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0)
+    qt.gdn_nax.check_status(dev, sync=True)
+    lib = qt._lib.lib()
+    assert lib.qt_gdn_phase_b_poll_limit(1) == 0
+    try:
+        _, _, s_gave_up = _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0)
+        torch.cuda.synchronize()
+    finally:
+        assert lib.qt_gdn_phase_b_poll_limit(0) == 0
+    check_tensors_equal("the chain is not affected by output workgroups that gave up", s_gave_up, s_want)
+    flag_halves = lib.qt_gdn_chunk_snap_bytes(0) // 2
+    off = lib.qt_gdn_chunk_status_offset() // 4
+    for snap in qt.gdn_nax._SNAP.values():
+        words = snap[:flag_halves].view(torch.int32).clone()
+        assert int(words[off].item()) & qt.gdn_nax.GAVE_UP
+        words[off] = 0
+        assert int(words.ne(0).sum().item()) == 0, "progress words, done count or queue head left set"
+    with pytest.raises(qt.gdn_nax.ChunkedPrefillError, match="gave up"):
+        qt.gdn_nax.check_status(dev, sync=True)
+    got, _, s_got = _core(qt, dev, proj, cs, cw, A_log, dtb, gw, S0)
+    qt.gdn_nax.check_status(dev, sync=True)
+    check_tensors_equal("outputs of the launch after a give-up", got, want)
+    check_tensors_equal("state of the launch after a give-up", s_got, s_want)
+
+
+@pytest.mark.parametrize("T", [4096, 4100])
+def test_phase_b_through_the_c_abi_with_a_caller_owned_snap(qt, dev, T):
+    """qt_gdn_phase_b_norm called directly (ctypes) with a snap buffer the caller allocated and zeroed once: two launches in a row
+    give the bits of the wrapper path, and the flag area is zero after each"""
+    import ctypes
+    proj, cs, cw, A_log, dtb, gw, S0 = proj_inputs(3000 + T, T)
+    dproj, dgw, dS0 = to_dev(proj, dev, BF16), to_dev(gw, dev), to_dev(S0[None], dev)
+    _, _, _, ops, U, gC = qt.gdn_nax._phase_a(dproj, to_dev(cs, dev, BF16), to_dev(cw, dev, BF16), to_dev(A_log, dev), to_dev(dtb, dev),
+                                              want_qkv=False)
+    want, s_want = qt.gdn_nax.phase_b_norm(dproj, ops, U, gC, dS0, dgw)
+    lib = qt._lib.lib()
+    nbytes = lib.qt_gdn_chunk_snap_bytes(T)
+    flag_bytes = lib.qt_gdn_chunk_snap_bytes(0)
+    snap = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    snap.fill_(0xAB)                                                          # snapshots may hold anything ...
+    snap[:flag_bytes].zero_()                                                 # ... the flag area must be zero
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for launch in range(2):
+        out = torch.empty((T, 2048), dtype=BF16, device=dev)
+        s1 = torch.empty_like(dS0)
+        rc = lib.qt_gdn_phase_b_norm(p(ops), p(U), p(gC), p(snap), p(dS0), p(s1), p(dproj), p(dgw), 1e-6, p(out), T, stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        check_tensors_equal(f"launch {launch}: outputs", out, want)
+        check_tensors_equal(f"launch {launch}: state", s1, s_want)
+        assert int(snap[:flag_bytes].ne(0).sum().item()) == 0, "flag area (status word included) not zero after the launch"

@@ -48,7 +48,7 @@ def test_attn_b_layout_of_reference_test(qt, dev):
     run_case(qt, dev, rng, 6, 1024, np.array([3, 0, 5, 1, 2, 4], np.int32), np.array([0, 1, 31, 32, 300, 1023], np.int32), 1)
 
 
-@pytest.mark.parametrize("M", [2, 3, 4])
+@pytest.mark.parametrize("M", [2, 3, 4, 5, 6, 8, 9, 16])
 def test_attn_b_verify_rows(qt, dev, M):
     """reference tests/batch_spec.py:69-101: M query rows per sequence, causal among the new keys"""
     rng = np.random.default_rng(M)
@@ -86,7 +86,34 @@ def test_attn_b_out_of_range_rows_are_skipped(qt, dev):
     check_tensors_equal("pools untouched by a bad slot / a full sequence", Kp, K0)
     check_tensors_equal("pools untouched", Vp, V0)
     with pytest.raises(ValueError):
-        qt.batch.attn_b(q, kn, kn, Kp, Vp, torch.tensor([0], dtype=torch.int32, device=dev), torch.tensor([0], dtype=torch.int32, device=dev), M=5)
+        qt.batch.attn_b(q, kn, kn, Kp, Vp, torch.tensor([0], dtype=torch.int32, device=dev), torch.tensor([0], dtype=torch.int32, device=dev), M=17)
+
+
+@pytest.mark.parametrize("M", [5, 8])
+def test_attn_b_more_than_four_tokens_full_or_bad_rows(qt, dev, M):
+    """the reference kernel is generic in M (qwen35/batch.py:230-237, run.py:15 lets k be anything): a sequence whose M rows do
+    not all fit, or whose slot is outside the pool, is skipped as a whole by every pass (nothing of it is appended); its
+    neighbours are computed, rows of the later passes included"""
+    rng = np.random.default_rng(70 + M)
+    Lmax, S = 96, 4
+    slots = np.array([2, 9, 0, 1], np.int32)                                   # slot 9 is outside the pool
+    pos = np.array([Lmax - M, 5, Lmax - M + 1, 0], np.int32)                    # sequence 2: one row too many
+    Kp = bf(rng.standard_normal((S + 1, 2, Lmax, 256)))
+    Vp = bf(rng.standard_normal((S + 1, 2, Lmax, 256)))
+    q = bf(rng.standard_normal((4 * M, 8, 256)))
+    kn = bf(rng.standard_normal((4 * M, 2, 256)))
+    vn = bf(rng.standard_normal((4 * M, 2, 256)))
+    dK, dV = to_dev(Kp, dev, BF16), to_dev(Vp, dev, BF16)
+    o = to_np(qt.batch.attn_b(to_dev(q, dev, BF16), to_dev(kn, dev, BF16), to_dev(vn, dev, BF16), dK, dV, to_dev(slots, dev),
+                              to_dev(pos, dev), M))
+    oK, oV = Kp.copy(), Vp.copy()
+    good = np.array([0, 3])
+    rows = (good[:, None] * M + np.arange(M)[None]).ravel()
+    ref = O.attn_b(q[rows], kn[rows], vn[rows], oK, oV, slots[good], pos[good], M)
+    for i, r in enumerate(rows):
+        check_attn(f"o row {r}", o[r], ref[i])
+    check_equal("K pool", to_np(dK), oK)
+    check_equal("V pool", to_np(dV), oV)
 
 
 @pytest.mark.parametrize("B,M,Lmax", [(64, 1, 640), (64, 4, 640), (40, 1, 640), (40, 3, 640), (130, 2, 640), (300, 4, 200),

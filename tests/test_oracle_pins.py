@@ -584,3 +584,62 @@ def test_fused_gemv_gnorm_prologue_is_gated_norm():
     gw = (1 + 0.1 * rng.standard_normal(128)).astype(np.float32)
     W = bf(rng.standard_normal((8, 2048)) * 0.05)
     assert np.array_equal(O.fused_gemv(W, y, gnorm=(proj, gw)), O.fused_gemv(W, O.gated_norm(y, proj, gw)))
+
+
+# ---------------------------------------------------------------------------------------------- the layer core as a whole
+def _layer_core_float64(proj, cs, cw, A_log, dtb, S0, gw, swap_gates=False):
+    """An independent composition of the GatedDeltaNet layer core in float64, with no bf16 rounding anywhere and none of the
+    oracle's helpers: torch.conv1d over [state; x] (model.py:128-131), SiLU, textbook L2 normalisation of q and k
+    (gated_delta.py:21-30), textbook gates (gated_delta.py:16-18,158), the matrix form of the delta rule per head
+    S_t = g S (I - beta k k^T) + beta v k^T, y_t = S_t q, and rms_norm(y) * silu(z) (model.py:137-139)."""
+    T = proj.shape[0]
+    X = np.concatenate([cs, proj[:, :6144]], 0).astype(np.float64)
+    conv = torch.nn.functional.conv1d(torch.from_numpy(X).T[None], torch.from_numpy(cw.astype(np.float64))[:, None, :], groups=6144)[0].T
+    u = torch.nn.functional.silu(conv).numpy()
+    q, k, v = (u[:, i * 2048:(i + 1) * 2048].reshape(T, 16, 128) for i in range(3))
+    k = k / np.linalg.norm(k, axis=-1, keepdims=True)
+    q = q / np.linalg.norm(q, axis=-1, keepdims=True) / np.sqrt(128.0)
+    z = proj[:, 6144:8192].astype(np.float64).reshape(T, 16, 128)
+    b_in, a_in = proj[:, 8192:8208].astype(np.float64), proj[:, 8208:8224].astype(np.float64)
+    if swap_gates:
+        a_in, b_in = b_in, a_in
+    g = np.exp(-np.exp(A_log.astype(np.float64)) * np.logaddexp(0.0, a_in + dtb.astype(np.float64)))
+    beta = 1.0 / (1.0 + np.exp(-b_in))
+    S = S0.astype(np.float64).copy()                                             # [head][dv][dk]
+    y = np.zeros((T, 16, 128))
+    for t in range(T):
+        for h in range(16):
+            kk = k[t, h]
+            S[h] = g[t, h] * S[h] @ (np.eye(128) - beta[t, h] * np.outer(kk, kk)) + beta[t, h] * np.outer(v[t, h], kk)
+            y[t, h] = S[h] @ q[t, h]
+    out = (torch.nn.functional.rms_norm(torch.from_numpy(y), (128,), torch.from_numpy(gw.astype(np.float64)), 1e-6)
+           * torch.nn.functional.silu(torch.from_numpy(z))).reshape(T, 2048).numpy()
+    return out, y.reshape(T, 2048), S
+
+
+@pytest.mark.parametrize("T", [1, 2, 8])
+def test_prefill_gdn_vs_independent_float64_composition(T):
+    """O.prefill_gdn (the composition the chunked-prefill GPU tests compare with) against a composition that shares nothing with
+    it: column layout of the projection row, head mapping, state layout [dv][dk], conv tail.  The two differ by the bf16
+    roundings of the reference's arithmetic only (a few 2^-8 steps per stage); a swapped gate column, a transposed state or a
+    shifted conv window differ by tens of percent."""
+    rng = np.random.default_rng(40 + T)
+    cw, A_log, dtb = _layer_params(rng)
+    gw = rng.uniform(0.5, 1.5, 128).astype(np.float32)
+    proj = bf(rng.standard_normal((T, O.PW)))
+    cs = bf(rng.standard_normal((3, O.CD)))
+    S0 = (rng.standard_normal((16, 128, 128)) * 0.5).astype(np.float32)
+    out, y, tail, S1 = O.prefill_gdn(proj, cs, cw, A_log, dtb, S0, gw)
+    rout, ry, rS = _layer_core_float64(proj, cs, cw, A_log, dtb, S0, gw)
+    rel = lambda a, b: float(np.linalg.norm(np.asarray(a, np.float64) - b) / np.linalg.norm(b))
+    assert rel(S1, rS) < 1e-2                  # k, v, beta each carry a bf16 rounding (2^-9) into every rank-one term
+    assert rel(y, ry) < 2e-2
+    assert rel(out, rout) < 2.5e-2
+    assert np.array_equal(tail, np.concatenate([cs, proj[:, :6144]], 0)[-3:])       # prefill.py:262-263
+    # plausible mistakes are far outside those bounds
+    bout, by, bS = _layer_core_float64(proj, cs, cw, A_log, dtb, S0, gw, swap_gates=True)
+    assert rel(y, by) > 0.1
+    ty = _layer_core_float64(proj, cs, cw, A_log, dtb, np.ascontiguousarray(S0.transpose(0, 2, 1)), gw)[1]
+    assert rel(y[0], ty[0]) > 0.1                                                 # (the first token reads the initial state undecayed)
+    sy = _layer_core_float64(proj, np.roll(cs, 1, axis=0), cw, A_log, dtb, S0, gw)[1]
+    assert rel(y, sy) > 0.1

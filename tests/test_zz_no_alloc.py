@@ -36,12 +36,18 @@ def _case(lib, dev, seed, B, M, Lmax, lo, hi):
     # the allocation-free one
     K2, V2 = Kp.clone(), Vp.clone()
     o2 = torch.zeros((B * M, 8, 256), dtype=BF16, device=dev)
+    # a first call on scratch pools: the symbol lookup and the lazy load of the kernels' code object happen there, once
+    K3, V3, o3 = Kp.clone(), Vp.clone(), torch.zeros_like(o2)
+    rc = lib.qt_gqa_attn_decode_static(p(q), p(kn), p(vn), p(K3), p(V3), p(dslots), p(dpos), p(o3), B, M, Lmax, S + 1, CH, stream)
+    assert rc == 0, rc
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated(dev)
+    before = torch.cuda.memory_allocated(dev)           # torch's caching allocator ...
+    free_before = torch.cuda.mem_get_info(dev)[0]       # ... and the driver's own count of free device memory (sees a hipMalloc)
     rc = lib.qt_gqa_attn_decode_static(p(q), p(kn), p(vn), p(K2), p(V2), p(dslots), p(dpos), p(o2), B, M, Lmax, S + 1, CH, stream)
     assert rc == 0, rc
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before, "the driver's free-memory count moved across the call"
     check_tensors_equal(f"out (B={B}, M={M})", o2, o1)
     check_tensors_equal("K pool", K2, K1)
     check_tensors_equal("V pool", V2, V1)
@@ -54,6 +60,7 @@ def test_static_scratch_entry_point_matches_workspace_entry_point(dev):
     _case(lib, dev, 1, 16, 4, 4096 + 8, 1024, 4096)       # fills most of the partial slots
     _case(lib, dev, 2, 3, 1, 512, 0, 300)                 # smaller, right after: stale partials of the first call must not matter
     _case(lib, dev, 3, 128, 2, 256, 0, 250)               # the largest batch the static array takes
+    _case(lib, dev, 4, 5, 7, 300, 0, 290)                 # more than four tokens per sequence: two passes over one array
 
 
 def test_static_scratch_entry_point_rejects_larger_batches(dev):
