@@ -154,7 +154,7 @@ def test_gated_delta_update_value_dim_multiple_of_8(qt, dev, Dv):
     check_rel("state", to_np(s1), os_, 1e-4, rel_max)
     check_ulp("y", to_np(y), oy)
     with pytest.raises(ValueError):
-        qt.gated_delta.gated_delta_update(to_dev(q, dev, BF16), to_dev(k, dev, BF16), to_dev(v[..., :12], dev, BF16).contiguous(),
+        qt.gated_delta.gated_delta_update(to_dev(q, dev, BF16), to_dev(k, dev, BF16), to_dev(rand_bf(gen, (B, T, H, 12)), dev, BF16),
                                           to_dev(a, dev, BF16), to_dev(b, dev, BF16), to_dev(A_log[:H], dev), to_dev(dtb[:H], dev))
 
 
