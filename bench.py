@@ -257,6 +257,42 @@ def bench_attn(torch, qt, dev, B, M, lo, hi, seed):
             "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
 
 
+def bench_attn_layer(torch, qt, dev, B, M, lo, hi, seed):
+    """the attention half of a full-attention layer at a decode / verify step, between its qkv and o projections
+    (qwen35/batch.py:505-513): as attention.qkv_prep + batch.attn_b + attention.out_gate (four launches) and as
+    batch.attn_layer_b (two); pools rotated as in bench_attn"""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    Lmax = hi + 8
+    pos = torch.from_numpy(rng.integers(lo, hi, B).astype(np.int32)).to(dev)
+    slots = torch.from_numpy(rng.permutation(B).astype(np.int32)).to(dev)
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    nbytes = int(pos.sum().item()) * 2 * 2 * 256 * 2
+    n_pools = max(2, min(16, -(-1100000000 // nbytes)))
+    Kp0 = torch.randn((B + 1, 2, Lmax, 256), generator=g).to(bf).to(dev)
+    Vp0 = torch.randn((B + 1, 2, Lmax, 256), generator=g).to(bf).to(dev)
+    pools = [(Kp0, Vp0)] + [(Kp0.clone(), Vp0.clone()) for _ in range(n_pools - 1)]
+    qkv = torch.randn((B * M, 5120), generator=g).to(bf).to(dev)
+    qn, kn = torch.ones(256, dtype=bf, device=dev), torch.ones(256, dtype=bf, device=dev)
+    it = [0]
+
+    def four():
+        Kp, Vp = pools[it[0] % n_pools]
+        it[0] += 1
+        q, k, v = qt.attention.qkv_prep(qkv, qn, kn, pos, M)
+        qt.attention.out_gate(qt.batch.attn_b(q, k, v, Kp, Vp, slots, pos, M), qkv)
+
+    def two():
+        Kp, Vp = pools[it[0] % n_pools]
+        it[0] += 1
+        qt.batch.attn_layer_b(qkv, qn, kn, Kp, Vp, slots, pos, M)
+    t4 = time_graph(torch, four, reps=n_pools * 12, inner=n_pools)
+    t2 = time_graph(torch, two, reps=n_pools * 12, inner=n_pools)
+    return {"B": B, "M": M, "pools": n_pools, "sum_L": int(pos.sum().item()), "four_launches_us": t4 * 1e6, "two_launches_us": t2 * 1e6,
+            "bytes": nbytes, "two_launches_GBps": nbytes / t2 / 1e9, "two_launches_hbm_frac": nbytes / t2 / 1e9 / HBM_PEAK_GBS}
+
+
 def bench_attn_prefill(torch, qt, dev, S=2048, seed=7):
     """causal prefill attention over S rows; the calls rotate over enough (q, K, V) sets to exceed the last-level cache"""
     g = torch.Generator().manual_seed(seed)
@@ -457,6 +493,8 @@ def profile_leg(torch, qt, dev, args):
         bench_attn(torch, qt, dev, 16, 1, 512, 32768, 1003)
     elif leg == "attn_verify":
         bench_attn(torch, qt, dev, 16, 4, 1024, 8192, 1004)
+    elif leg == "attn_layer":
+        bench_attn_layer(torch, qt, dev, 16, 4, 1024, 8192, 1004)
     elif leg == "attn_prefill":
         bench_attn_prefill(torch, qt, dev)
     elif leg == "projections":
@@ -497,7 +535,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the B sweep and the single-pool run")
     ap.add_argument("--only", default="", help="profile helper: run only one leg a few times and exit "
-                                               "(decode | copy | prefill | prefill_long | verify | attn_decode | attn_verify | attn_prefill | attn_prefill_long | "
+                                               "(decode | copy | prefill | prefill_long | verify | attn_decode | attn_verify | attn_layer | attn_prefill | attn_prefill_long | "
                                                "projections | state_admission | prefix_cache | attn_glue)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -587,6 +625,10 @@ def main():
         extras["attn_decode_config3"] = bench_attn(torch, qt, dev, 16, 1, 512, 32768, 1003)
         torch.cuda.empty_cache()
         extras["attn_verify_config4"] = bench_attn(torch, qt, dev, 16, 4, 1024, 8192, 1004)
+        extras["attn_layer_half_config4"] = bench_attn_layer(torch, qt, dev, 16, 4, 1024, 8192, 1004)
+        torch.cuda.empty_cache()
+        extras["attn_layer_half_config3"] = bench_attn_layer(torch, qt, dev, 16, 1, 512, 32768, 1003)
+        torch.cuda.empty_cache()
         extras["attn_prefill_causal"] = [bench_attn_prefill(torch, qt, dev, S) for S in (2048, 8192)]
         extras["state_admission"] = bench_state_admission(torch, qt, dev)
         extras["attn_glue"] = bench_attn_glue(torch, qt, dev)

@@ -104,6 +104,20 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
 int qt_gqa_attn_decode_static(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
                               const int32_t* pos, void* out, int B, int M, int Lmax, int n_slots, int CH, qt_stream_t stream);
 
+/* The attention half of a full-attention layer at a decode / verify step, between its qkv and o projections, in two launches per
+ * pass of four tokens: qt_attn_qkv_prep, qt_gqa_attn_decode and qt_attn_out_gate in one (qwen35/batch.py:505-513: mx.fast.rms_norm
+ * and mx.fast.rope on q / k, attn_b, o * sigmoid(gate)).  qkv [B*M,5120] bf16 as for qt_attn_qkv_prep; q_norm, k_norm [256] bf16;
+ * out [B*M,2048] bf16, the same values as the three calls give.  The query rows and the new keys are normed and roped inside
+ * the attention kernel by every workgroup that needs them, the gate is applied where the split-K parts are merged; q, k, v
+ * and the un-gated o are never stored.  rope_table: the (cos, sin) pairs of positions 0 .. table_positions - 1
+ * (qt_rope_table_bytes(n) bytes, written once by qt_rope_table_build, owned by the caller, 16-byte aligned); table_positions >=
+ * Lmax.  Workspace, limits and the treatment of out-of-range rows as for qt_gqa_attn_decode. */
+long qt_rope_table_bytes(int n_pos);
+int qt_rope_table_build(void* table, int n_pos, qt_stream_t stream);
+int qt_gqa_attn_layer_decode(const void* qkv, const void* q_norm, const void* k_norm, const void* rope_table, int table_positions,
+                             void* Kp, void* Vp, const int32_t* slots, const int32_t* pos, void* out, void* workspace,
+                             long workspace_bytes, int B, int M, int Lmax, int n_slots, int CH, float eps, qt_stream_t stream);
+
 /* Chunked (chunk = 64) GatedDeltaNet prefill, two phases (qwen35/gdn_nax.py:394-426: prep_a / gdn_chunked's phase A, phase_b).
  * Phase A is parallel over (chunk, head): it takes q, k, v [S,16,128] bf16 (qt_gdn_conv_prep's outputs) and the gate inputs in
  * proj [S,8224], and computes the gates, K K^T / Q K^T on fp16 MFMA, the 64 x 64 unit-lower-triangular inverse in fp32 and the

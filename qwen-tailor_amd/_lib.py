@@ -29,6 +29,8 @@ _SIGS = {
     "qt_gdn_recurrent": [_vp] * 8 + [_i] * 6 + [_vp],
     "qt_gqa_attn_decode": [_vp] * 9 + [_l, _i, _i, _i, _i, _i, _vp],
     "qt_gqa_attn_decode_static": [_vp] * 8 + [_i, _i, _i, _i, _i, _vp],
+    "qt_gqa_attn_layer_decode": [_vp] * 4 + [_i] + [_vp] * 6 + [_l, _i, _i, _i, _i, _i, _f, _vp],
+    "qt_rope_table_build": [_vp, _i, _vp],
     "qt_gdn_phase_b": [_vp] * 7 + [_i, _vp],
     "qt_gdn_phase_b_poll_limit": [_i],
     "qt_gdn_phase_b_norm": [_vp] * 8 + [_f, _vp, _i, _vp],
@@ -57,6 +59,7 @@ def lib():
             fn.argtypes, fn.restype = args, ctypes.c_int
         L.qt_gqa_attn_workspace_bytes.argtypes, L.qt_gqa_attn_workspace_bytes.restype = [_i] * 4, ctypes.c_long
         L.qt_gdn_chunk_status_offset.argtypes, L.qt_gdn_chunk_status_offset.restype = [], ctypes.c_long
+        L.qt_rope_table_bytes.argtypes, L.qt_rope_table_bytes.restype = [_i], ctypes.c_long
         for name in ("qt_gdn_chunk_ops_bytes", "qt_gdn_chunk_u_bytes", "qt_gdn_chunk_gc_bytes", "qt_gdn_chunk_snap_bytes",
                      "qt_gqa_prefill_workspace_bytes"):
             getattr(L, name).argtypes, getattr(L, name).restype = [_i], ctypes.c_long
@@ -90,6 +93,24 @@ def silu_table(dev):
         call("qt_silu_table_build", ptr(t), stream())
         _SILU_TABLES[dev] = t
     return t
+
+
+_ROPE_TABLES = {}        # device -> float32 [positions, 32, 2]
+_ROPE_RETIRED = []       # outgrown tables stay alive: a captured HIP graph may hold their address
+
+
+def rope_table(dev, n_pos):
+    """The (cos, sin) pairs of the rotary embedding for positions 0 .. n_pos - 1 on `dev` (built by the library, owned here;
+    grown in steps of 16384 positions).  Returns (tensor, positions it covers)."""
+    t = _ROPE_TABLES.get(dev)
+    if t is None or t.shape[0] < n_pos:
+        if t is not None:
+            _ROPE_RETIRED.append(t)
+        n = -(-max(n_pos, 1) // 16384) * 16384
+        t = torch.empty((n, 32, 2), dtype=torch.float32, device=dev)
+        call("qt_rope_table_build", ptr(t), n, stream())
+        _ROPE_TABLES[dev] = t
+    return t, t.shape[0]
 
 
 def stream():

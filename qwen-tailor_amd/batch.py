@@ -100,6 +100,39 @@ def attn_b(q, k, v, Kp, Vp, slots, pos, M=1, split=None, workspace=None):
     return o
 
 
+def attn_layer_b(qkv, q_norm, k_norm, Kp, Vp, slots, pos, M=1, eps=1e-6, split=None, workspace=None):
+    """The attention half of a full-attention layer at a decode / verify step (qwen35/batch.py:505-513), between the qkv and o
+    projections: q / k RMSNorm and rotary embedding, attn_b, and o * sigmoid(gate), in two launches per pass of four tokens
+    (attention.qkv_prep + attn_b + attention.out_gate are four), with the same bits.  qkv [B*M,5120] bf16 = [(q_h | gate_h) x 8 |
+    k x 2 | v x 2]; q_norm, k_norm [256] bf16; pools, slots, pos, M as for attn_b (the new K / V rows are appended in place).
+    Returns [B*M,2048] bf16."""
+    qkv = L.dev(qkv, BF16, "qkv", (None, 5120))
+    R = qkv.shape[0]
+    if M < 1 or M > 16 or R % M:
+        raise ValueError(f"attn_layer_b: M = {M} (1..16) must divide the number of rows ({R})")
+    B = R // M
+    qn, kn = L.dev(q_norm, BF16, "q_norm", (256,)), L.dev(k_norm, BF16, "k_norm", (256,))
+    Kp = L.dev(Kp, BF16, "Kp", (None, 2, None, 256))
+    Vp = L.dev(Vp, BF16, "Vp", tuple(Kp.shape))
+    n_slots, Lmax = Kp.shape[0], Kp.shape[2]
+    slots, pos = L.i32(slots, "slots", B), L.i32(pos, "pos", B)
+    CH = split or split_size(Lmax, B)
+    nbytes = L.lib().qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)
+    if nbytes < 0:
+        raise ValueError("attn_layer_b: bad split size")
+    if workspace is None:
+        ws = _workspace(qkv.device, nbytes)
+    else:
+        ws = L.dev(workspace, torch.uint8, "workspace")
+        if ws.numel() < nbytes:
+            raise ValueError(f"attn_layer_b: workspace of {ws.numel()} bytes, {nbytes} needed")
+    table, n_pos = L.rope_table(qkv.device, Lmax)
+    out = torch.empty((R, 2048), dtype=BF16, device=qkv.device)
+    L.call("qt_gqa_attn_layer_decode", L.ptr(qkv), L.ptr(qn), L.ptr(kn), L.ptr(table), n_pos, L.ptr(Kp), L.ptr(Vp), L.ptr(slots),
+           L.ptr(pos), L.ptr(out), L.ptr(ws), ws.numel(), B, M, Lmax, n_slots, CH, float(eps), L.stream())
+    return out
+
+
 def gnorm_rows(y, proj, gw, eps=1e-6):
     """Gated RMSNorm of the delta-rule output (qwen35/batch.py:338-343): y [B, 2048] bf16, proj [B, 8224] bf16 (its z slice
     is at 6144:8192), gw float32 [128].  Returns [B, 2048] bf16."""

@@ -92,6 +92,16 @@ __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const bf16_t* __rest
     }
 }
 
+// (cos, sin) of every rotary angle of positions 0 .. n_pos - 1, exactly the values the kernel above evaluates per row:
+// table[p][i] = ((float)cos((double)th), (float)sin((double)th)), th = float(p) * rope_freq[i] rounded to float
+__global__ __launch_bounds__(256) void rope_table_kernel(float2* __restrict__ table, int n_pos) {
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (long)n_pos * (ROPE_DIM / 2)) return;
+    const int p = (int)(t / (ROPE_DIM / 2)), i = (int)(t % (ROPE_DIM / 2));
+    const float th = __fmul_rn((float)p, rope_freq[i]);
+    table[t] = make_float2((float)cos((double)th), (float)sin((double)th));
+}
+
 // out[r][h*256 + d] = BF(o[r][h][d] * sigmoid_bf16(gate_h[d])), gate_h = qkv[r][h*512 + 256 ..]; 8 elements per thread
 __global__ __launch_bounds__(256) void attn_out_gate_kernel(const bf16_t* __restrict__ o, const bf16_t* __restrict__ qkv,
                                                             bf16_t* __restrict__ out, long R) {
@@ -123,6 +133,17 @@ int qt_attn_qkv_prep(const void* qkv, const void* q_norm, const void* k_norm, co
         if (reinterpret_cast<uintptr_t>(p) & 7u) return QT_ERR_ALIGN;
     hipLaunchKernelGGL(attn_qkv_prep_kernel, dim3((unsigned)R), dim3(256), 0, stream, (const bf16_t*)qkv, (const bf16_t*)q_norm,
                        (const bf16_t*)k_norm, pos, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, R, M, eps);
+    QT_CHECK_LAUNCH();
+    return QT_OK;
+}
+
+int qt_rope_table_build(void* table, int n_pos, hipStream_t stream) {
+    if (!table) return QT_ERR_NULL;
+    if (n_pos < 0) return QT_ERR_DIM;
+    if (reinterpret_cast<uintptr_t>(table) & 15u) return QT_ERR_ALIGN;
+    if (n_pos == 0) return QT_OK;
+    const long n = (long)n_pos * (ROPE_DIM / 2);
+    hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, (float2*)table, n_pos);
     QT_CHECK_LAUNCH();
     return QT_OK;
 }

@@ -48,6 +48,10 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// ---- the layer form: q / k RMSNorm and rotary embedding inside the attention kernel (qwen35/batch.py:505-512) ----------------
+constexpr int QKV_W = AH * 2 * AD + 2 * AKV * AD;      // 5120: [(q_h | gate_h) x 8 | k x 2 | v x 2]
+constexpr int ROPE_PAIRS = 32;                         // rotary pairs (i, i + 32), i < 32, of the first 64 features
+
 // Online-softmax update of one tile of 16 keys from its transposed scores: lane (row n, group g) holds keys 4g .. 4g+3.
 // Leaves the probabilities of those keys in p (fp32) and writes the row's rescale factor to c_lds[row].
 __device__ __forceinline__ void softmax_tile(const f32x4& acc, int nvalid, bool causal, float& m_run, float& l_run, float (&p)[4],
@@ -112,14 +116,14 @@ constexpr int VISIT_TILES = 5;
 
 // Exclusive prefix of the segments' tile counts -> seg_start[0 .. nseg] (LDS); returns the total.  Rows whose slot or position
 // is out of range own no tiles (they are skipped by both kernels).  Every thread of the workgroup must call it.
-template <int M>
+template <int M, int VISIT>
 __device__ __forceinline__ int build_segments(int* seg_start, const int* __restrict__ slots, const int* __restrict__ pos, int nseg,
                                               int Lmax, int n_slots, int Mtot, int j0) {
     const int tid = threadIdx.x, lane = tid & 63;
     for (int sg = tid; sg < nseg; sg += 256) {
         const int b = sg / AKV, slot = slots[b], p0 = pos[b];
         const bool ok = (unsigned)slot < (unsigned)n_slots && p0 >= 0 && p0 + Mtot <= Lmax;    // all of the sequence's rows fit, or none is taken
-        seg_start[sg + 1] = ok ? max(1, (p0 + j0 + 15) >> 4) + VISIT_TILES : 0;
+        seg_start[sg + 1] = ok ? max(1, (p0 + j0 + 15) >> 4) + VISIT : 0;
     }
     if (tid == 0) seg_start[0] = 0;
     __syncthreads();
@@ -145,13 +149,18 @@ __device__ __forceinline__ int tiles_per_wg(int total, int nwg, int min_tiles) {
 
 // partial results: slot id = workgroup + segment (unique, and consecutive for the workgroups that share a segment);
 // part_o [slot][4*M rows][256] f32 (unnormalised), part_ml [slot][4*M][2] = (running max, running sum)
-template <int M>
-__global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_new,
+// LAYER: q is the layer's qkv rows [B*Mtot, 5120]; the query rows and the new keys are normed and roped here, the
+// new values are read from the rows' v part, and k_new / v_new are not used.
+// (one workgroup per CU in that form: it holds the staged query rows in LDS beside the tiles)
+template <int M, bool LAYER>
+__global__ __launch_bounds__(256, LAYER ? 1 : 2) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_new,
                                                            const bf16_t* __restrict__ v_new, bf16_t* Kp, bf16_t* Vp,
                                                            const int* __restrict__ slots, const int* __restrict__ pos,
                                                            float* __restrict__ part_o, float* __restrict__ part_ml,
                                                            int* __restrict__ seg_tab, int B, int Lmax, int min_tiles, int n_slots,
-                                                           int Mtot, int j0) {
+                                                           int Mtot, int j0, const bf16_t* __restrict__ q_norm,
+                                                           const bf16_t* __restrict__ k_norm, const float2* __restrict__ rope_tab,
+                                                           float eps) {
     // M = tokens of this pass (rows j0 .. j0 + M - 1 of each sequence's Mtot rows)
     constexpr int R = 4 * M;
     __shared__ int seg_start[MAX_SEG + 1];
@@ -164,7 +173,9 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     float* const mo = reinterpret_cast<float*>(tile_s);
 
     const int nseg = B * AKV;
-    const int total = build_segments<M>(seg_start, slots, pos, nseg, Lmax, n_slots, Mtot, j0);
+    // (both forms cut the tile space alike, so that the layer form sums its partial results in the order of the plain one: same bits)
+    constexpr int VISIT = VISIT_TILES;
+    const int total = build_segments<M, VISIT>(seg_start, slots, pos, nseg, Lmax, n_slots, Mtot, j0);
     if (blockIdx.x == 0)                                         // the merge kernel reads the table instead of building it again
         for (int i = threadIdx.x; i <= nseg; i += 256) seg_tab[i] = seg_start[i];
     const int per = tiles_per_wg(total, gridDim.x, min_tiles);
@@ -185,12 +196,111 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     const int kvh = sg % AKV, b = sg / AKV;
     const int slot = slots[b], p0 = pos[b] + j0;                 // the pass's rows start at p0; the keys below it are in the pool
     const bool first = wt0 <= ss;                                // this workgroup holds the segment's first tile
-    const int lo = max(0, max(wt0, ss) - ss - VISIT_TILES) * 16, hi = min(max(0, min(wt1, se) - ss - VISIT_TILES) * 16, p0);
+    const int lo = max(0, max(wt0, ss) - ss - VISIT) * 16, hi = min(max(0, min(wt1, se) - ss - VISIT) * 16, p0);
     const size_t pslot = (size_t)blockIdx.x + sg;
+
+    const size_t pbase = ((size_t)slot * AKV + kvh) * Lmax * AD;
+    const bf16_t* kbase = Kp + pbase;
+    const bf16_t* vbase = Vp + pbase;
+    bf16_t* vl = tile_s + w * (16 * VL_LD);
+    bf16_t* kl = tile_s + 4 * (16 * VL_LD) + w * (16 * KL_LD);
+    const int ntiles = hi > lo ? (hi - lo + 15) / 16 : 0;
+    // Row addresses of a tile: key 2i (lower half wavefront) / 2i + 1 (upper half), 8 columns per lane, so one load covers
+    // two whole 512-byte rows (a wavefront-wide load of 16 rows x 64 bytes streams about 15 % slower from HBM).  Keys past
+    // `hi` re-read the tile's first key (they are masked / weighted by 0).
+    auto row_ptr = [&](const bf16_t* base, int t, int i) {
+        const int key0 = lo + t * 16, key = key0 + 2 * i + hw;
+        return reinterpret_cast<const u32x4*>(base + (size_t)(key < hi ? key : key0) * AD) + cl;
+    };
+    u32x4 a[8], vv[8];
 
     // Q^T as the MFMA B operand: lane (row n, group g) holds q[row n][32 kb + 8 g .. + 8]; row n = token (n / 4), head n % 4
     bf16x8 bq[8];
-    {
+    u32x4 knew[8];                                                // (layer form: the new keys, wavefront 3 of the first workgroup)
+    if constexpr (LAYER) {
+        // The wavefront's first tile is requested before anything else: the norm and the rotary embedding below run while it
+        // is on its way from HBM.
+        if (w < ntiles) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) a[i] = __builtin_nontemporal_load(row_ptr(kbase, w, i));
+#pragma unroll
+            for (int i = 0; i < 8; i++) vv[i] = __builtin_nontemporal_load(row_ptr(vbase, w, i));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // The 4 M query rows are normed and roped once per workgroup: wavefront w takes token w (its four heads, a row per
+        // 16-lane group, 16 consecutive elements per lane) and leaves the rows in LDS, where every wavefront picks up its
+        // B operand.  The workgroup that holds the segment's first tile does the same for the M new keys (wavefront 0, a key
+        // per 16-lane group), which it also appends to the pool (batch.py:196-201).  Same arithmetic, value for value, as
+        // attn_qkv_prep_kernel: sum of squares exact in double and rounded once, correctly rounded 1 / sqrt,
+        // BF(w * BF(x * inv)), rotary products and sums rounded one by one; (cos, sin) from the table qt_rope_table_build wrote.
+        __shared__ __align__(16) bf16_t q_s[16 * KL_LD], k_s[4 * KL_LD];
+        const int rr = lane >> 4, c = lane & 15;
+        auto glue16 = [&](const bf16_t* x, const bf16_t* wgt, const float2* cs, u32x4& o0, u32x4& o1) {
+            const u32x4 x0 = reinterpret_cast<const u32x4*>(x)[0], x1 = reinterpret_cast<const u32x4*>(x)[1];
+            const u32x4 w0 = reinterpret_cast<const u32x4*>(wgt)[0], w1 = reinterpret_cast<const u32x4*>(wgt)[1];
+            f32x4 cv[8];                                          // rotary pairs 16 (c & 1) .. + 15 (used by lanes c < 4 only)
+#pragma unroll
+            for (int e = 0; e < 8; e++) cv[e] = reinterpret_cast<const f32x4*>(cs)[e];
+            float y[16], wt[16];
+            unpack8(make_uint4(x0[0], x0[1], x0[2], x0[3]), reinterpret_cast<float(&)[8]>(y[0]));
+            unpack8(make_uint4(x1[0], x1[1], x1[2], x1[3]), reinterpret_cast<float(&)[8]>(y[8]));
+            unpack8(make_uint4(w0[0], w0[1], w0[2], w0[3]), reinterpret_cast<float(&)[8]>(wt[0]));
+            unpack8(make_uint4(w1[0], w1[1], w1[2], w1[3]), reinterpret_cast<float(&)[8]>(wt[8]));
+            double ss = 0.0;
+#pragma unroll
+            for (int e = 0; e < 16; e++) ss += (double)y[e] * y[e];
+            const float inv = rsqrt_rn((float)row16_sum_d(ss) / (float)AD + eps);
+#pragma unroll
+            for (int e = 0; e < 16; e++) y[e] = BF(wt[e] * BF(y[e] * inv));
+            // rotary pairs (i, i + 32), i < 32: lanes 0, 1 of a row hold the first halves, lanes 2, 3 their partners
+            float other[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++) other[e] = __shfl_xor(y[e], 2, 64);
+            if (c < 4) {
+#pragma clang fp contract(off)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const float cs_c = cv[e >> 1][2 * (e & 1)], cs_s = cv[e >> 1][2 * (e & 1) + 1];
+                    const float own = y[e] * cs_c, oth = other[e] * cs_s;
+                    y[e] = BF(c < 2 ? own - oth                   // y1 c - y2 s
+                                    : oth + own);                 // y1 s + y2 c
+                }
+            }
+            o0 = u32x4{pack2_bf(y[0], y[1]), pack2_bf(y[2], y[3]), pack2_bf(y[4], y[5]), pack2_bf(y[6], y[7])};
+            o1 = u32x4{pack2_bf(y[8], y[9]), pack2_bf(y[10], y[11]), pack2_bf(y[12], y[13]), pack2_bf(y[14], y[15])};
+        };
+        {
+            u32x4 o0 = {0, 0, 0, 0}, o1 = {0, 0, 0, 0};           // (rows past 4 M: zeros)
+            if (w < M)
+                glue16(q + (size_t)(b * Mtot + j0 + w) * QKV_W + (kvh * GQA + rr) * 2 * AD + 16 * c, q_norm + 16 * c,
+                       rope_tab + (size_t)(p0 + w) * ROPE_PAIRS + 16 * (c & 1), o0, o1);
+            *reinterpret_cast<u32x4*>(q_s + (4 * w + rr) * KL_LD + 16 * c) = o0;
+            *reinterpret_cast<u32x4*>(q_s + (4 * w + rr) * KL_LD + 16 * c + 8) = o1;
+        }
+        if (first && w == 0) {
+            const int key = rr < M ? rr : 0;                      // (idle groups work on a copy of key 0 and store nothing)
+            u32x4 o0, o1;
+            glue16(q + (size_t)(b * Mtot + j0 + key) * QKV_W + AH * 2 * AD + kvh * AD + 16 * c, k_norm + 16 * c,
+                   rope_tab + (size_t)(p0 + key) * ROPE_PAIRS + 16 * (c & 1), o0, o1);
+            if (rr < M) {
+                *reinterpret_cast<u32x4*>(k_s + rr * KL_LD + 16 * c) = o0;
+                *reinterpret_cast<u32x4*>(k_s + rr * KL_LD + 16 * c + 8) = o1;
+                *reinterpret_cast<u32x4*>(Kp + pbase + (size_t)(p0 + rr) * AD + 16 * c) = o0;
+                *reinterpret_cast<u32x4*>(Kp + pbase + (size_t)(p0 + rr) * AD + 16 * c + 8) = o1;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kb = 0; kb < 8; kb++) bq[kb] = as_bf16x8(*reinterpret_cast<const u32x4*>(q_s + n * KL_LD + 32 * kb + 8 * g));
+        if (first && w == 3) {                                    // the new keys as the A operand of their scores, parked in `a`
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) {
+                u32x4 v = *reinterpret_cast<const u32x4*>(k_s + (n & 3) * KL_LD + 32 * kb + 8 * g);
+                if (n >= M) v = u32x4{0, 0, 0, 0};
+                knew[kb] = v;
+            }
+        }
+    } else {
         const bool real = n < R;
         const bf16_t* qr = q + ((size_t)(b * Mtot + j0 + (real ? n / GQA : 0)) * AH + kvh * GQA + (n % GQA)) * AD;
 #pragma unroll
@@ -205,25 +315,13 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
 #pragma unroll
     for (int j = 0; j < 16; j++) O[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const size_t pbase = ((size_t)slot * AKV + kvh) * Lmax * AD;
-    const bf16_t* kbase = Kp + pbase;
-    const bf16_t* vbase = Vp + pbase;
-    bf16_t* vl = tile_s + w * (16 * VL_LD);
-    bf16_t* kl = tile_s + 4 * (16 * VL_LD) + w * (16 * KL_LD);
-    const int ntiles = hi > lo ? (hi - lo + 15) / 16 : 0;
     if (w < ntiles) {
-        // Row addresses of a tile: key 2i (lower half wavefront) / 2i + 1 (upper half), 8 columns per lane, so one load covers
-        // two whole 512-byte rows (a wavefront-wide load of 16 rows x 64 bytes streams about 15 % slower from HBM).  Keys past
-        // `hi` re-read the tile's first key (they are masked / weighted by 0).
-        auto row_ptr = [&](const bf16_t* base, int t, int i) {
-            const int key0 = lo + t * 16, key = key0 + 2 * i + hw;
-            return reinterpret_cast<const u32x4*>(base + (size_t)(key < hi ? key : key0) * AD) + cl;
-        };
-        u32x4 a[8], vv[8];
+        if constexpr (!LAYER) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) a[i] = __builtin_nontemporal_load(row_ptr(kbase, w, i));
+            for (int i = 0; i < 8; i++) a[i] = __builtin_nontemporal_load(row_ptr(kbase, w, i));
 #pragma unroll
-        for (int i = 0; i < 8; i++) vv[i] = __builtin_nontemporal_load(row_ptr(vbase, w, i));
+            for (int i = 0; i < 8; i++) vv[i] = __builtin_nontemporal_load(row_ptr(vbase, w, i));
+        }
         __builtin_amdgcn_sched_barrier(0);
         for (int t = w; t < ntiles; t += 4) {
             const int tn = t + 4 < ntiles ? t + 4 : t;           // the last step re-reads its own tile
@@ -258,11 +356,16 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     if (first && w == 3) {
         // The M new keys of this sequence, straight from the inputs (batch.py:143-145), with the causal rule among them:
         // key i is visible to query token j only if i <= j.  Not pipelined: it runs once per sequence.
-        const bf16_t* kn = k_new + ((size_t)(b * Mtot + j0) * AKV + kvh) * AD;
-        const bf16_t* vn = v_new + ((size_t)(b * Mtot + j0) * AKV + kvh) * AD;
-        const size_t stride = (size_t)AKV * AD;
+        const bf16_t* kn = LAYER ? q + (size_t)(b * Mtot + j0) * QKV_W + AH * 2 * AD + kvh * AD
+                                 : k_new + ((size_t)(b * Mtot + j0) * AKV + kvh) * AD;
+        const bf16_t* vn = LAYER ? q + (size_t)(b * Mtot + j0) * QKV_W + AH * 2 * AD + AKV * AD + kvh * AD
+                                 : v_new + ((size_t)(b * Mtot + j0) * AKV + kvh) * AD;
+        const size_t stride = LAYER ? (size_t)QKV_W : (size_t)AKV * AD;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        {
+        if constexpr (LAYER) {
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(knew[kb]), bq[kb], acc, 0, 0, 0);
+        } else {
             const u32x4* kr = reinterpret_cast<const u32x4*>(kn + (size_t)(n < M ? n : 0) * stride);
             u32x4 a[8];
 #pragma unroll
@@ -286,10 +389,15 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
     if (first && w == 0) {
         // append (batch.py:196-201): row j of this sequence goes to pool position p0 + j
         for (int j = 0; j < M; j++) {
-            const uint2 kk = reinterpret_cast<const uint2*>(k_new + ((size_t)(b * Mtot + j0 + j) * AKV + kvh) * AD)[lane];
-            const uint2 vv2 = reinterpret_cast<const uint2*>(v_new + ((size_t)(b * Mtot + j0 + j) * AKV + kvh) * AD)[lane];
-            reinterpret_cast<uint2*>(Kp + pbase + (size_t)(p0 + j) * AD)[lane] = kk;
-            reinterpret_cast<uint2*>(Vp + pbase + (size_t)(p0 + j) * AD)[lane] = vv2;
+            if constexpr (LAYER) {                               // (the keys are appended by the wavefront that norms them)
+                const uint2 vv2 = reinterpret_cast<const uint2*>(q + (size_t)(b * Mtot + j0 + j) * QKV_W + AH * 2 * AD + AKV * AD + kvh * AD)[lane];
+                reinterpret_cast<uint2*>(Vp + pbase + (size_t)(p0 + j) * AD)[lane] = vv2;
+            } else {
+                const uint2 kk = reinterpret_cast<const uint2*>(k_new + ((size_t)(b * Mtot + j0 + j) * AKV + kvh) * AD)[lane];
+                const uint2 vv2 = reinterpret_cast<const uint2*>(v_new + ((size_t)(b * Mtot + j0 + j) * AKV + kvh) * AD)[lane];
+                reinterpret_cast<uint2*>(Kp + pbase + (size_t)(p0 + j) * AD)[lane] = kk;
+                reinterpret_cast<uint2*>(Vp + pbase + (size_t)(p0 + j) * AD)[lane] = vv2;
+            }
         }
     }
 
@@ -338,16 +446,22 @@ __global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __re
 // computed by one thread each; then wavefront w sums the partials s = w, w+4, ... (a lane owns 4 output columns, four
 // partials' loads in flight) and the four wavefronts are added in order.
 constexpr int MAX_SPLITS = 4096;
-template <int M>
+// GATE: out [R,2048] = BF(o * sigmoid_bf16(gate)) with the row's gate from its qkv row (qwen35/batch.py:513), value for value what
+// attn_out_gate_kernel makes of the bf16 o that this kernel would store otherwise.
+template <int M, bool GATE>
 __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                          const int* __restrict__ seg_tab, bf16_t* __restrict__ out, int B, int nwg,
-                                                         int min_tiles, int Mtot, int j0) {
+                                                         int min_tiles, int Mtot, int j0, const bf16_t* __restrict__ qkv) {
     constexpr int R = 4 * M;
     __shared__ float fs_s[MAX_SPLITS];
     __shared__ float red_m[4], red_l[4];
     __shared__ __align__(16) float acc_s[4][AD];
     const int r = blockIdx.x % R, sg = blockIdx.x / R, kvh = sg % AKV, b = sg / AKV;
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
+    const size_t row = (size_t)(b * Mtot + j0 + r / GQA);
+    const int head = kvh * GQA + (r % GQA);
+    bf16_t gate_raw = 0;
+    if constexpr (GATE) gate_raw = qkv[row * QKV_W + head * 2 * AD + AD + tid];   // requested first, needed last
     const int total = seg_tab[B * AKV], ss = seg_tab[sg], se = seg_tab[sg + 1];   // written by the partial kernel
     if (se == ss) return;                                        // a skipped row
     const int per = tiles_per_wg(total, nwg, min_tiles);
@@ -386,7 +500,11 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
     const int d = tid;
     const float a = (acc_s[0][d] + acc_s[1][d]) + (acc_s[2][d] + acc_s[3][d]);
     const float ov = l == 0.f ? a : a / l;                                           // batch.py:216
-    out[((size_t)(b * Mtot + j0 + r / GQA) * AH + kvh * GQA + (r % GQA)) * AD + d] = f2bf(ov);
+    if constexpr (GATE) {
+        out[(row * AH + head) * AD + d] = f2bf(BF(ov) * sigmoid_bf16(bf2f(gate_raw)));
+    } else {
+        out[(row * AH + head) * AD + d] = f2bf(ov);
+    }
 }
 
 }  // namespace
@@ -415,20 +533,30 @@ long qt_gqa_attn_workspace_bytes(int B, int M, int Lmax, int CH) {
 
 // Both entry points: checks, grid size and the two launches.  The partial results of at most `slot_cap` slots
 // (slot = workgroup + segment < grid + 2 B) start at part_o / part_ml; seg_tab holds 2 B + 1 ints.
+struct LayerArgs {                      // the layer form's extra operands (null q_norm: the plain form)
+    const bf16_t* q_norm;
+    const bf16_t* k_norm;
+    const float2* rope_tab;
+    float eps;
+};
+
 static int attn_launch(const void* q, const void* k_new, const void* v_new, void* Kp, void* Vp, const int32_t* slots,
                        const int32_t* pos, void* out, float* part_o, float* part_ml, int* seg_tab, int max_grid, int B, int M,
-                       int Lmax, int n_slots, int CH, hipStream_t stream) {
+                       int Lmax, int n_slots, int CH, hipStream_t stream, LayerArgs la = LayerArgs{nullptr, nullptr, nullptr, 0.f}) {
     const int min_tiles = CH / 16;                               // a workgroup takes at least CH keys
     const long max_tiles = (long)B * AKV * ((Lmax + 15) / 16);
     const long want = (max_tiles + min_tiles - 1) / min_tiles;
     const int nwg = (int)(want < max_grid ? want : max_grid);
     const dim3 g1((unsigned)nwg);
-#define QT_ATTN_LAUNCH(MM)                                                                                                \
-    hipLaunchKernelGGL(attn_partial_kernel<MM>, g1, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)k_new,         \
+    const bool layer = la.q_norm != nullptr;
+#define QT_ATTN_LAUNCH2(MM, LY)                                                                                           \
+    hipLaunchKernelGGL((attn_partial_kernel<MM, LY>), g1, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)k_new,   \
                        (const bf16_t*)v_new, (bf16_t*)Kp, (bf16_t*)Vp, slots, pos, part_o, part_ml, seg_tab, B, Lmax, min_tiles,    \
-                       n_slots, M, j0);                                                                                   \
-    hipLaunchKernelGGL(attn_merge_kernel<MM>, dim3((unsigned)(B * AKV * 4 * MM)), dim3(256), 0, stream, part_o, part_ml, seg_tab,   \
-                       (bf16_t*)out, B, nwg, min_tiles, M, j0);
+                       n_slots, M, j0, la.q_norm, la.k_norm, la.rope_tab, la.eps);                                        \
+    hipLaunchKernelGGL((attn_merge_kernel<MM, LY>), dim3((unsigned)(B * AKV * 4 * MM)), dim3(256), 0, stream, part_o, part_ml,      \
+                       seg_tab, (bf16_t*)out, B, nwg, min_tiles, M, j0, (const bf16_t*)q);
+#define QT_ATTN_LAUNCH(MM)                                                                                                \
+    if (layer) { QT_ATTN_LAUNCH2(MM, true) } else { QT_ATTN_LAUNCH2(MM, false) }
     for (int j0 = 0; j0 < M; j0 += MAX_PASS_M) {                 // passes of up to four tokens per sequence
         switch (M - j0 < MAX_PASS_M ? M - j0 : MAX_PASS_M) {
             case 1: QT_ATTN_LAUNCH(1) break;
@@ -439,6 +567,7 @@ static int attn_launch(const void* q, const void* k_new, const void* v_new, void
         QT_CHECK_LAUNCH();
     }
 #undef QT_ATTN_LAUNCH
+#undef QT_ATTN_LAUNCH2
     return QT_OK;
 }
 
@@ -467,6 +596,29 @@ int qt_gqa_attn_decode(const void* q, const void* k_new, const void* v_new, void
     int* seg_tab = reinterpret_cast<int*>(part_ml + cap * (4 * mp) * 2);
     return attn_launch(q, k_new, v_new, Kp, Vp, slots, pos, out, part_o, part_ml, seg_tab, partial_grid(), B, M, Lmax, n_slots, CH,
                        stream);
+}
+
+// The attention half of a full-attention layer at a decode / verify step in two launches per pass: q / k RMSNorm, rotary
+// embedding, the split of the qkv rows, attn_b and the output gate (qwen35/batch.py:505-513).
+long qt_rope_table_bytes(int n_pos) { return n_pos < 0 ? -1 : (long)n_pos * ROPE_PAIRS * (long)sizeof(float2); }
+
+int qt_gqa_attn_layer_decode(const void* qkv, const void* q_norm, const void* k_norm, const void* rope_table, int table_positions,
+                             void* Kp, void* Vp, const int32_t* slots, const int32_t* pos, void* out, void* workspace,
+                             long workspace_bytes, int B, int M, int Lmax, int n_slots, int CH, float eps, hipStream_t stream) {
+    if (!workspace || !q_norm || !k_norm || !rope_table) return QT_ERR_NULL;
+    if (const int rc = attn_check(qkv, qkv, qkv, Kp, Vp, slots, pos, out, B, M, Lmax, n_slots, CH)) return rc;
+    if (table_positions < Lmax) return QT_ERR_DIM;               // every position a row can sit at has its (cos, sin) pairs
+    if (B == 0) return QT_OK;
+    for (const void* p : {(const void*)workspace, q_norm, k_norm, rope_table, (const void*)out})
+        if (reinterpret_cast<uintptr_t>(p) & 15u) return QT_ERR_ALIGN;
+    if (workspace_bytes < qt_gqa_attn_workspace_bytes(B, M, Lmax, CH)) return -6;
+    const size_t cap = (size_t)MAX_WG + (size_t)B * AKV;
+    const int mp = M < MAX_PASS_M ? M : MAX_PASS_M;
+    float* part_o = (float*)workspace;
+    float* part_ml = part_o + cap * (4 * mp) * AD;
+    int* seg_tab = reinterpret_cast<int*>(part_ml + cap * (4 * mp) * 2);
+    return attn_launch(qkv, nullptr, nullptr, Kp, Vp, slots, pos, out, part_o, part_ml, seg_tab, partial_grid(), B, M, Lmax, n_slots,
+                       CH, stream, LayerArgs{(const bf16_t*)q_norm, (const bf16_t*)k_norm, (const float2*)rope_table, eps});
 }
 
 // ---- the same operator for callers that cannot allocate: the partial results live in a static device array -------------------

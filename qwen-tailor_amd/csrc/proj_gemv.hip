@@ -227,16 +227,22 @@ __global__ __launch_bounds__(64 * NWV) void wide_gemm_kernel(const bf16_t* __res
 // wavefront's W block [16 features][1024] is 32 loads, all issued up front (128 registers); every W fragment then meets MS
 // x fragments read from LDS.  Accumulator element i of lane (n, g) is feature 4 g + i of row 16 ms + n: four adjacent
 // features, stored as 8 bytes.  grid = ceil(N / (16 WPB)), block = 64 WPB.
+// With `full` > 0 the launch is one workgroup for every CU whatever N: wavefronts 0 .. WPB - 2 of workgroup i take feature
+// blocks (WPB - 1) i + w, and the last wavefront takes block `full` + i, which exists in the first few workgroups only (the
+// 514 blocks of N = 8224 are 2 x 256 + 2: with three blocks per workgroup 84 of 256 CUs would have none, and what bounds the
+// launch is the bytes one CU has to pull in).  A wavefront without a block still helps to bring in the rows.
 constexpr int XK = 1024;
 template <int MS, int WPB, int EPI>
 __global__ __launch_bounds__(64 * WPB) void xlds_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ x,
-                                                        const bf16_t* __restrict__ res, bf16_t* __restrict__ y, int M, int N) {
+                                                        const bf16_t* __restrict__ res, bf16_t* __restrict__ y, int M, int N, int full) {
     __shared__ __align__(1024) bf16_t x_s[16 * MS * XK];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
-    const int n0 = (blockIdx.x * WPB + w) * 16;                   // this wavefront's feature block (may lie past N)
+    // this wavefront's feature block (may lie past N: then it multiplies a copy of the last row block and stores nothing)
+    const int n0 = 16 * (full <= 0 ? blockIdx.x * WPB + w : w < WPB - 1 ? blockIdx.x * (WPB - 1) + w : full + blockIdx.x);
     // W first (it comes from HBM): the wavefront's block is 32 loads, all in flight at once
     u32x4 a[XK / 32];
-    {
+    const bool has_block = n0 < N;                                // (the same for the whole wavefront)
+    if (has_block) {
         const bf16_t* wp = W + (size_t)min(n0 + n, N - 1) * XK + 8 * g;
 #pragma unroll
         for (int c = 0; c < XK / 32; c++) a[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + 32 * c));
@@ -253,6 +259,7 @@ __global__ __launch_bounds__(64 * WPB) void xlds_gemm_kernel(const bf16_t* __res
     // products cannot start under the tail of the W stream; both streams are drained here)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    if (!has_block) return;                                       // it has done its share of the rows
     f32x4 acc[MS];
 #pragma unroll
     for (int ms = 0; ms < MS; ms++) acc[ms] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -299,26 +306,38 @@ __global__ __launch_bounds__(64 * WPB) void xlds_gemm_kernel(const bf16_t* __res
 }
 
 template <int MS, int WPB>
-void launch_xlds_wpb(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, bf16_t* y, int M, int N, hipStream_t stream) {
-    const int blocks = (N + 15) / 16;
-    const dim3 grid((blocks + WPB - 1) / WPB), block(64 * WPB);
+void launch_xlds_wpb(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, bf16_t* y, int M, int N, hipStream_t stream, int grid_x,
+                     int full) {
+    const dim3 grid(grid_x), block(64 * WPB);
     if (epi == EPI_NONE)
-        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_NONE>), grid, block, 0, stream, W, x, res, y, M, N);
+        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_NONE>), grid, block, 0, stream, W, x, res, y, M, N, full);
     else if (epi == EPI_ADD)
-        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_ADD>), grid, block, 0, stream, W, x, res, y, M, N);
+        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_ADD>), grid, block, 0, stream, W, x, res, y, M, N, full);
     else
-        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_SWIGLU>), grid, block, 0, stream, W, x, res, y, M, N);
+        hipLaunchKernelGGL((xlds_gemm_kernel<MS, WPB, EPI_SWIGLU>), grid, block, 0, stream, W, x, res, y, M, N, full);
 }
 template <int MS>
 void launch_xlds_ms(int epi, const bf16_t* W, const bf16_t* x, const bf16_t* res, bf16_t* y, int M, int N, hipStream_t stream, int cus) {
     // as few wavefronts per workgroup as keep the launch within one workgroup per CU (the rows take most of a CU's LDS)
     const int blocks = (N + 15) / 16, wpb = (blocks + cus - 1) / cus;
+    // a few blocks more than a whole number per CU: every CU gets that number, the first few workgroups one more
+    const int base = blocks / cus, rest = blocks - base * cus;
+    if (base >= 1 && base <= 3 && rest > 0 && rest <= cus / 16) {
+        const int full = base * cus;
+        if (base == 1)
+            launch_xlds_wpb<MS, 2>(epi, W, x, res, y, M, N, stream, cus, full);
+        else if (base == 2)
+            launch_xlds_wpb<MS, 3>(epi, W, x, res, y, M, N, stream, cus, full);
+        else
+            launch_xlds_wpb<MS, 4>(epi, W, x, res, y, M, N, stream, cus, full);
+        return;
+    }
     if (wpb <= 2)
-        launch_xlds_wpb<MS, 2>(epi, W, x, res, y, M, N, stream);
+        launch_xlds_wpb<MS, 2>(epi, W, x, res, y, M, N, stream, (blocks + 1) / 2, 0);
     else if (wpb == 3)
-        launch_xlds_wpb<MS, 3>(epi, W, x, res, y, M, N, stream);
+        launch_xlds_wpb<MS, 3>(epi, W, x, res, y, M, N, stream, (blocks + 2) / 3, 0);
     else
-        launch_xlds_wpb<MS, 4>(epi, W, x, res, y, M, N, stream);
+        launch_xlds_wpb<MS, 4>(epi, W, x, res, y, M, N, stream, (blocks + 3) / 4, 0);
 }
 
 // row blocks per pass: 1, 2 or 4 (3 rounds up)

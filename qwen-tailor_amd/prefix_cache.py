@@ -67,8 +67,10 @@ def common_prefix(a, b):
 
 
 class PrefixCache:
-    MIN_SPLIT = 32        # a shared prefix shorter than this is not worth a checkpoint of its own   (prefix_cache.py:56)
-    MIN_GAIN = 32         # ... nor one that saves fewer tokens than this over the best existing hit  (prefix_cache.py:57)
+    # thresholds of split learning, in tokens (values of qwen35/prefix_cache.py:58-59): the common prefix of two prompts becomes a
+    # checkpoint only if it is at least MIN_SPLIT long and reaches at least MIN_GAIN past the checkpoint a lookup already hits
+    MIN_SPLIT = 32
+    MIN_GAIN = 32
 
     def __init__(self, budget_mb=1024):
         self.budget = int(budget_mb * (1 << 20))
@@ -140,15 +142,21 @@ class PrefixCache:
 
     @staticmethod
     def cat_rows(chain, get, total, axis):
-        """Concatenate the per-node segments `get(node)` ([..., n, ...] tensors or None) along `axis`, zero-padded to `total`
-        rows (qwen35/prefix_cache.py:128-137; the owning engine uses it for its `extra` segments)."""
-        parts = [g for g in (get(c) for c in chain) if g is not None]
-        have = sum(p.shape[axis] for p in parts)
-        if total > have:
-            shp = list(parts[0].shape)
-            shp[axis] = total - have
-            parts.append(torch.zeros(shp, dtype=parts[0].dtype, device=parts[0].device))
-        return torch.cat(parts, dim=axis) if len(parts) > 1 else parts[0]
+        """The segments `get(node)` of the nodes of `chain` (tensors that differ along `axis` only; None = the node has none)
+        laid end to end along `axis` in one tensor of `total` rows, the rows past the last segment zero (the role of
+        qwen35/prefix_cache.py:124-132; the owning engine uses it for its `extra` segments).  At least one node must have a segment."""
+        segs = [t for t in map(get, chain) if t is not None]
+        first = segs[0]
+        shape = list(first.shape)
+        shape[axis] = max(total, sum(t.shape[axis] for t in segs))
+        if len(segs) == 1 and shape[axis] == first.shape[axis]:
+            return first
+        out = torch.zeros(shape, dtype=first.dtype, device=first.device)
+        at = 0
+        for t in segs:
+            out.narrow(axis, at, t.shape[axis]).copy_(t)
+            at += t.shape[axis]
+        return out
 
     def restore(self, node, max_len):
         """(state, chain): the state dict of the checkpoint ({"kv": [(K, V)] x6 [1,2,max_len,256], "conv": [...], "ssm": [...]}),

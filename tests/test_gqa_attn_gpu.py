@@ -405,3 +405,54 @@ def test_attention_layer_core_decode_rows(qt, dev):
     oo = O.attn_b(oq, ok, ov, Kp, Vp, slots, pos, 1)
     check_rel("layer core", to_np(out), O.attn_out_gate(oo, qkv), 1e-2, rel_max)
     check_equal("appended K", to_np(dK), Kp)                                   # the oracle appended the same rows in place
+
+
+def _layer_case(qt, dev, seed, B, M, Lmax, lo, hi, bad=False):
+    """the three-call chain (qkv_prep, attn_b, out_gate) and the two-launch layer form on the same inputs; returns both results"""
+    rng = np.random.default_rng(seed)
+    S = B + 2
+    slots = rng.permutation(S)[:B].astype(np.int32)
+    pos = rng.integers(lo, hi, B).astype(np.int32)
+    pos[0] = lo
+    if bad:
+        slots[1], pos[B - 1] = S + 3, Lmax - M + 1                              # skipped rows: outputs undefined, pools untouched
+    qkv = bf(rng.standard_normal((B * M, O.QKV_W)) * 1.5)
+    qn, kn = bf(1 + 0.2 * rng.standard_normal(256)), bf(1 + 0.2 * rng.standard_normal(256))
+    Kp = to_dev(bf(rng.standard_normal((S + 1, 2, Lmax, 256))), dev, BF16)
+    Vp = to_dev(bf(rng.standard_normal((S + 1, 2, Lmax, 256))), dev, BF16)
+    dq, dqn, dkn, dslots, dpos = to_dev(qkv, dev, BF16), to_dev(qn, dev, BF16), to_dev(kn, dev, BF16), to_dev(slots, dev), to_dev(pos, dev)
+    K1, V1 = Kp.clone(), Vp.clone()
+    q, k, v = qt.attention.qkv_prep(dq, dqn, dkn, dpos, M)
+    want = qt.attention.out_gate(qt.batch.attn_b(q, k, v, K1, V1, dslots, dpos, M), dq)
+    K2, V2 = Kp.clone(), Vp.clone()
+    got = qt.batch.attn_layer_b(dq, dqn, dkn, K2, V2, dslots, dpos, M)
+    good = np.ones(B, bool)
+    if bad:
+        good[[1, B - 1]] = False
+    rows = torch.from_numpy(np.flatnonzero(np.repeat(good, M))).to(dev)
+    check_tensors_equal(f"layer form, outputs (B={B}, M={M})", got[rows], want[rows])
+    check_tensors_equal("layer form, K pool", K2, K1)
+    check_tensors_equal("layer form, V pool", V2, V1)
+    return qkv, qn, kn, slots, pos, to_np(Kp), to_np(Vp), to_np(got), good
+
+
+@pytest.mark.parametrize("B,M,Lmax,lo,hi", [(5, 1, 256, 0, 250), (6, 4, 1024, 0, 1000), (3, 2, 96, 0, 90), (16, 3, 640, 0, 600),
+                                            (40, 1, 640, 0, 630), (130, 2, 200, 0, 190), (4, 7, 300, 0, 290), (2, 16, 128, 0, 100)])
+def test_attention_layer_two_launches_equal_the_three_calls(qt, dev, B, M, Lmax, lo, hi):
+    """batch.attn_layer_b (q / k norm and rotary embedding inside the attention kernel, the output gate in the merge) against
+    attention.qkv_prep -> batch.attn_b -> attention.out_gate: the same bits in the outputs and in the pools, also with skipped
+    rows, with more segments than workgroups and with more than four tokens per sequence; and against the oracle chain"""
+    qkv, qn, kn, slots, pos, Kp, Vp, got, good = _layer_case(qt, dev, 500 + B + M, B, M, Lmax, lo, hi, bad=B >= 5)
+    if B * M <= 64:
+        keep = np.flatnonzero(good)
+        rows = (keep[:, None] * M + np.arange(M)[None]).ravel()
+        oq, ok, ov = O.attn_qkv_prep(qkv[rows], qn, kn, pos[keep], M)
+        oo = O.attn_b(oq, ok, ov, Kp, Vp, slots[keep], pos[keep], M)
+        ref = O.attn_out_gate(oo, qkv[rows])
+        for i, r in enumerate(rows):
+            check_attn(f"row {r} against the oracle chain", got[r], ref[i])
+
+
+def test_attention_layer_config4_two_launches(qt, dev):
+    """benchmark config 4's attention half (B = 16 x M = 4, ragged lengths in [1024, 8192]) through the layer form"""
+    _layer_case(qt, dev, 1004, 16, 4, 8192 + 8, 1024, 8192)
