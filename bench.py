@@ -476,6 +476,10 @@ def profile_leg(torch, qt, dev, args):
             l = i % N_LAYERS
             qt.batch.deltanet_b(st["proj"][l & 3], st["conv"][l], st["cw"][l], st["A_log"][l], st["dtb"][l], st["ssm"][l], st["slots"],
                                 st["pos"][(i // N_LAYERS) & 1])
+    elif leg == "decode_graph":
+        # the headline's launch form: HIP graphs of 18 launches (one per layer pool), replayed
+        st = build_decode_state(torch, dev, args.batch, N_LAYERS)
+        time_decode(torch, qt, st, args.batch, N_LAYERS, 18 * max(1, n // 18), 36, use_graph=True, min_total_s=0.0, max_regions=3)
     elif leg == "copy":
         # plain copy of known size: the scale factor for the FETCH_SIZE / WRITE_SIZE counters (64 MiB read + 64 MiB written)
         src = [torch.randn(16 * 1024 * 1024, device=dev) for _ in range(N_LAYERS)]
@@ -483,10 +487,9 @@ def profile_leg(torch, qt, dev, args):
         for i in range(n):
             dst[i & 1].copy_(src[i % N_LAYERS])
     elif leg == "prefill":
-        for _ in range(3):
-            bench_prefill_once(torch, qt, dev, 2048)
+        bench_prefill_once(torch, qt, dev, 2048, calls=20)
     elif leg == "prefill_long":
-        bench_prefill_once(torch, qt, dev, 8192)
+        bench_prefill_once(torch, qt, dev, 8192, calls=10)
     elif leg == "verify":
         bench_verify_gdn(torch, qt, dev)
     elif leg == "attn_decode":
@@ -513,16 +516,20 @@ def profile_leg(torch, qt, dev, args):
     print(json.dumps({"profiled": leg, "launches": n}))
 
 
-def bench_prefill_once(torch, qt, dev, T, seed=1002):
+def bench_prefill_once(torch, qt, dev, T, seed=1002, calls=15):
+    """the layer core over T tokens, launched eagerly `calls` times on input sets that rotate past the last-level cache"""
     g = torch.Generator().manual_seed(seed)
     bf = torch.bfloat16
-    proj = torch.randn((T, PW), generator=g).to(bf).to(dev)
-    cs = torch.randn((1, 3, CD), generator=g).to(bf).to(dev)
+    n_sets = max(8, -(-(LLC_BYTES + LLC_BYTES // 4) // (T * PW * 2)))
+    base = torch.randn((T, PW), generator=g).to(bf)
+    sets = [(torch.roll(base, shifts=i * 37, dims=0).to(dev), torch.randn((1, 3, CD), generator=g).to(bf).to(dev),
+             (torch.randn((1, HV, DV, DK), generator=g) * 0.02).to(dev)) for i in range(n_sets)]
     cw = (torch.randn((CD, 4), generator=g) * 0.5).to(bf).to(dev)
     A, dtb = (torch.rand(HV, generator=g) * 2.7).to(dev), (torch.randn(HV, generator=g) * 0.1).to(dev)
-    S0 = (torch.randn((1, HV, DV, DK), generator=g) * 0.02).to(dev)
-    for _ in range(5):
-        qt.prefill.gdn_core(proj, cs, S0, cw, A, dtb, torch.ones(DV, device=dev))
+    gw = torch.ones(DV, device=dev)
+    for i in range(calls):
+        proj, cs, S0 = sets[i % n_sets]
+        qt.prefill.gdn_core(proj, cs, S0, cw, A, dtb, gw)
 
 
 def main():
@@ -535,7 +542,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the B sweep and the single-pool run")
     ap.add_argument("--only", default="", help="profile helper: run only one leg a few times and exit "
-                                               "(decode | copy | prefill | prefill_long | verify | attn_decode | attn_verify | attn_layer | attn_prefill | attn_prefill_long | "
+                                               "(decode | decode_graph | copy | prefill | prefill_long | verify | attn_decode | attn_verify | attn_layer | attn_prefill | attn_prefill_long | "
                                                "projections | state_admission | prefix_cache | attn_glue)")
     args = ap.parse_args()
     if args.gpus != 1:

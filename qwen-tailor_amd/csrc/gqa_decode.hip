@@ -151,9 +151,8 @@ __device__ __forceinline__ int tiles_per_wg(int total, int nwg, int min_tiles) {
 // part_o [slot][4*M rows][256] f32 (unnormalised), part_ml [slot][4*M][2] = (running max, running sum)
 // LAYER: q is the layer's qkv rows [B*Mtot, 5120]; the query rows and the new keys are normed and roped here, the
 // new values are read from the rows' v part, and k_new / v_new are not used.
-// (one workgroup per CU in that form: it holds the staged query rows in LDS beside the tiles)
 template <int M, bool LAYER>
-__global__ __launch_bounds__(256, LAYER ? 1 : 2) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_new,
+__global__ __launch_bounds__(256, 2) void attn_partial_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_new,
                                                            const bf16_t* __restrict__ v_new, bf16_t* Kp, bf16_t* Vp,
                                                            const int* __restrict__ slots, const int* __restrict__ pos,
                                                            float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -216,7 +215,13 @@ __global__ __launch_bounds__(256, LAYER ? 1 : 2) void attn_partial_kernel(const 
 
     // Q^T as the MFMA B operand: lane (row n, group g) holds q[row n][32 kb + 8 g .. + 8]; row n = token (n / 4), head n % 4
     bf16x8 bq[8];
-    u32x4 knew[8];                                                // (layer form: the new keys, wavefront 3 of the first workgroup)
+    // layer form: the staged query rows lie in wavefront 0's V tile (the tiles are not in use yet), the staged new keys in an
+    // array of their own (they are read after the tile loop).  With the query rows in an array of their own the workgroup's LDS
+    // would pass half of a CU's: the compiler then plans for one workgroup per CU and all 512 registers, puts O into the
+    // accumulation registers, and the rescale of O in the tile loop costs a register copy each way (+4 us per launch).
+    __shared__ __align__(16) bf16_t k_s[LAYER ? 4 * KL_LD : 8];
+    bf16_t* const q_s = tile_s;
+    static_assert(16 * KL_LD <= 16 * VL_LD, "the staged query rows must fit into one V tile");
     if constexpr (LAYER) {
         // The wavefront's first tile is requested before anything else: the norm and the rotary embedding below run while it
         // is on its way from HBM.
@@ -233,7 +238,6 @@ __global__ __launch_bounds__(256, LAYER ? 1 : 2) void attn_partial_kernel(const 
         // per 16-lane group), which it also appends to the pool (batch.py:196-201).  Same arithmetic, value for value, as
         // attn_qkv_prep_kernel: sum of squares exact in double and rounded once, correctly rounded 1 / sqrt,
         // BF(w * BF(x * inv)), rotary products and sums rounded one by one; (cos, sin) from the table qt_rope_table_build wrote.
-        __shared__ __align__(16) bf16_t q_s[16 * KL_LD], k_s[4 * KL_LD];
         const int rr = lane >> 4, c = lane & 15;
         auto glue16 = [&](const bf16_t* x, const bf16_t* wgt, const float2* cs, u32x4& o0, u32x4& o1) {
             const u32x4 x0 = reinterpret_cast<const u32x4*>(x)[0], x1 = reinterpret_cast<const u32x4*>(x)[1];
@@ -292,14 +296,7 @@ __global__ __launch_bounds__(256, LAYER ? 1 : 2) void attn_partial_kernel(const 
         __syncthreads();
 #pragma unroll
         for (int kb = 0; kb < 8; kb++) bq[kb] = as_bf16x8(*reinterpret_cast<const u32x4*>(q_s + n * KL_LD + 32 * kb + 8 * g));
-        if (first && w == 3) {                                    // the new keys as the A operand of their scores, parked in `a`
-#pragma unroll
-            for (int kb = 0; kb < 8; kb++) {
-                u32x4 v = *reinterpret_cast<const u32x4*>(k_s + (n & 3) * KL_LD + 32 * kb + 8 * g);
-                if (n >= M) v = u32x4{0, 0, 0, 0};
-                knew[kb] = v;
-            }
-        }
+        __syncthreads();                                          // every wavefront has its rows: wavefront 0 may park its first tile there
     } else {
         const bool real = n < R;
         const bf16_t* qr = q + ((size_t)(b * Mtot + j0 + (real ? n / GQA : 0)) * AH + kvh * GQA + (n % GQA)) * AD;
@@ -362,9 +359,13 @@ __global__ __launch_bounds__(256, LAYER ? 1 : 2) void attn_partial_kernel(const 
                                  : v_new + ((size_t)(b * Mtot + j0) * AKV + kvh) * AD;
         const size_t stride = LAYER ? (size_t)QKV_W : (size_t)AKV * AD;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (LAYER) {
+        if constexpr (LAYER) {                                    // the new keys as wavefront 0 left them in LDS
 #pragma unroll
-            for (int kb = 0; kb < 8; kb++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(knew[kb]), bq[kb], acc, 0, 0, 0);
+            for (int kb = 0; kb < 8; kb++) {
+                u32x4 v = *reinterpret_cast<const u32x4*>(k_s + (n & 3) * KL_LD + 32 * kb + 8 * g);
+                if (n >= M) v = u32x4{0, 0, 0, 0};
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(v), bq[kb], acc, 0, 0, 0);
+            }
         } else {
             const u32x4* kr = reinterpret_cast<const u32x4*>(kn + (size_t)(n < M ? n : 0) * stride);
             u32x4 a[8];
