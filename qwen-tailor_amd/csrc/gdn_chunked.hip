@@ -530,10 +530,8 @@ __global__ __launch_bounds__(384) void gdn_chain_kernel(const _Float16* ops, con
     __shared__ ChainLds chain_lds;
     chain_role<false, 4>(chain_lds, blockIdx.x, ops, U, gates, st_in, st_out, snap + FLAG_HALVES, reinterpret_cast<int*>(snap), NC);
 }
-// (two workgroups per SIMD's worth of registers at most: with all 512 to itself the compiler keeps the MFMA results in the
-// accumulation registers, which the gamma scaling and the conversion to bf16 can only reach through copies)
 template <bool NORM>
-__global__ __launch_bounds__(256, 2) void gdn_output_kernel(const _Float16* __restrict__ ops, const _Float16* __restrict__ snap,
+__global__ __launch_bounds__(256) void gdn_output_kernel(const _Float16* __restrict__ ops, const _Float16* __restrict__ snap,
                                                          const float* __restrict__ gates, bf16_t* __restrict__ y,
                                                          const bf16_t* __restrict__ proj, const float* __restrict__ gw, float eps,
                                                          int S, int NC) {
