@@ -21,13 +21,13 @@ if ROOT not in sys.path:
 HV, DK, DV, CD, PW = 16, 128, 128, 6144, 8224
 N_LAYERS = 18
 HBM_PEAK_GBS = 8000.0
-# HBM bytes of one B = 64 decode launch measured with rocprofv3 --pmc (FETCH_SIZE 34 563.5 KiB x 1.9993 + WRITE_SIZE 68 142.9 KiB,
+# HBM bytes of one B = 64 decode launch measured with rocprofv3 --pmc (FETCH_SIZE 34 564.9 KiB x 1.9993 + WRITE_SIZE 68 145.9 KiB,
 # scale factors from a 64 MiB copy; profiles/gdn_decode_wide_kernel_B64.md).  Reported as `roofline.traffic` for that batch only.
-DECODE_TRAFFIC_B64 = int((34563.5 * 1.9993 + 68142.9) * 1024)
+DECODE_TRAFFIC_B64 = int((34564.9 * 1.9993 + 68145.9) * 1024)
 DECODE_TRAFFIC_SOURCE = ("profiles/gdn_decode_wide_kernel_B64.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gdn_decode_wide_kernel<4> at "
                          "B=64 (a recorded measurement of that kernel, not of this run)")
 # same for the three kernels of the T = 2048 prefill (profiles/gdn_prefill_T2048.md)
-PREFILL_TRAFFIC_T2048 = int(((16710.2 + 13618.8 + 23732.0) * 1.9993 + 37172 + 25600 + 8192) * 1024)
+PREFILL_TRAFFIC_T2048 = int(((16691.8 + 13314.7 + 23734.0) * 1.9993 + 37172.2 + 25600 + 8192) * 1024)
 PREFILL_TRAFFIC_SOURCE = ("profiles/gdn_prefill_T2048.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gdn_phase_a_kernel, gdn_chain_kernel and "
                           "gdn_output_kernel at T=2048 (a recorded measurement of those kernels, not of this run)")
 
