@@ -105,7 +105,8 @@ def attn_layer_b(qkv, q_norm, k_norm, Kp, Vp, slots, pos, M=1, eps=1e-6, split=N
     projections: q / k RMSNorm and rotary embedding, attn_b, and o * sigmoid(gate), in two launches per pass of four tokens
     (attention.qkv_prep + attn_b + attention.out_gate are four), with the same bits.  qkv [B*M,5120] bf16 = [(q_h | gate_h) x 8 |
     k x 2 | v x 2]; q_norm, k_norm [256] bf16; pools, slots, pos, M as for attn_b (the new K / V rows are appended in place).
-    Returns [B*M,2048] bf16."""
+    Returns [B*M,2048] bf16.  The first call on a device (and the first one with a longer pool) builds the rotary table: make
+    it outside HIP graph capture."""
     qkv = L.dev(qkv, BF16, "qkv", (None, 5120))
     R = qkv.shape[0]
     if M < 1 or M > 16 or R % M:
