@@ -35,6 +35,7 @@ constexpr float SCALE_LOG2E = 0.0625f * 1.4426950408889634f;   // 256^-0.5 log2 
 constexpr float NEG = -3.0e38f;
 constexpr float LAZY = 8.0f;            // log2 of the growth of a row maximum that is tolerated before the row is rescaled
 constexpr int KT = 64;                 // keys per tile
+constexpr int FRAG_AHEAD = 5;          // steps between the LDS read of a K fragment and its MFMAs in the tile loop
 constexpr int TILE = KT * AD;          // elements of one K or V tile in LDS (32 KiB), rows unpadded, chunks swizzled
 
 // PHASE_FENCE(): the phases of a tile are scheduled separately
@@ -44,6 +45,33 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// One direct-to-LDS load of 16 bytes per lane (global_load_lds_dwordx4): lane l fetches base + voff + IMM and the 64 pieces land
+// at lds + IMM + 16 l.  Issued as inline assembly, not through the builtin: while a direct-to-LDS load that the compiler knows
+// of is outstanding, it closes every wait for an LDS read with lgkmcnt(0) (the load counts as an access of both memories), and
+// the tile loop below always has such loads in flight, so each of its fragment reads would be waited for in full.  These loads
+// are waited for by hand (vmcnt(0) before the workgroup barrier of a tile).  base and lds are wavefront-uniform.
+template <int IMM>
+__device__ __forceinline__ void lds_dma16(const char* base, unsigned voff, const bf16_t* lds) {
+    const unsigned la = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds);
+    unsigned keep;                                                // M0 belongs to the compiler: put back what it held
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%4\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(voff), "s"(base), "s"(la), "n"(IMM)
+                 : "memory");
+}
+// four such loads, KiB 0 .. 3 behind lds, under one setting of M0 (a wavefront issues one instruction every four clocks, and
+// the tile loop is bound by exactly that, so the five scalar instructions around a single load count)
+__device__ __forceinline__ void lds_dma16x4(const char* base, unsigned v0, unsigned v1, unsigned v2, unsigned v3, const bf16_t* lds) {
+    const unsigned la = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds);
+    unsigned keep;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %6\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(v0), "v"(v1), "v"(v2), "v"(v3), "s"(base), "s"(la)
+                 : "memory");
 }
 
 // max over the four lanes n, n + 16, n + 32, n + 48 with the VALU lane swaps of gfx950 (v_permlane32_swap exchanges the upper half
@@ -155,30 +183,25 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         asm volatile("" : "+v"(off0));
         return off0;
     };
-    auto load_one = [&](const char* src, bf16_t* dst, int t, int i, unsigned off0) {   // load i of tile t (L >= KT)
-        // the row part of load i (2 i rows = 1024 i bytes) goes into the instruction's immediate offset, which moves the global
-        // address and the LDS destination alike (at most 4095: the upper four loads start 4 KiB further in both)
-        const auto gp = (const __attribute__((address_space(1))) void*)(src + (size_t)tile_row0(t) * (AD * 2) + 4096 * (i >> 2) +
-                                                                        (off0 ^ (32u * i)));
-        const auto lp = (__attribute__((address_space(3))) void*)(dst + (8 * w + 4 * (i >> 2)) * 512);
-        switch (i & 3) {                                         // the immediate has to be a literal
-            case 0: __builtin_amdgcn_global_load_lds(gp, lp, 16, 0, 0); break;
-            case 1: __builtin_amdgcn_global_load_lds(gp, lp, 16, 1024, 0); break;
-            case 2: __builtin_amdgcn_global_load_lds(gp, lp, 16, 2048, 0); break;
-            default: __builtin_amdgcn_global_load_lds(gp, lp, 16, 3072, 0);
-        }
+    // the row part of a load (2 i rows = 1024 i bytes) goes into the instruction's immediate offset, which moves the global
+    // address and the LDS destination alike (at most 4095: the upper four loads start 4 KiB further in both)
+    auto load_four = [&](const char* src, bf16_t* dst, int t, int half, unsigned off0) {   // loads 4 half .. 4 half + 3 of tile t
+        const char* base = src + (size_t)tile_row0(t) * (AD * 2) + 4096 * half;
+        const unsigned i0 = 4u * half;
+        lds_dma16x4(base, off0 ^ (32u * i0), off0 ^ (32u * (i0 + 1)), off0 ^ (32u * (i0 + 2)), off0 ^ (32u * (i0 + 3)),
+                    dst + (8 * w + 4 * half) * 512);
     };
     auto load_rows = [&](const char* src, bf16_t* dst, int t) {  // one K or V tile: this wavefront's eight direct loads
         if (L >= KT) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) load_one(src, dst, t, i, ld_off0);
+            const unsigned off0 = opaque_off0();
+            load_four(src, dst, t, 0, off0);
+            load_four(src, dst, t, 1, off0);
         } else {                                                 // t = 0: rows past the end repeat the last key; they are masked
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 const unsigned o = ld_off0 ^ (1056u * i);
                 const unsigned off = (unsigned)min((int)(o >> 9), L - 1) * (AD * 2) + (o & 511u);
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + off),
-                                                 (__attribute__((address_space(3))) void*)(dst + (8 * w + i) * 512), 16, 0, 0);
+                lds_dma16<0>(src, off, dst + (8 * w + i) * 512);
             }
         }
     };
@@ -282,32 +305,20 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         };
         s16x8 P[NH][2];
         s16x4 Bf[3][4];
-        bool rescale = false;
+        float mx[NH];
         auto body = [&](auto with_scores) {
             constexpr bool SC = decltype(with_scores)::value;
-            bf16x8 Af[2][8];
+            // K fragments: a ring, each read FRAG_AHEAD steps before the MFMAs that consume it (fragment f = 8 kt + kb)
+            bf16x8 Af[FRAG_AHEAD + 1];
             if (SC) {
 #pragma unroll
-                for (int kb = 0; kb < 8; kb++) Af[0][kb] = k_frag(ka, 0, kb);
+                for (int f = 0; f < FRAG_AHEAD; f++) Af[f] = k_frag(ka, f >> 3, f & 7);
             }
-            float m_new[NH];
+            // The exponentials are taken against the running reference point of each row at once, on the bet that no row's
+            // maximum grows by more than 2^LAZY in this tile (true for all but the first few tiles of a row block); the
+            // maxima are folded in beside them and the bet is checked after the steps (`grow` below).
 #pragma unroll
-            for (int hh = 0; hh < NH; hh++) {
-                float mx = NEG;
-#pragma unroll
-                for (int kt = 0; kt < 4; kt++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) mx = fmaxf(mx, acc[hh][kt][i]);
-                mx = max_over_groups(mx);
-                // the reference point of a row only moves when its maximum has grown by more than 2^LAZY: until then p stays
-                // below 2^LAZY, which bf16 and the f32 sums hold as well as values below 1, and the accumulators are left alone
-                mx *= SCALE_LOG2E;
-                m_new[hh] = mx > m_run[hh] + LAZY ? mx : m_run[hh];
-                const float corr = __builtin_amdgcn_exp2f(m_run[hh] - m_new[hh]);   // m_run = NEG initially: 2^-huge = 0
-                m_run[hh] = m_new[hh];
-                c_s[w][hh][n] = corr;                            // all four groups store the same value: no divergent branch
-                rescale |= corr != 1.0f;
-            }
+            for (int hh = 0; hh < NH; hh++) mx[hh] = NEG;
             PHASE_FENCE();
             const unsigned step_off0 = SC ? opaque_off0() : 0u;
             // 32 steps: two score MFMAs of tile t + 1 (one K fragment x both heads) and one softmax element of tile t
@@ -316,14 +327,15 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             for (int st = 0; st < 32; st++) {
                 const int kt = st >> 3, kb = st & 7;
                 __builtin_amdgcn_sched_barrier(0);
-                if (SC && (st & 1) == 0) {
+                if (SC && (st & 7) == 0) {
                     if (st < 16)
-                        load_one(kg, k_cur, tk, st >> 1, step_off0);
+                        load_four(kg, k_cur, tk, st >> 3, step_off0);
                     else
-                        load_one(vg, v_nxt, tv, (st >> 1) - 8, step_off0);
+                        load_four(vg, v_nxt, tv, (st >> 3) - 2, step_off0);
                 }
                 if (SC) {
-                    if (kt < 3) Af[(kt + 1) & 1][kb] = k_frag(ka, kt + 1, kb);
+                    if (st + FRAG_AHEAD < 32)
+                        Af[(st + FRAG_AHEAD) % (FRAG_AHEAD + 1)] = k_frag(ka, (st + FRAG_AHEAD) >> 3, (st + FRAG_AHEAD) & 7);
                     if (st >= 30) {                              // the first V fragments of P.V ride along with the last steps
 #pragma unroll
                         for (int q4 = 0; q4 < 4; q4++) Bf[st - 30][q4] = v_frag(st - 30, q4);
@@ -331,13 +343,14 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
 #pragma unroll
                     for (int hh = 0; hh < NH; hh++)
                         acc_next[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            Af[kt & 1][kb], bq[hh][kb], kb == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc_next[hh][kt], 0, 0, 0);
+                            Af[st % (FRAG_AHEAD + 1)], bq[hh][kb], kb == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc_next[hh][kt], 0, 0, 0);
                 }
                 // softmax elements: NH * 16 of them over the 32 steps
 #pragma unroll
                 for (int e = (NH * 16 * st) / 32; e < (NH * 16 * (st + 1)) / 32; e++) {
                     const int hh = e >> 4, kt2 = (e >> 2) & 3, i = e & 3;
-                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_new[hh]));
+                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_run[hh]));
+                    mx[hh] = fmaxf(mx[hh], acc[hh][kt2][i]);
                     if (i & 1) {
                         const uint32_t pk = pack_bf(pv_prev, pv);
                         P[hh][kt2 >> 1][(kt2 & 1) * 4 + i - 1] = (short)(pk & 0xffff);
@@ -359,9 +372,36 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             body(std::true_type{});
         else
             body(std::false_type{});
-        wave_lds_sync();
         PHASE_FENCE();
-        if (__any(rescale)) {                                    // wavefront-uniform: most tiles leave every row's max alone
+        // the reference point of a row only moves when its maximum has grown by more than 2^LAZY: until then p stays below
+        // 2^LAZY, which bf16 and the f32 sums hold as well as values below 1, and the accumulators are left alone
+        bool grow = false;
+#pragma unroll
+        for (int hh = 0; hh < NH; hh++) {
+            mx[hh] = max_over_groups(mx[hh]) * SCALE_LOG2E;
+            grow |= mx[hh] > m_run[hh] + LAZY;
+        }
+        if (__any(grow)) {                                       // wavefront-uniform and rare: the bet was lost for some row
+#pragma unroll
+            for (int hh = 0; hh < NH; hh++) {
+                const float m_new = mx[hh] > m_run[hh] + LAZY ? mx[hh] : m_run[hh];
+                const float corr = __builtin_amdgcn_exp2f(m_run[hh] - m_new);   // m_run = NEG initially: 2^-huge = 0
+                m_run[hh] = m_new;
+                c_s[w][hh][n] = corr;                            // all four groups store the same value: no divergent branch
+                // this tile's p again, against the new reference points (rows that did not move get the same bits)
+#pragma unroll
+                for (int kt2 = 0; kt2 < 4; kt2++)
+#pragma unroll
+                    for (int i = 0; i < 4; i += 2) {
+                        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_new));
+                        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i + 1], SCALE_LOG2E, -m_new));
+                        const uint32_t pk = pack_bf(p0, p1);
+                        P[hh][kt2 >> 1][(kt2 & 1) * 4 + i] = (short)(pk & 0xffff);
+                        P[hh][kt2 >> 1][(kt2 & 1) * 4 + i + 1] = (short)(pk >> 16);
+                        __builtin_amdgcn_sched_barrier(0);       // pair by pair: scheduled freely, the 32 values take registers
+                    }
+            }
+            wave_lds_sync();
 #pragma unroll
             for (int hh = 0; hh < NH; hh++) {
                 const f32x4 c4 = *reinterpret_cast<const f32x4*>(&c_s[w][hh][4 * g]);
@@ -369,10 +409,13 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                 for (int j = 0; j < 16; j++) {
                     PIN_ACC(O[hh][j]);
                     O[hh][j] *= c4;
+                    PIN_ACC(O[hh][j]);                           // and back at once: 128 products would not fit beside the rest
                 }
                 PIN_ACC(Lsum[hh]);
                 Lsum[hh] *= c4;
+                PIN_ACC(Lsum[hh]);
             }
+            wave_lds_sync();                                     // c_s is rewritten by the next tile that moves a reference
         }
         PHASE_FENCE();
         // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs and serve
@@ -407,7 +450,6 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         }
         __builtin_amdgcn_sched_barrier(0);
         PHASE_FENCE();
-        wave_lds_sync();                                         // c_s is rewritten by the next tile
     };
 
     if (ta < tb) {                                               // (a part past the block's last tile is empty)
