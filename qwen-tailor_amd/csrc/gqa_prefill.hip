@@ -52,9 +52,14 @@ __device__ __forceinline__ void wave_lds_sync() {
 // of is outstanding, it closes every wait for an LDS read with lgkmcnt(0) (the load counts as an access of both memories), and
 // the tile loop below always has such loads in flight, so each of its fragment reads would be waited for in full.  These loads
 // are waited for by hand (vmcnt(0) before the workgroup barrier of a tile).  base and lds are wavefront-uniform.
+// LDS byte address of a __shared__ array, taken of the array itself: a constant.  (Taken of a pointer that has been moved, the
+// cast from a generic pointer costs a null test and two scalar registers per use.)
+__device__ __forceinline__ unsigned lds_address(const bf16_t* shared_array) {
+    return (unsigned)(size_t)(__attribute__((address_space(3))) const void*)shared_array;
+}
 template <int IMM>
-__device__ __forceinline__ void lds_dma16(const char* base, unsigned voff, const bf16_t* lds) {
-    const unsigned la = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds);
+__device__ __forceinline__ void lds_dma16(const char* base, unsigned voff, unsigned lds) {
+    const unsigned la = __builtin_amdgcn_readfirstlane(lds);
     unsigned keep;                                                // M0 belongs to the compiler: put back what it held
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%4\n\ts_mov_b32 m0, %0"
                  : "=&s"(keep)
@@ -63,8 +68,8 @@ __device__ __forceinline__ void lds_dma16(const char* base, unsigned voff, const
 }
 // four such loads, KiB 0 .. 3 behind lds, under one setting of M0 (a wavefront issues one instruction every four clocks, and
 // the tile loop is bound by exactly that, so the five scalar instructions around a single load count)
-__device__ __forceinline__ void lds_dma16x4(const char* base, unsigned v0, unsigned v1, unsigned v2, unsigned v3, const bf16_t* lds) {
-    const unsigned la = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds);
+__device__ __forceinline__ void lds_dma16x4(const char* base, unsigned v0, unsigned v1, unsigned v2, unsigned v3, unsigned lds) {
+    const unsigned la = __builtin_amdgcn_readfirstlane(lds);
     unsigned keep;
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %6\n\ts_nop 0\n\t"
                  "global_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
@@ -185,13 +190,15 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     };
     // the row part of a load (2 i rows = 1024 i bytes) goes into the instruction's immediate offset, which moves the global
     // address and the LDS destination alike (at most 4095: the upper four loads start 4 KiB further in both)
-    auto load_four = [&](const char* src, bf16_t* dst, int t, int half, unsigned off0) {   // loads 4 half .. 4 half + 3 of tile t
+    // (dst: LDS byte address of the tile buffer)
+    const unsigned w_lds = 8192u * w;                            // this wavefront's 8 KiB of a tile buffer
+    auto load_four = [&](const char* src, unsigned dst, int t, int half, unsigned off0) {   // loads 4 half .. 4 half + 3 of tile t
         const char* base = src + (size_t)tile_row0(t) * (AD * 2) + 4096 * half;
         const unsigned i0 = 4u * half;
         lds_dma16x4(base, off0 ^ (32u * i0), off0 ^ (32u * (i0 + 1)), off0 ^ (32u * (i0 + 2)), off0 ^ (32u * (i0 + 3)),
-                    dst + (8 * w + 4 * half) * 512);
+                    dst + w_lds + 4096u * half);
     };
-    auto load_rows = [&](const char* src, bf16_t* dst, int t) {  // one K or V tile: this wavefront's eight direct loads
+    auto load_rows = [&](const char* src, unsigned dst, int t) {  // one K or V tile: this wavefront's eight direct loads
         if (L >= KT) {
             const unsigned off0 = opaque_off0();
             load_four(src, dst, t, 0, off0);
@@ -201,7 +208,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             for (int i = 0; i < 8; i++) {
                 const unsigned o = ld_off0 ^ (1056u * i);
                 const unsigned off = (unsigned)min((int)(o >> 9), L - 1) * (AD * 2) + (o & 511u);
-                lds_dma16<0>(src, off, dst + (8 * w + i) * 512);
+                lds_dma16<0>(src, off, dst + w_lds + 1024u * i);
             }
         }
     };
@@ -265,10 +272,10 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         constexpr int PAR = decltype(par)::value;
         f32x4 (&acc)[NH][4] = accs[PAR];
         f32x4 (&acc_next)[NH][4] = accs[PAR ^ 1];
-        bf16_t* const k_cur = PAR ? k_s1 : k_s0;                 // K(t): consumed already, refilled with K(t + 2)
+        const unsigned k_cur = lds_address(PAR ? k_s1 : k_s0);   // K(t): consumed already, refilled with K(t + 2)
         const bf16_t* const k_nxt = PAR ? k_s0 : k_s1;           // K(t + 1)
         const bf16_t* const v_cur = PAR ? v_s1 : v_s0;           // V(t)
-        bf16_t* const v_nxt = PAR ? v_s0 : v_s1;                 // V(t - 1): consumed, refilled with V(t + 1)
+        const unsigned v_nxt = lds_address(PAR ? v_s0 : v_s1);   // V(t - 1): consumed, refilled with V(t + 1)
         PHASE_FENCE();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wavefront's loads of K(t + 1), V(t) have landed in LDS
         PHASE_FENCE();
@@ -453,11 +460,11 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     };
 
     if (ta < tb) {                                               // (a part past the block's last tile is empty)
-        load_rows(kg, k_s0, ta);
-        load_rows(vg, v_s0, ta);
+        load_rows(kg, lds_address(k_s0), ta);
+        load_rows(vg, lds_address(v_s0), ta);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tb - ta > 1) load_rows(kg, k_s1, ta + 1);
+        if (tb - ta > 1) load_rows(kg, lds_address(k_s1), ta + 1);
         if (tw > ta) scores_first(k_s0 + ka_row, accs[0]);
         for (int t = ta; t < tb; t += 2) {
             tile(t, std::integral_constant<int, 0>{});
