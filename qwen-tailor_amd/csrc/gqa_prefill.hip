@@ -15,7 +15,8 @@
 // registers in between) into double-buffered tiles.  The LDS rows are unpadded (a direct load cannot pad); instead the
 // 16-byte chunks of row r are stored XOR-swizzled by r & 15 (the loading lane picks the matching global chunk), which keeps
 // the fragment reads of 16 rows on distinct banks.  The tile loop is software-pipelined around one workgroup barrier per tile:
-// the score MFMAs of tile t + 1 are interleaved step by step with the softmax of tile t (see `tile` below).
+// the score MFMAs of tile t + 1 are interleaved step by step with the exponentials of tile t, which are taken against the
+// running reference points before the tile's row maxima are known and checked afterwards (see `tile` below).
 #include "qt_common.h"
 
 #include <algorithm>
@@ -121,8 +122,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
                                                            const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
                                                            int q_pos0, long q_head_stride, long kv_head_stride, int tmax,
                                                            _Float16* __restrict__ part_o, float* __restrict__ part_ml) {
-    // four separate arrays, not [2][TILE]: the compiler tracks outstanding direct-to-LDS loads per LDS variable, so a read of
-    // one buffer does not wait for the loads in flight to the others
+    // four separate arrays: the loaders take each buffer's LDS address as a constant (lds_address)
     __shared__ __align__(1024) bf16_t k_s0[TILE];
     __shared__ __align__(1024) bf16_t k_s1[TILE];
     __shared__ __align__(1024) bf16_t v_s0[TILE];
