@@ -290,6 +290,23 @@ inline int pick_rs(int nseq, int rows_split) {
     return 1;
 }
 
+// The decode step's shape: whole heads per workgroup (1, 2 or 4) while B x 16 heads give every CU a workgroup (measured, us at
+// 1 / 2 / 4 heads: B = 16 6.7 / 7.7 / 11.4, 24 11.9 / 9.8 / 12.1, 32 12.4 / 12.3 / 13.5, 48 19.2 / 21.2 / 18.5, 64 25.6 / 24.8 /
+// 23.7), below that a head split over 2, 4 or 8 workgroups (B = 8: 5.5 us at 2 or 4 parts, B = 4: 4.5 us at 4).
+// Beyond one round of four-head workgroups (B > 64) small workgroups balance the rounds better: half a head each (B = 96
+// 38.1 against 39.5 us, B = 128 50.7 against 52.1), a whole head where the fused norm needs one.
+inline int decode_heads_per_wg(int B) {
+    const long heads = (long)B * HV, cus = cu_count();
+    return heads > 4 * cus ? 1 : heads > 2 * cus ? 4 : heads > cus ? 2 : 1;
+}
+inline int decode_rs(int B) {                                    // 16-row groups per workgroup when a head is split
+    const long heads = (long)B * HV, cus = cu_count();
+    if (heads > 4 * cus) return 4;
+    int rs = 8;
+    while (rs > 1 && heads * (8 / rs) * 2 <= cus) rs >>= 1;
+    return rs;
+}
+
 }  // namespace
 
 #define QT_DISPATCH_RS(rs, KERNEL, nseq, stream, ...)                                                  \
@@ -310,8 +327,9 @@ int qt_gdn_decode_step(const void* proj, void* conv_pool, const void* conv_w, co
     if (B == 0) return QT_OK;
     if (!aligned16(ssm_pool) || (reinterpret_cast<uintptr_t>(conv_w) & 7u)) return QT_ERR_ALIGN;
     // Many rows: 2 or 4 whole heads of a row per workgroup (128 / 256 KiB of contiguous state per workgroup); measured at
-    // B = 64: 23.3 us against 26.0 us with one head per workgroup.  Few rows: split heads so the chip still fills.
-    const int hpw = rows_per_wg == 512 ? 4 : rows_per_wg == 256 ? 2 : rows_per_wg != 0 ? 1 : B >= 64 ? 4 : B >= 32 ? 2 : 1;
+    // B = 64: 23.3 us against 26.0 us with one head per workgroup.  Few rows: split heads so the chip still fills.  The shape
+    // that wins at every batch size measured (4 .. 64 rows) is the largest one that still gives every CU a workgroup.
+    const int hpw = rows_per_wg == 512 ? 4 : rows_per_wg == 256 ? 2 : rows_per_wg != 0 ? 1 : decode_heads_per_wg(B);
     if (hpw == 4) {
         hipLaunchKernelGGL(gdn_decode_wide_kernel<4>, dim3(B * (HV / 4)), dim3(1024), 0, stream, (const bf16_t*)proj,
                            (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log, dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
@@ -319,7 +337,7 @@ int qt_gdn_decode_step(const void* proj, void* conv_pool, const void* conv_w, co
         hipLaunchKernelGGL(gdn_decode_wide_kernel<2>, dim3(B * (HV / 2)), dim3(512), 0, stream, (const bf16_t*)proj,
                            (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log, dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
     } else {
-        const int rs = pick_rs(B, rows_per_wg);
+        const int rs = rows_per_wg ? pick_rs(B, rows_per_wg) : decode_rs(B);
         QT_DISPATCH_RS(rs, gdn_decode_kernel, B, stream, (const bf16_t*)proj, (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log,
                        dt_bias, ssm_pool, slots, pos, (bf16_t*)y, n_slots);
     }
@@ -339,8 +357,9 @@ int qt_gdn_decode_step_gnorm(const void* proj, void* conv_pool, const void* conv
 #define QT_GNORM_LAUNCH(HPW_)                                                                                                  \
     hipLaunchKernelGGL((gdn_decode_wide_kernel<HPW_, true>), dim3(B * (HV / HPW_)), dim3(256 * HPW_), 0, stream, (const bf16_t*)proj, \
                        (bf16_t*)conv_pool, (const bf16_t*)conv_w, A_log, dt_bias, ssm_pool, slots, pos, (bf16_t*)out, n_slots, gw, eps)
-    if (B >= 64) QT_GNORM_LAUNCH(4);
-    else if (B >= 32) QT_GNORM_LAUNCH(2);
+    const int hpw = decode_heads_per_wg(B);
+    if (hpw == 4) QT_GNORM_LAUNCH(4);
+    else if (hpw == 2) QT_GNORM_LAUNCH(2);
     else QT_GNORM_LAUNCH(1);
     QT_CHECK_LAUNCH();
     return QT_OK;
