@@ -277,9 +277,9 @@ def test_deltanet_b_layout_of_reference_test(qt, dev):
         check_tensors_equal(f'ssm pool rows_per_wg={rows}', ssm2, ssm_pool)
 
 
-@pytest.mark.parametrize("B", [1, 16, 64])
+@pytest.mark.parametrize("B", [1, 16, 24, 48, 64, 96])              # (every default workgroup shape: split head, 1, 2, 4 heads, half heads)
 def test_deltanet_b_config1_steps(qt, dev, B):
-    """benchmark config 1 (B in {1,16,64}): consecutive steps with advancing positions; state ~ N(0,0.02).  The C oracle steps
+    """benchmark config 1 (B = 1, 16, 64, and sizes between and beyond that take the other default shapes): consecutive steps with advancing positions; state ~ N(0,0.02).  The C oracle steps
     alongside from its own state (free running) and must stay within 1e-4 relative at every step."""
     gen = torch.Generator().manual_seed(1001)
     cw, A_log, dtb, gw = layer_params(9)
@@ -421,7 +421,7 @@ def test_deltanet_bm_config4_size(qt, dev):
     check_equal("trash entry", got[NS], sp[NS])
 
 
-@pytest.mark.parametrize("B", [1, 5, 32, 64])
+@pytest.mark.parametrize("B", [1, 5, 24, 32, 48, 64, 80])
 def test_deltanet_b_gnorm_equals_two_launches(qt, dev, B):
     """the decode step with the gated RMSNorm fused in == deltanet_b followed by gnorm_rows (batch.py:497-499), bit for bit,
     for each workgroup shape the batch size selects (1, 2 or 4 heads per workgroup)"""
