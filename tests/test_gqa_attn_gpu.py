@@ -238,6 +238,35 @@ def test_prefill_causal_8192_two_heads_per_wavefront(qt, dev):
     check_equal("row 0 == v[0]", o[:, 0], np.repeat(Vn[:, 0], 4, axis=0))
 
 
+@pytest.mark.parametrize("S", [2048, 4800])
+def test_prefill_causal_reference_points_that_move_late(qt, dev, S):
+    """Two heads per wavefront, split along the keys (S = 2048) and unsplit (S = 4800).  The kernel exponentiates a tile against the
+    running reference points before it knows the tile's maxima and takes the tile again when a row's maximum grew by more
+    than 2^8: here a handful of keys deep inside the sequence are aligned with a block of query rows and scaled up, so that rows
+    which have settled long ago jump by 2^10 .. 2^60 in one tile, some rows of a wavefront and not others, more than once."""
+    g = torch.Generator().manual_seed(S)
+    q = torch.randn((8, S, 256), generator=g)
+    K = torch.randn((2, S, 256), generator=g)
+    V = torch.randn((2, S, 256), generator=g).bfloat16()
+    rng = np.random.default_rng(S)
+    special = sorted(int(k) for k in rng.choice(np.arange(300, S - 200), 6, replace=False))
+    for j, k in enumerate(special):
+        h = int(rng.integers(0, 8))
+        r0 = k + int(rng.integers(1, 150))                       # rows that see the key: a ragged set across wavefront borders
+        rows = slice(r0, min(S, r0 + int(rng.integers(3, 40))))
+        K[h // 4, k] = q[h, r0] * (0.6 + 0.5 * j)                # score ~ |q|^2 (0.6 ..) / 16 = 10 .. 50 (base e) above the rest
+        q[h, rows] = q[h, r0] + 0.05 * torch.randn((rows.stop - rows.start, 256), generator=g)
+    q, K = q.bfloat16(), K.bfloat16()
+    o = to_np(qt.attention.scaled_dot_product_attention(q.to(dev)[None], K.to(dev)[None], V.to(dev)[None], scale=256 ** -0.5,
+                                                        mask="causal"))[0]
+    qn, Kn, Vn = q.float().numpy(), K.float().numpy(), V.float().numpy()
+    rows = set(int(r) for r in rng.integers(0, S, 24))
+    for k in special:
+        rows.update(range(k - 2, min(S, k + 190), 7))
+    for r in sorted(rows):
+        check_attn(f"S={S} row {r}", o[:, r:r + 1], O.sdpa_causal(qn[:, r:r + 1], Kn[:, :r + 1], Vn[:, :r + 1]))
+
+
 def test_prefill_causal_long_ragged_continuation(qt, dev):
     """two heads per wavefront with nothing aligned: S = 8170 query rows continue a prefix of 37 keys (L = 8207: the last tile is
     shifted back, the last row blocks are partial, some wavefronts have one tile less than their workgroup)"""
