@@ -243,7 +243,8 @@ def test_prefill_causal_reference_points_that_move_late(qt, dev, S):
     """Two heads per wavefront, split along the keys (S = 2048) and unsplit (S = 4800).  The kernel exponentiates a tile against the
     running reference points before it knows the tile's maxima and takes the tile again when a row's maximum grew by more
     than 2^8: here a handful of keys deep inside the sequence are aligned with a block of query rows and scaled up, so that rows
-    which have settled long ago jump by 2^10 .. 2^60 in one tile, some rows of a wavefront and not others, more than once."""
+    which have settled long ago jump by 2^14 .. 2^187 in one tile (the last ones overflow the exponential taken on the bet), some
+    rows of a wavefront and not others, more than once."""
     g = torch.Generator().manual_seed(S)
     q = torch.randn((8, S, 256), generator=g)
     K = torch.randn((2, S, 256), generator=g)
@@ -254,7 +255,7 @@ def test_prefill_causal_reference_points_that_move_late(qt, dev, S):
         h = int(rng.integers(0, 8))
         r0 = k + int(rng.integers(1, 150))                       # rows that see the key: a ragged set across wavefront borders
         rows = slice(r0, min(S, r0 + int(rng.integers(3, 40))))
-        K[h // 4, k] = q[h, r0] * (0.6 + 0.5 * j)                # score ~ |q|^2 (0.6 ..) / 16 = 10 .. 50 (base e) above the rest
+        K[h // 4, k] = q[h, r0] * (0.6 + 1.5 * j)                # score ~ |q|^2 (0.6 .. 8.1) / 16 = 10 .. 130 (base e) above the rest
         q[h, rows] = q[h, r0] + 0.05 * torch.randn((rows.stop - rows.start, 256), generator=g)
     q, K = q.bfloat16(), K.bfloat16()
     o = to_np(qt.attention.scaled_dot_product_attention(q.to(dev)[None], K.to(dev)[None], V.to(dev)[None], scale=256 ** -0.5,
