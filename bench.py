@@ -562,7 +562,7 @@ def main():
     st = build_decode_state(torch, dev, B, N_LAYERS)
     wall, dev_s, n_regions = time_decode(torch, qt, st, B, N_LAYERS, args.steps, args.warmup, use_graph=not args.no_graph)
     # Two clocks around the same regions.  `value` and `ms_per_step` are on the host's wall clock (device synchronisation on both
-    # sides of exactly `steps` launches: what a caller waits for, and the clock of the first round's record); the roofline is on
+    # sides of exactly `steps` launches: what a caller waits for); the roofline is on
     # the device clock (HIP events on the launching stream), which leaves out the bracket's own cost.
     launch_s = dev_s / args.steps
     wall_step_s = wall / args.steps
