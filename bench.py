@@ -105,21 +105,29 @@ def time_decode(torch, qt, st, B, n_layers, steps, warmup, use_graph=True, min_t
         return ((i + n_layers - 1) // n_layers) * n_layers if graphs is not None else i
 
     i = align(run(warmup))
-    regions, total = [], 0.0
-    while len(regions) < 3 or (total < min_total_s and len(regions) < max_regions):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    walls, devs, total = [], [], 0.0
+    # regions alternate between the two clocks: an event record is a packet of its own on the stream, and inside a wall-clock
+    # region of a few launches the two of them would be timed as if they were part of the work
+    while min(len(walls), len(devs)) < 3 or (total < min_total_s and len(walls) + len(devs) < max_regions):
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record()
-        i = align(run(steps, i))
-        e1.record()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        regions.append((e0.elapsed_time(e1) * 1e-3, wall))
-        total += wall
-    dev_s = sorted(r[0] for r in regions)[len(regions) // 2]
-    wall = sorted(r[1] for r in regions)[len(regions) // 2]
-    return wall, dev_s, len(regions)
+        if len(walls) <= len(devs):
+            t0 = time.perf_counter()
+            i = run(steps, i)
+            torch.cuda.synchronize()
+            walls.append(time.perf_counter() - t0)
+            total += walls[-1]
+        else:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            i = run(steps, i)
+            e1.record()
+            torch.cuda.synchronize()
+            devs.append(e0.elapsed_time(e1) * 1e-3)
+            total += devs[-1]
+        i = align(i)
+    dev_s = sorted(devs)[len(devs) // 2]
+    wall = sorted(walls)[len(walls) // 2]
+    return wall, dev_s, len(walls) + len(devs)
 
 
 def time_graph(torch, fn, reps=200, inner=10):
