@@ -35,24 +35,57 @@ struct BlitJob {
     long nvec, ny, dstride, sstride;
 };
 constexpr int MAX_JOBS = 64;           // 64 x 48 bytes of kernel arguments
+constexpr int BLIT_WGS_PER_CU = 8;
 struct BlitJobs {
     BlitJob job[MAX_JOBS];
+    int first_block[MAX_JOBS + 1];     // exclusive prefix of the jobs' (row, 1024-vector block) counts
 };
-// grid = (x, number of jobs): the x workgroups of a job walk its (row, 1024-vector block) pairs with a grid stride
-__global__ __launch_bounds__(256) void blit_batch_kernel(const BlitJobs jobs) {
-    const BlitJob& j = jobs.job[blockIdx.y];
-    const long blocks_per_row = (j.nvec + 1023) / 1024, nblocks = blocks_per_row * j.ny;
-    for (long b = blockIdx.x; b < nblocks; b += gridDim.x) {
-        const long y = b / blocks_per_row, i0 = (b % blocks_per_row) * 1024 + threadIdx.x;
-        u32x4* d = j.dst + y * j.dstride;
-        const u32x4* s = j.src + y * j.sstride;
-        u32x4 v[4];
+// One flat space of (job, row, 1024-vector block) units of 16 KiB, walked with a grid stride: every workgroup moves the same
+// number of units whatever the mix of job sizes, and asks for its next unit's vectors before it stores the current one's.
+__global__ __launch_bounds__(256) void blit_batch_kernel(const BlitJobs jobs, int njobs) {
+    const int total = jobs.first_block[njobs];
+    auto locate = [&](int b, const u32x4*& s, u32x4*& d, long& left) {
+        int lo = 0, hi = njobs - 1;                                  // the job that holds unit b (uniform binary search)
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (jobs.first_block[mid] <= b) lo = mid; else hi = mid - 1;
+        }
+        const BlitJob& j = jobs.job[lo];
+        const long r = b - jobs.first_block[lo], blocks_per_row = (j.nvec + 1023) / 1024;
+        const long y = r / blocks_per_row, i0 = (r % blocks_per_row) * 1024 + threadIdx.x;
+        s = j.src + y * j.sstride + i0;
+        d = j.dst + y * j.dstride + i0;
+        left = j.nvec - i0;                                          // vectors of the row from this lane's first one on
+    };
+    int b = blockIdx.x;
+    if (b >= total) return;
+    const u32x4* s;
+    u32x4* d;
+    long left;
+    locate(b, s, d, left);
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (k * 256 < left) v[k] = __builtin_nontemporal_load(s + k * 256);
+    while (true) {
+        const int nb = b + gridDim.x;
+        const u32x4* s2 = nullptr;
+        u32x4* d2 = nullptr;
+        long left2 = 0;
+        u32x4 v2[4];
+        if (nb < total) {
+            locate(nb, s2, d2, left2);
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                if (k * 256 < left2) v2[k] = __builtin_nontemporal_load(s2 + k * 256);
+        }
 #pragma unroll
         for (int k = 0; k < 4; k++)
-            if (i0 + k * 256 < j.nvec) v[k] = __builtin_nontemporal_load(s + i0 + k * 256);
+            if (k * 256 < left) __builtin_nontemporal_store(v[k], d + k * 256);
+        if (nb >= total) break;
+        b = nb, d = d2, left = left2;
 #pragma unroll
-        for (int k = 0; k < 4; k++)
-            if (i0 + k * 256 < j.nvec) __builtin_nontemporal_store(v[k], d + i0 + k * 256);
+        for (int k = 0; k < 4; k++) v[k] = v2[k];
     }
 }
 
@@ -112,7 +145,7 @@ int qt_blit_batch(void* const* dst, const void* const* src, const long* meta, in
     for (int k0 = 0; k0 < count; k0 += MAX_JOBS) {
         BlitJobs jobs;
         const int nj = count - k0 < MAX_JOBS ? count - k0 : MAX_JOBS;
-        long most = 1;
+        long total = 0;
         for (int k = 0; k < nj; k++) {
             const long* m = meta + 7 * (k0 + k);
             const long per = 16 / m[0];
@@ -123,11 +156,15 @@ int qt_blit_batch(void* const* dst, const void* const* src, const long* meta, in
             j.ny = m[4];
             j.dstride = m[5] / per;
             j.sstride = m[6] / per;
-            const long nb = (j.nvec + 1023) / 1024 * j.ny;
-            if (nb > most) most = nb;
+            jobs.first_block[k] = (int)total;
+            total += (j.nvec + 1023) / 1024 * j.ny;
+            if (total > 0x7fffffffL) return QT_ERR_DIM;                  // (32 TiB in one call)
         }
         for (int k = nj; k < MAX_JOBS; k++) jobs.job[k] = BlitJob{nullptr, nullptr, 0, 0, 0, 0};
-        hipLaunchKernelGGL(blit_batch_kernel, dim3((unsigned)(most < 256 ? most : 256), (unsigned)nj), dim3(256), 0, stream, jobs);
+        for (int k = nj; k <= MAX_JOBS; k++) jobs.first_block[k] = (int)total;
+        if (total == 0) continue;
+        const long wgs = (long)qt::cu_count() * BLIT_WGS_PER_CU;
+        hipLaunchKernelGGL(blit_batch_kernel, dim3((unsigned)(total < wgs ? total : wgs)), dim3(256), 0, stream, jobs, nj);
         QT_CHECK_LAUNCH();
     }
     return QT_OK;
