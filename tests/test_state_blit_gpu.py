@@ -128,3 +128,24 @@ def test_blit_batch_equals_single_blits(qt, dev):
         check_equal(f"job {k}", to_np(j[0]), w)
     with pytest.raises(ValueError):
         qt.batch.blit_batch([(jobs[0][0], jobs[0][1], 7, 0, 0, 1, 0, 0)])       # 28 bytes: not 16-byte granular
+
+
+def test_blit_batch_with_empty_jobs_and_more_units_than_workgroups(qt, dev):
+    """A launch is one flat space of 16 KiB units over all its copies.  Here: copies of no rows or no elements before, between and
+    behind the others (their unit ranges are empty), rows that end inside a unit, and one copy of 48 MiB, which gives every
+    workgroup several units with the next one requested before the current one is stored."""
+    rng = np.random.default_rng(4)
+    shapes = [(0, 0, 0, 3, 16, 16, BF16), (4096 + 8, 8, 0, 3, 8192, 4104, BF16), (128, 0, 0, 0, 0, 0, torch.float32),
+              (12 << 20, 4, 8, 1, 0, 0, torch.float32), (0, 0, 0, 1, 0, 0, BF16), (8, 8, 0, 7, 16, 8, BF16), (16, 0, 0, 0, 0, 0, BF16)]
+    jobs, want = [], []
+    for n, d0, s0, ny, ds, ss, dt in shapes:
+        nd, ns = d0 + max(ny - 1, 0) * ds + n + 16, s0 + max(ny - 1, 0) * ss + n + 8
+        dst0 = bf(rng.standard_normal(nd))
+        src = bf(rng.standard_normal(ns))
+        jobs.append((to_dev(dst0, dev, dt), to_dev(src, dev, dt), n, d0, s0, ny, ds, ss))
+        want.append(O.blit(dst0.copy(), src, n, d0, s0, ny, ds, ss) if n and ny else dst0)
+    qt.batch.blit_batch(jobs)
+    for k, (j, w) in enumerate(zip(jobs, want)):
+        check_equal(f"job {k}", to_np(j[0]), w)
+    qt.batch.blit_batch([jobs[0], jobs[2]])                                  # nothing to move at all
+    check_equal("empty launch", to_np(jobs[0][0]), want[0])
