@@ -84,8 +84,7 @@ __global__ __launch_bounds__(256) void blit_batch_kernel(const BlitJobs jobs, in
             if (k * 256 < left) __builtin_nontemporal_store(v[k], d + k * 256);
         if (nb >= total) break;
         b = nb, d = d2, left = left2;
-#pragma unroll
-        for (int k = 0; k < 4; k++) v[k] = v2[k];
+        v[0] = v2[0], v[1] = v2[1], v[2] = v2[2], v[3] = v2[3];
     }
 }
 
