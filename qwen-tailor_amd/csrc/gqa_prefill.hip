@@ -2,9 +2,13 @@
 // Replaces the call mx.fast.scaled_dot_product_attention(q, K[:, :, :kv_len], V[:, :, :kv_len], scale=256**-0.5,
 // mask="causal") of the reference's full-attention layers (qwen35/model.py:160-167, qwen35/prefill.py:468).
 //
-// One workgroup = 32 query rows x the 4 query heads that share a KV head: wavefront w owns the 16 rows of block w >> 1 for
-// the two heads 2 (w & 1), 2 (w & 1) + 1, so a K / V tile of 64 keys is fetched from HBM once and staged in LDS for all of
-// them, and every K or V fragment a wavefront reads from LDS feeds two MFMAs (one per head).  Per tile and wavefront:
+// Two kernels over one data path:
+//   attn_prefill_ws_kernel   32 query rows x the 4 query heads that share a KV head per workgroup, on eight wavefronts in two
+//                            roles (a "score" and an "output" wavefront per 16 rows x 2 heads): launches of about 1500 rows
+//                            and more.  Every K or V fragment read from LDS feeds two MFMAs (one per head).
+//   attn_prefill_kernel      16 query rows x the 4 heads, one head per wavefront, the whole tile loop on each: twice the
+//                            workgroups (and twice the LDS traffic per MFMA), for launches that would otherwise leave CUs idle.
+// The data path, per 64-key tile and 16 rows of a head:
 //     S^T[keys x rows] = K_tile . Q^T     A = K rows from LDS, B = Q^T resident in registers (16x16x32 bf16 MFMA)
 //     online softmax in the accumulator layout: lane (row n, group g) holds keys 4g..4g+3 of each 16-key sub-tile
 //     O[rows x 256]   += P . V            A = two exponentiated S^T accumulators packed to bf16 (they ARE the A operand
@@ -14,9 +18,9 @@
 // K / V tiles travel HBM -> LDS directly (global_load_lds_dwordx4: 64 lanes x 16 bytes land as one contiguous KiB, no
 // registers in between) into double-buffered tiles.  The LDS rows are unpadded (a direct load cannot pad); instead the
 // 16-byte chunks of row r are stored XOR-swizzled by r & 15 (the loading lane picks the matching global chunk), which keeps
-// the fragment reads of 16 rows on distinct banks.  The tile loop is software-pipelined around one workgroup barrier per tile:
-// the score MFMAs of tile t + 1 are interleaved step by step with the exponentials of tile t, which are taken against the
-// running reference points before the tile's row maxima are known and checked afterwards (see `tile` below).
+// the fragment reads of 16 rows on distinct banks.  The tile loops are software-pipelined around one workgroup barrier per
+// tile: the score MFMAs of tile t + 1 run while tile t is exponentiated, against the running reference points, before the
+// tile's row maxima are known; the bet is checked afterwards (see `tile` and `publish` below).
 #include "qt_common.h"
 
 #include <algorithm>
@@ -37,6 +41,7 @@ constexpr float NEG = -3.0e38f;
 constexpr float LAZY = 8.0f;            // log2 of the growth of a row maximum that is tolerated before the row is rescaled
 constexpr int KT = 64;                 // keys per tile
 constexpr int FRAG_AHEAD = 5;          // steps between the LDS read of a K fragment and its MFMAs in the tile loop
+constexpr int V_FRAG_AHEAD = 2;        // 16-column blocks between the LDS reads of V fragments and their MFMAs (two-role kernel)
 constexpr int TILE = KT * AD;          // elements of one K or V tile in LDS (32 KiB), rows unpadded, chunks swizzled
 
 // PHASE_FENCE(): the phases of a tile are scheduled separately
@@ -114,10 +119,8 @@ constexpr int part_o_floats(int RB) { return 4 * RB * AD; }
 constexpr long part_bytes(int RB) { return (long)part_o_floats(RB) * 2 + (long)(4 * 2 * RB) * 4; }
 constexpr int part_ml_floats(int RB) { return 4 * 2 * RB; }
 
-// NH = heads per wavefront: 2 (32 query rows per workgroup, as described above) for long sequences; 1 (16 rows per workgroup,
-// one head per wavefront: twice the workgroups, LDS-bound) when the launch would otherwise leave CUs idle.
+// One head per wavefront: wavefront w owns the workgroup's 16 rows for head w of the KV group.
 // grid = (row blocks, or parts when tmax > 0) x KV heads
-template <int NH>
 __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
                                                            const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
                                                            int q_pos0, long q_head_stride, long kv_head_stride, int tmax,
@@ -128,6 +131,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     __shared__ __align__(1024) bf16_t v_s0[TILE];
     __shared__ __align__(1024) bf16_t v_s1[TILE];
     __shared__ __align__(16) float c_s[4][2][16];
+    constexpr int NH = 1;                                        // heads per wavefront (the loops over them stay, for the shape
+                                                                 // of the arithmetic it shares with attn_prefill_ws_kernel)
     constexpr int RB = 16 * NH;
     // grid = items x KV heads in one dimension, the KV head varying fastest: workgroups are dispatched in the order of their
     // index, so both heads' long row blocks come first
@@ -147,8 +152,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     const int kvh = blockIdx.x % AKV;
     const size_t slot = (size_t)kvh * nitems + (nitems - 1 - item);     // parts of a block: consecutive slots
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
-    const int h0 = kvh * (AH / AKV) + (NH == 2 ? 2 * (w & 1) : w);       // this wavefront's heads: h0 (, h0 + 1)
-    const int r0 = rb * RB + (NH == 2 ? 16 * (w >> 1) : 0), row = r0 + n;   // this wavefront's 16 rows
+    const int h0 = kvh * (AH / AKV) + w;                         // this wavefront's head
+    const int r0 = rb * RB, row = r0 + n;                        // its 16 rows
     const bool row_ok = row < S;
     const int my_last = q_pos0 + row;                            // last key this query row may see
     const int kend = min(L, q_pos0 + min(rb * RB + RB - 1, S - 1) + 1);        // keys any row of the workgroup sees
@@ -485,7 +490,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
         const int first_key = ta * KT, lr0 = r0 - rb * RB;       // this wavefront's first row within the block
 #pragma unroll
         for (int hh = 0; hh < NH; hh++) {
-            const int hq = (NH == 2 ? 2 * (w & 1) : w) + hh;     // head within the KV group
+            const int hq = w + hh;                               // head within the KV group
             _Float16* po = part_o + (slot * 4 + hq) * (RB * AD);
             float* pml = part_ml + (slot * 4 + hq) * (2 * RB);
 #pragma unroll
@@ -510,6 +515,424 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
             if (orow < S) {
                 const float inv = 1.0f / Lsum[hh][r];
                 bf16_t* dst = out + (size_t)(h0 + hh) * q_head_stride + (size_t)orow * AD + n_e;
+#pragma unroll
+                for (int j = 0; j < 16; j++) dst[16 * j] = f2bf(O[hh][j][r] * inv);
+            }
+        }
+    }
+}
+
+// a word of LDS as a volatile object in the LDS address space (through a generic pointer, a volatile access is a flat
+// instruction, which is also counted, and waited for, as an access of global memory)
+__device__ __forceinline__ volatile __attribute__((address_space(3))) int* lds_word(int* shared_word) {
+    return (volatile __attribute__((address_space(3))) int*)shared_word;
+}
+
+// The tile loop with the two halves of a tile's work on different wavefronts.  A workgroup is 32 query rows x 4 heads on
+// eight wavefronts, two per SIMD: wavefront pr (0 .. 3, the "score" wavefront of pair pr) computes the scores and the softmax
+// of rows 16 (pr >> 1) .. + 16 for heads 2 (pr & 1), + 1, and wavefront 4 + pr (the pair's "output" wavefront) multiplies the
+// resulting P by V, one tile behind.  A wavefront's instructions issue one after the other (an MFMA holds its wavefront for
+// about as long as it holds the matrix unit, and every LDS read, exponential or wait comes on top), while two wavefronts
+// of a SIMD do overlap: one feeds the unit Q K^T while the other reads V fragments, and the softmax arithmetic of the one
+// runs beside the P V MFMAs of the other.  (All of it on one wavefront per SIMD, with these 32 rows x 4 heads, measures
+// 5 - 7 % slower; the compiler's order within the score wavefront, the softmax arithmetic as one block and then the MFMA
+// steps back to back, measures better than the same arithmetic tied into the steps.)  With eight wavefronts the 512 registers
+// of a SIMD lane are split in two, 256 per wavefront and no separate accumulation half: the score side holds Q^T (64
+// registers) and two tiles of scores (64), the output side O (128).
+//     iteration t (after barrier X(t): K(t + 1) and V(t - 1) are in LDS):
+//         score wavefront:  softmax of tile t (its scores are in registers since iteration t - 1) and the score MFMAs of
+//                           tile t + 1; then P(t), as packed A operands, and the rows' rescale factors go to LDS
+//         output wavefront: takes P(t - 1) and the factors from LDS, rescales O and the row sums if any row's reference
+//                           moved, O += P(t - 1) V(t - 1)
+//         all eight:        direct-to-LDS loads of K(t + 2) into K(t)'s buffer and of V(t) into V(t - 2)'s
+// P has one buffer per pair: the output wavefront reads it into registers first thing in an iteration and says so
+// (taken_s[pr] = t), and the score wavefront, which writes the next P a few thousand clocks later, looks at that word first.
+// The loader here has no path for fewer than 64 keys: the host picks this kernel from about 1500 query rows on.
+__global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
+                                                              const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
+                                                              int q_pos0, long q_head_stride, long kv_head_stride, int tmax,
+                                                              _Float16* __restrict__ part_o, float* __restrict__ part_ml) {
+    __shared__ __align__(1024) bf16_t kv_s[4 * TILE];            // K tiles of even / odd iterations, then the V tiles
+    __shared__ __align__(16) u32x4 p_s[4][2][2][64];             // [pair][head][32-key half][lane]: P as the lanes hold it
+    __shared__ __align__(16) float c_s[4][2][16];                // [pair][head][row]: factor of a row whose reference moved
+    __shared__ float m_s[4][2][16];                              // final reference points (only the parts' epilogue needs them)
+    __shared__ int moved_s[4];                                   // pair: did any reference move in the tile whose P lies in p_s
+    __shared__ int taken_s[4];                                   // pair: the iteration in which p_s / c_s / moved_s were last read
+    constexpr int RB = 32;
+    const int nitems = gridDim.x / AKV, item = blockIdx.x / AKV;
+    int rb = nitems - 1 - item;                                  // long rows first
+    int part = 0, nparts = 1;
+    if (tmax > 0) {                                              // items are parts (see attn_prefill_kernel)
+        const int c = (KT / RB) * tmax, p = (q_pos0 + RB - 1) / RB;
+        const long y = (long)rb + parts_upto(p, c);
+        int k = 0;
+        while ((long)c * ((k + 1) * (k + 2) / 2) <= y) k++;
+        const int nn = k * c + (int)((y - (long)c * (k * (k + 1) / 2)) / (k + 1));
+        part = (int)(y - parts_upto(nn, c));
+        nparts = k + 1;
+        rb = nn - p;
+    }
+    const int kvh = blockIdx.x % AKV;
+    const size_t slot = (size_t)kvh * nitems + (nitems - 1 - item);
+    const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int pr = w & 3;                                        // pair; w >> 2: 0 = score, 1 = output wavefront
+    const int h0 = kvh * (AH / AKV) + 2 * (pr & 1);
+    const int r0 = rb * RB + 16 * (pr >> 1), row = r0 + n;
+    const bool row_ok = row < S;
+    const int my_last = q_pos0 + row;
+    const int kend = min(L, q_pos0 + min(rb * RB + RB - 1, S - 1) + 1);
+    const int ntiles = (kend + KT - 1) / KT;
+    const int kend_w = r0 < S ? min(L, q_pos0 + min(r0 + 15, S - 1) + 1) : 0;
+    const int ntiles_w = (kend_w + KT - 1) / KT;
+    const int ta = part * tmax, tb = tmax > 0 ? min(ntiles, ta + tmax) : ntiles;
+    const int tw = min(ntiles_w, tb);
+
+    // tile loader: wavefront w issues four direct-to-LDS loads of K and four of V per tile; load i fills rows 8 w + 2 i, + 1
+    // (one KiB): lane l lands at chunk l & 31 of row 8 w + 2 i + (l >> 5) and fetches chunk (l & 31) ^ (row & 15).  L >= KT here.
+    const char* kg = reinterpret_cast<const char*>(K + (size_t)kvh * kv_head_stride);
+    const char* vg = reinterpret_cast<const char*>(V + (size_t)kvh * kv_head_stride);
+    const unsigned ld_row0 = 8u * w + (lane >> 5);
+    const unsigned ld_off0 = ld_row0 * (AD * 2) + ((unsigned)((lane & 31) ^ (ld_row0 & 15u)) << 4);
+    auto tile_row0 = [&](int t) { return max(0, min(t * KT, L - KT)); };
+    auto opaque_off0 = [&]() {
+        unsigned off0 = ld_off0;
+        asm volatile("" : "+v"(off0));
+        return off0;
+    };
+    const unsigned w_lds = 4096u * w;                            // this wavefront's 4 KiB of a tile buffer
+    auto load_four = [&](const char* src, unsigned dst, int t, unsigned off0) {
+        const char* base = src + (size_t)tile_row0(t) * (AD * 2);
+        lds_dma16x4(base, off0, off0 ^ 32u, off0 ^ 64u, off0 ^ 96u, dst + w_lds);
+    };
+    const int ka_row = n * AD;
+    const int vrow = 4 * g + (n >> 2);
+    const int va_row = vrow * AD + 4 * (n & 1), vc0 = (n & 3) >> 1;
+    auto k_frag = [&](const bf16_t* ka, int kt, int kb) {
+        return *reinterpret_cast<const bf16x8*>(ka + 16 * kt * AD + (((4 * (kb & 3) + g) ^ n) << 3) + 128 * (kb >> 2));
+    };
+
+    if (tid < 4) taken_s[tid] = -1, moved_s[tid] = 0;
+    if (tid < 128) (&m_s[0][0][0])[tid] = NEG;
+    if (ta < tb) {                                               // (a part past the block's last tile is empty)
+        load_four(kg, lds_address(kv_s), ta, ld_off0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tb - ta > 1) load_four(kg, lds_address(kv_s) + 2 * TILE, ta + 1, ld_off0);
+    }
+
+    if (w < 4) {
+        // ------------------------------------------------------------------------------------------ score wavefront
+        if (ta >= tb) return;
+        bf16x8 bq[2][8];
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+            const u32x4* qr = reinterpret_cast<const u32x4*>(q + (size_t)(h0 + hh) * q_head_stride + (size_t)(row_ok ? row : 0) * AD);
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) {
+                u32x4 v = qr[kb * 4 + g];
+                if (!row_ok) v = u32x4{0, 0, 0, 0};
+                bq[hh][kb] = __builtin_bit_cast(bf16x8, v);
+            }
+        }
+        float m_run[2] = {NEG, NEG};
+        auto first_scores = [&](f32x4 (&acc0)[2][4]) {
+            const bf16_t* ka = kv_s + ka_row;
+            bf16x8 Af[2][8];
+#pragma unroll
+            for (int kb = 0; kb < 8; kb++) Af[0][kb] = k_frag(ka, 0, kb);
+#pragma unroll
+            for (int kt = 0; kt < 4; kt++) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (kt < 3) {
+#pragma unroll
+                    for (int kb = 0; kb < 8; kb++) Af[(kt + 1) & 1][kb] = k_frag(ka, kt + 1, kb);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++) acc0[hh][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kb = 0; kb < 8; kb++)
+#pragma unroll
+                    for (int hh = 0; hh < 2; hh++)
+                        acc0[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kt & 1][kb], bq[hh][kb], acc0[hh][kt], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        f32x4 acc[2][4] = {};                                    // scores of tile t
+        if (tw > ta) first_scores(acc);
+        for (int t = ta; t <= tb; t++) {
+            const unsigned par = (unsigned)(t - ta) & 1u;
+            const unsigned k_cur = lds_address(kv_s) + par * (2 * TILE);           // K(t): consumed, refilled with K(t + 2)
+            const bf16_t* const k_nxt = kv_s + (par ^ 1u) * TILE;                  // K(t + 1)
+            const unsigned v_new = lds_address(kv_s) + 4 * TILE + par * (2 * TILE);   // takes V(t)
+            PHASE_FENCE();
+            // this wavefront's loads of K(t + 1), V(t - 1) have landed, and its writes of P(t - 1) (the wait for those is
+            // spelled out: at a loop header the compiler does not always see the LDS stores that arrive over the back edge)
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            PHASE_FENCE();
+            __syncthreads();                                         // X(t)
+            const bool more = t + 1 < tw;
+            const int tk = min(t + 2, tb - 1);
+            if (!more) {
+                if (t + 2 < tb) load_four(kg, k_cur, t + 2, opaque_off0());
+                if (t < tb) load_four(vg, v_new, t, opaque_off0());
+            }
+            PHASE_FENCE();
+            if (t >= tw) continue;
+            if (t * KT + KT - 1 > q_pos0 + r0 || t * KT + KT > L) {
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+                    for (int kt = 0; kt < 4; kt++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int key = tile_row0(t) + 16 * kt + 4 * g + i;
+                            if (!(key >= t * KT && key <= my_last && key < L)) acc[hh][kt][i] = NEG;
+                        }
+            }
+            const bf16_t* ka = k_nxt + ka_row;
+            f32x4 acc_next[2][4];
+            // Tile t's softmax rides on the 32 score steps of tile t + 1.  The exponentials are taken against the running
+            // reference points on the bet that no row's maximum grows by more than 2^LAZY in this tile; the maxima are folded
+            // in beside them and the bet is checked in `publish`.
+            auto publish = [&](s16x8 (&P)[2][2], float (&mx)[2], int taken_early) {
+                bool grow = false;
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++) {
+                    mx[hh] = max_over_groups(mx[hh]) * SCALE_LOG2E;
+                    grow |= mx[hh] > m_run[hh] + LAZY;
+                }
+                const bool any_grow = __any(grow);
+                float corr[2] = {1.f, 1.f};
+                if (any_grow) {                                      // wavefront-uniform and rare
+#pragma unroll
+                    for (int hh = 0; hh < 2; hh++) {
+                        const float m_new = mx[hh] > m_run[hh] + LAZY ? mx[hh] : m_run[hh];
+                        corr[hh] = __builtin_amdgcn_exp2f(m_run[hh] - m_new);    // m_run = NEG initially: 2^-huge = 0
+                        m_run[hh] = m_new;
+                        // this tile's p again, against the new reference points (rows that did not move get the same bits)
+#pragma unroll
+                        for (int kt2 = 0; kt2 < 4; kt2++)
+#pragma unroll
+                            for (int i = 0; i < 4; i += 2) {
+                                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_new));
+                                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i + 1], SCALE_LOG2E, -m_new));
+                                const uint32_t pk = pack_bf(p0, p1);
+                                P[hh][kt2 >> 1][(kt2 & 1) * 4 + i] = (short)(pk & 0xffff);
+                                P[hh][kt2 >> 1][(kt2 & 1) * 4 + i + 1] = (short)(pk >> 16);
+                            }
+                    }
+                }
+                // the pair's buffers are free once the output wavefront has read tile t - 1 out of them (it does so first
+                // thing in this iteration; the word was read some steps ago, so that its LDS latency is not waited for here).
+                // The wait is bounded: the word is always written, and a bound costs nothing.
+                if (t > ta && __builtin_amdgcn_readfirstlane(taken_early) != t) {
+                    for (int spin = 0; spin < (1 << 16); spin++) {
+                        if (__builtin_amdgcn_readfirstlane(*lds_word(&taken_s[pr])) == t) break;
+                        __builtin_amdgcn_s_sleep(1);
+                    }
+                }
+                asm volatile("" ::: "memory");
+                if (any_grow) {
+                    c_s[pr][0][n] = corr[0];                         // all four groups store the same value
+                    c_s[pr][1][n] = corr[1];
+                }
+                moved_s[pr] = any_grow ? 1 : 0;
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+                    for (int pp = 0; pp < 2; pp++) p_s[pr][hh][pp][lane] = __builtin_bit_cast(u32x4, P[hh][pp]);
+                if (t == tw - 1) {
+                    m_s[pr][0][n] = m_run[0];
+                    m_s[pr][1][n] = m_run[1];
+                }
+            };
+            auto body = [&](auto with_scores) {
+                constexpr bool SC = decltype(with_scores)::value;
+                s16x8 P[2][2];
+                float mx[2] = {NEG, NEG};
+                bf16x8 Af[FRAG_AHEAD + 1];
+                if (SC) {
+#pragma unroll
+                    for (int f = 0; f < FRAG_AHEAD; f++) Af[f] = k_frag(ka, f >> 3, f & 7);
+                }
+                // softmax elements 2 e, 2 e + 1 of tile t
+                auto softmax_pair = [&](int e) {
+                    const int hh = e >> 3, kt2 = (e >> 1) & 3, i = 2 * (e & 1);
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_run[hh]));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i + 1], SCALE_LOG2E, -m_run[hh]));
+                    mx[hh] = fmaxf(mx[hh], fmaxf(acc[hh][kt2][i], acc[hh][kt2][i + 1]));
+                    const uint32_t pk = pack_bf(p0, p1);
+                    P[hh][kt2 >> 1][(kt2 & 1) * 4 + i] = (short)(pk & 0xffff);
+                    P[hh][kt2 >> 1][(kt2 & 1) * 4 + i + 1] = (short)(pk >> 16);
+                };
+                PHASE_FENCE();
+                const unsigned step_off0 = SC ? opaque_off0() : 0u;
+                int taken_early = -1;
+#pragma unroll
+                for (int st = 0; st < 32; st++) {
+                    const int kt = st >> 3, kb = st & 7;
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (SC && st == 0) load_four(kg, k_cur, tk, step_off0);
+                    if (SC && st == 20) load_four(vg, v_new, t, step_off0);
+                    if (SC) {
+                        if (st + FRAG_AHEAD < 32)
+                            Af[(st + FRAG_AHEAD) % (FRAG_AHEAD + 1)] = k_frag(ka, (st + FRAG_AHEAD) >> 3, (st + FRAG_AHEAD) & 7);
+#pragma unroll
+                        for (int hh = 0; hh < 2; hh++)
+                            acc_next[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                Af[st % (FRAG_AHEAD + 1)], bq[hh][kb], kb == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc_next[hh][kt], 0, 0, 0);
+                    }
+                    if ((st & 1) == 0) softmax_pair(st >> 1);
+                    if (st == 20) taken_early = *lds_word(&taken_s[pr]);   // (read early: its LDS latency passes under the steps)
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                publish(P, mx, taken_early);
+            };
+            if (more)
+                body(std::true_type{});
+            else
+                body(std::false_type{});
+            PHASE_FENCE();
+            if (more) {
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+                    for (int kt = 0; kt < 4; kt++) acc[hh][kt] = acc_next[hh][kt];
+            }
+            PHASE_FENCE();
+        }
+        return;
+    }
+    // ---------------------------------------------------------------------------------------------- output wavefront
+    f32x4 O[2][16];
+    f32x4 Lsum[2];                                                   // row sums of P, accumulated by MFMA against a block of ones
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+        Lsum[hh] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 16; j++) O[hh][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    // iterations in which this wavefront only loads: the first one (no P yet), and those after its rows' last tile
+    auto idle_iter = [&](int t) {
+        const unsigned par = (unsigned)(t - ta) & 1u;
+        PHASE_FENCE();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PHASE_FENCE();
+        __syncthreads();                                             // X(t)
+        if (t + 2 < tb) load_four(kg, lds_address(kv_s) + par * (2 * TILE), t + 2, opaque_off0());
+        if (t < tb) load_four(vg, lds_address(kv_s) + 4 * TILE + par * (2 * TILE), t, opaque_off0());
+    };
+    if (ta < tb) idle_iter(ta);
+    for (int t = ta + 1; t <= tw; t++) {                             // (tw <= tb; nothing if tw <= ta)
+        const unsigned par = (unsigned)(t - ta) & 1u;
+        const unsigned k_cur = lds_address(kv_s) + par * (2 * TILE);               // takes K(t + 2)
+        const unsigned v_new = lds_address(kv_s) + 4 * TILE + par * (2 * TILE);    // takes V(t)
+        const bf16_t* const v_cur = kv_s + 2 * TILE + (par ^ 1u) * TILE;           // V(t - 1)
+        PHASE_FENCE();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PHASE_FENCE();
+        __syncthreads();                                             // X(t)
+        const int mv = __builtin_amdgcn_readfirstlane(moved_s[pr]);
+        s16x8 P[2][2];
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) P[hh][pp] = __builtin_bit_cast(s16x8, p_s[pr][hh][pp][lane]);
+        f32x4 c4[2] = {f32x4{1.f, 1.f, 1.f, 1.f}, f32x4{1.f, 1.f, 1.f, 1.f}};
+        if (mv) {
+            c4[0] = *reinterpret_cast<const f32x4*>(&c_s[pr][0][4 * g]);
+            c4[1] = *reinterpret_cast<const f32x4*>(&c_s[pr][1][4 * g]);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        *lds_word(&taken_s[pr]) = t;
+        asm volatile("" ::: "memory");
+        const bf16_t* va = v_cur + va_row;
+        auto v_frag = [&](int j, int q4) {
+            return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * AD + (((2 * (j & 7) + vc0) ^ vrow) << 3) +
+                                                                             128 * (j >> 3))));
+        };
+        s16x4 Bf[V_FRAG_AHEAD + 1][4];
+#pragma unroll
+        for (int j = 0; j < V_FRAG_AHEAD; j++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) Bf[j][q4] = v_frag(j, q4);
+        if (mv) {                                                    // a reference moved: rescale what is accumulated
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+#pragma unroll
+                for (int j = 0; j < 16; j++) O[hh][j] *= c4[hh];
+                Lsum[hh] *= c4[hh];
+            }
+        }
+        PHASE_FENCE();
+        {                                                            // the row sums: P . 1, the sum of exactly the rounded values
+            s16x8 ones;
+#pragma unroll
+            for (int e = 0; e < 8; e++) ones[e] = (short)0x3f80;
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++)
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++)
+                    Lsum[hh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[hh][pp]),
+                                                                      __builtin_bit_cast(bf16x8, ones), Lsum[hh], 0, 0, 0);
+        }
+        const unsigned step_off0 = opaque_off0();
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (j == 0 && t + 2 < tb) load_four(kg, k_cur, t + 2, step_off0);
+            if (j == 8 && t < tb) load_four(vg, v_new, t, step_off0);
+            if (j + V_FRAG_AHEAD < 16) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) Bf[(j + V_FRAG_AHEAD) % (V_FRAG_AHEAD + 1)][q4] = v_frag(j + V_FRAG_AHEAD, q4);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                const s16x8 B = __builtin_shufflevector(Bf[j % (V_FRAG_AHEAD + 1)][2 * pp], Bf[j % (V_FRAG_AHEAD + 1)][2 * pp + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++)
+                    O[hh][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[hh][pp]),
+                                                                      __builtin_bit_cast(bf16x8, B), O[hh][j], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        PHASE_FENCE();
+    }
+    if (ta < tb)
+        for (int t = max(tw, ta) + 1; t <= tb; t++) idle_iter(t);
+    if (nparts > 1) {
+        // one part of several (see attn_prefill_kernel): O / l, m, l of this pair's heads; rows that see no key of the part
+        // are written as the neutral element
+        const int first_key = ta * KT, lr0 = r0 - rb * RB;
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+            const int hq = 2 * (pr & 1) + hh;
+            _Float16* po = part_o + (slot * 4 + hq) * (RB * AD);
+            float* pml = part_ml + (slot * 4 + hq) * (2 * RB);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int lr = lr0 + 4 * g + r;
+                const bool seen = q_pos0 + rb * RB + lr >= first_key;
+                const float inv = seen ? 1.0f / Lsum[hh][r] : 0.f;
+#pragma unroll
+                for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n] = (_Float16)(seen ? O[hh][j][r] * inv : 0.f);
+                if (n == 0) pml[RB + lr] = seen ? Lsum[hh][r] : 0.f;
+            }
+            if (g == 0) pml[lr0 + n] = my_last >= first_key ? m_s[pr][hh][n] : NEG;
+        }
+        return;
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int orow = r0 + 4 * g + r;
+            if (orow < S) {
+                const float inv = 1.0f / Lsum[hh][r];
+                bf16_t* dst = out + (size_t)(h0 + hh) * q_head_stride + (size_t)orow * AD + n;
 #pragma unroll
                 for (int j = 0; j < 16; j++) dst[16 * j] = f2bf(O[hh][j][r] * inv);
             }
@@ -619,7 +1042,7 @@ KeySplit plan_split_nh(int S, int L, int q_pos0, int nh, int min_gain) {
 //                               2 us for two 16-row blocks, but its parts are twice the size);
 //   everything else             one head per wavefront, split if CUs would idle.
 KeySplit plan_split(int S, int L, int q_pos0) {
-    if (two_heads_per_wave(S)) {
+    if (two_heads_per_wave(S)) {                                 // (two heads: S >= 1472 in every case, so L >= one tile)
         KeySplit ks;
         ks.nh = 2;
         return ks;
@@ -674,10 +1097,10 @@ int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out
     _Float16* part_o = ks.tmax ? (_Float16*)workspace : nullptr;
     float* part_ml = ks.tmax ? reinterpret_cast<float*>(part_o + (size_t)ks.parts * AKV * part_o_floats(RB)) : nullptr;
     if (ks.nh == 2)
-        hipLaunchKernelGGL(attn_prefill_kernel<2>, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
+        hipLaunchKernelGGL(attn_prefill_ws_kernel, grid, dim3(512), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
                            (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
     else
-        hipLaunchKernelGGL(attn_prefill_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
+        hipLaunchKernelGGL(attn_prefill_kernel, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
                            (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
     if (ks.tmax) {
         const dim3 mgrid((unsigned)ks.split_blocks, AKV, (AH / AKV) * ks.nh);

@@ -175,7 +175,8 @@ def test_no_kernel_spills_or_reaches_a_barrier_with_an_unwaited_lds_store(tmp_pa
         with open(out) as f:
             asm = f.read()
         if os.path.basename(src) == "gqa_prefill.hip":
-            assert partial_lds_waits(asm, "attn_prefill_kernel") >= 50, "the tile loop waits for every LDS read in full"
+            for kernel in ("attn_prefill_kernel", "attn_prefill_ws_kernel"):
+                assert partial_lds_waits(asm, kernel) >= 50, f"{kernel}: the tile loop waits for every LDS read in full"
         return os.path.basename(src), asm.count("s_barrier"), unwaited_barriers(asm), scratch_users(asm)
 
     with ThreadPoolExecutor(max_workers=8) as ex:

@@ -268,6 +268,25 @@ def test_prefill_causal_reference_points_that_move_late(qt, dev, S):
         check_attn(f"S={S} row {r}", o[:, r:r + 1], O.sdpa_causal(qn[:, r:r + 1], Kn[:, :r + 1], Vn[:, :r + 1]))
 
 
+@pytest.mark.parametrize("S,P0", [(4800, 0), (2048, 0), (1536, 1000), (6001, 333)])
+def test_prefill_causal_two_role_kernel_is_repeatable(qt, dev, S, P0):
+    """From about 1500 rows on, a workgroup's wavefronts work in pairs: one computes a tile's scores and softmax and hands P (with
+    the rows' rescale factors) to its partner through LDS, one tile ahead of the partner's P.V.  An access of that hand-over that
+    is not ordered shows as a result that depends on timing: five calls on the same inputs (unsplit, split, after a prefix,
+    ragged) must agree in every bit, with other work on the GPU between them."""
+    L = S + P0
+    g = torch.Generator().manual_seed(S + P0)
+    q = torch.randn((1, 8, S, 256), generator=g).bfloat16().to(dev)
+    K = torch.randn((1, 2, L, 256), generator=g).bfloat16().to(dev)
+    V = torch.randn((1, 2, L, 256), generator=g).bfloat16().to(dev)
+    first = qt.attention.scaled_dot_product_attention(q, K, V, scale=256 ** -0.5, mask="causal").clone()
+    assert bool(torch.isfinite(first.float()).all())
+    for i in range(4):
+        (K.float() * (i + 2)).sum().item()                       # unrelated kernels and a synchronisation in between
+        again = qt.attention.scaled_dot_product_attention(q, K, V, scale=256 ** -0.5, mask="causal")
+        assert torch.equal(first, again), f"call {i + 2} differs from the first"
+
+
 def test_prefill_causal_long_ragged_continuation(qt, dev):
     """two heads per wavefront with nothing aligned: S = 8170 query rows continue a prefix of 37 keys (L = 8207: the last tile is
     shifted back, the last row blocks are partial, some wavefronts have one tile less than their workgroup)"""
