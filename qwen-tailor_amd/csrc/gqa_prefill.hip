@@ -2,13 +2,11 @@
 // Replaces the call mx.fast.scaled_dot_product_attention(q, K[:, :, :kv_len], V[:, :, :kv_len], scale=256**-0.5,
 // mask="causal") of the reference's full-attention layers (qwen35/model.py:160-167, qwen35/prefill.py:468).
 //
-// Two kernels over one data path:
-//   attn_prefill_ws_kernel   32 query rows x the 4 query heads that share a KV head per workgroup, on eight wavefronts in two
-//                            roles (a "score" and an "output" wavefront per 16 rows x 2 heads): launches of about 1500 rows
-//                            and more.  Every K or V fragment read from LDS feeds two MFMAs (one per head).
-//   attn_prefill_kernel      16 query rows x the 4 heads, one head per wavefront, the whole tile loop on each: twice the
-//                            workgroups (and twice the LDS traffic per MFMA), for launches that would otherwise leave CUs idle.
-// The data path, per 64-key tile and 16 rows of a head:
+// attn_prefill_kernel<NH>: one workgroup = 16 NH query rows x the 4 query heads that share a KV head, on eight wavefronts in
+// two roles; NH = heads per pair of wavefronts:
+//   NH = 2   32 rows; every K or V fragment read from LDS feeds two MFMAs (one per head): launches of about 1500 rows and more
+//   NH = 1   16 rows: twice the workgroups (and twice the LDS traffic per MFMA), for launches that would leave CUs idle
+// The arithmetic, per 64-key tile and 16 rows of a head:
 //     S^T[keys x rows] = K_tile . Q^T     A = K rows from LDS, B = Q^T resident in registers (16x16x32 bf16 MFMA)
 //     online softmax in the accumulator layout: lane (row n, group g) holds keys 4g..4g+3 of each 16-key sub-tile
 //     O[rows x 256]   += P . V            A = two exponentiated S^T accumulators packed to bf16 (they ARE the A operand
@@ -18,9 +16,9 @@
 // K / V tiles travel HBM -> LDS directly (global_load_lds_dwordx4: 64 lanes x 16 bytes land as one contiguous KiB, no
 // registers in between) into double-buffered tiles.  The LDS rows are unpadded (a direct load cannot pad); instead the
 // 16-byte chunks of row r are stored XOR-swizzled by r & 15 (the loading lane picks the matching global chunk), which keeps
-// the fragment reads of 16 rows on distinct banks.  The tile loops are software-pipelined around one workgroup barrier per
-// tile: the score MFMAs of tile t + 1 run while tile t is exponentiated, against the running reference points, before the
-// tile's row maxima are known; the bet is checked afterwards (see `tile` and `publish` below).
+// the fragment reads of 16 rows on distinct banks.  The tile loop runs around one workgroup barrier per tile: the score MFMAs
+// of tile t + 1 follow the exponentials of tile t, which are taken against the running reference points before the tile's
+// row maxima are known; the bet is checked afterwards (see `publish` below).
 #include "qt_common.h"
 
 #include <algorithm>
@@ -41,17 +39,11 @@ constexpr float NEG = -3.0e38f;
 constexpr float LAZY = 8.0f;            // log2 of the growth of a row maximum that is tolerated before the row is rescaled
 constexpr int KT = 64;                 // keys per tile
 constexpr int FRAG_AHEAD = 5;          // steps between the LDS read of a K fragment and its MFMAs in the tile loop
-constexpr int V_FRAG_AHEAD = 2;        // 16-column blocks between the LDS reads of V fragments and their MFMAs (two-role kernel)
+constexpr int V_FRAG_AHEAD = 2;        // 16-column blocks between the LDS reads of V fragments and their MFMAs
 constexpr int TILE = KT * AD;          // elements of one K or V tile in LDS (32 KiB), rows unpadded, chunks swizzled
 
-// PHASE_FENCE(): the phases of a tile are scheduled separately
+// PHASE_FENCE(): the phases of an iteration are scheduled separately
 #define PHASE_FENCE() __builtin_amdgcn_sched_barrier(0)
-
-__device__ __forceinline__ void wave_lds_sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 
 // One direct-to-LDS load of 16 bytes per lane (global_load_lds_dwordx4): lane l fetches base + voff + IMM and the 64 pieces land
 // at lds + IMM + 16 l.  Issued as inline assembly, not through the builtin: while a direct-to-LDS load that the compiler knows
@@ -96,11 +88,6 @@ __device__ __forceinline__ float max_over_groups(float x) {
     return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
-// The output accumulators live in the accumulation half of the register file, which MFMA reads and writes in place; only the
-// rare rescale moves them through VALU registers.  The empty asm ties that move to the inside of the rescale branch (otherwise
-// it is hoisted to the top of every tile and holds 128 VALU registers through the score phase).
-#define PIN_ACC(x) asm volatile("" : "+a"(x))
-
 // Key split.  A causal launch with few workgroups is as slow as its longest row block, twice the average.  With tmax > 0 the
 // tiles of a row block (RB = 16 or 32 rows) are cut into parts of tmax tiles, one workgroup per part; a block with more than
 // one part leaves unnormalised partial results (O, reference point m, row sums l) in the workspace and
@@ -119,23 +106,46 @@ constexpr int part_o_floats(int RB) { return 4 * RB * AD; }
 constexpr long part_bytes(int RB) { return (long)part_o_floats(RB) * 2 + (long)(4 * 2 * RB) * 4; }
 constexpr int part_ml_floats(int RB) { return 4 * 2 * RB; }
 
-// One head per wavefront: wavefront w owns the workgroup's 16 rows for head w of the KV group.
-// grid = (row blocks, or parts when tmax > 0) x KV heads
-__global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
-                                                           const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
-                                                           int q_pos0, long q_head_stride, long kv_head_stride, int tmax,
-                                                           _Float16* __restrict__ part_o, float* __restrict__ part_ml) {
-    // four separate arrays: the loaders take each buffer's LDS address as a constant (lds_address)
-    __shared__ __align__(1024) bf16_t k_s0[TILE];
-    __shared__ __align__(1024) bf16_t k_s1[TILE];
-    __shared__ __align__(1024) bf16_t v_s0[TILE];
-    __shared__ __align__(1024) bf16_t v_s1[TILE];
-    __shared__ __align__(16) float c_s[4][2][16];
-    constexpr int NH = 1;                                        // heads per wavefront (the loops over them stay, for the shape
-                                                                 // of the arithmetic it shares with attn_prefill_ws_kernel)
+// a word of LDS as a volatile object in the LDS address space (through a generic pointer, a volatile access is a flat
+// instruction, which is also counted, and waited for, as an access of global memory)
+__device__ __forceinline__ volatile __attribute__((address_space(3))) int* lds_word(int* shared_word) {
+    return (volatile __attribute__((address_space(3))) int*)shared_word;
+}
+
+// The tile loop, with the two halves of a tile's work on different wavefronts.  The eight wavefronts of a workgroup, two per
+// SIMD, form four pairs: wavefront pr (0 .. 3, the "score" wavefront of pair pr) computes the scores and the softmax of the
+// pair's 16 rows x NH heads (NH = 2: rows 16 (pr >> 1) .. + 16 of the block, heads 2 (pr & 1), + 1; NH = 1: the block's 16 rows,
+// head pr), and wavefront 4 + pr (the pair's "output" wavefront) multiplies the resulting P by V, one tile behind.  A
+// wavefront's instructions issue one after the other (an MFMA holds its wavefront for about as long as it holds the matrix
+// unit, and every LDS read, exponential or wait comes on top), while two wavefronts of a SIMD do overlap: one feeds the unit
+// Q K^T while the other reads V fragments, and the softmax arithmetic of the one runs beside the P V MFMAs of the other.
+// (The whole loop on one wavefront per SIMD, four per workgroup, measured 5 - 12 % slower on the same rows and heads; the
+// compiler's order within the score wavefront, the softmax arithmetic as one block and then the MFMA steps back to back,
+// measures better than the same arithmetic tied into the steps.)  With eight wavefronts the 512 registers of a SIMD lane are
+// split in two, 256 per wavefront and no separate accumulation half: for NH = 2 the score side holds Q^T (64 registers) and
+// two tiles of scores (64), the output side O (128).
+//     iteration t (after barrier X(t): K(t + 1) and V(t - 1) are in LDS):
+//         score wavefront:  softmax of tile t (its scores are in registers since iteration t - 1) and the score MFMAs of
+//                           tile t + 1; then P(t), as packed A operands, and the rows' rescale factors go to LDS
+//         output wavefront: takes P(t - 1) and the factors from LDS, rescales O and the row sums if any row's reference
+//                           moved, O += P(t - 1) V(t - 1)
+//         all eight:        direct-to-LDS loads of K(t + 2) into K(t)'s buffer and of V(t) into V(t - 2)'s
+// P has one buffer per pair: the output wavefront reads it into registers first thing in an iteration and says so
+// (taken_s[pr] = t), and the score wavefront, which writes the next P a few thousand clocks later, looks at that word first.
+// grid = (row blocks, or parts when tmax > 0) x KV heads in one dimension, the KV head varying fastest: workgroups are
+// dispatched in the order of their index, so both heads' long row blocks come first.
+template <int NH>
+__global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
+                                                              const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
+                                                              int q_pos0, long q_head_stride, long kv_head_stride, int tmax,
+                                                              _Float16* __restrict__ part_o, float* __restrict__ part_ml) {
+    __shared__ __align__(1024) bf16_t kv_s[4 * TILE];            // K tiles of even / odd iterations, then the V tiles
+    __shared__ __align__(16) u32x4 p_s[4][NH][2][64];             // [pair][head][32-key half][lane]: P as the lanes hold it
+    __shared__ __align__(16) float c_s[4][NH][16];               // [pair][head][row]: factor of a row whose reference moved
+    __shared__ float m_s[4][NH][16];                             // final reference points (only the parts' epilogue needs them)
+    __shared__ int moved_s[4];                                   // pair: did any reference move in the tile whose P lies in p_s
+    __shared__ int taken_s[4];                                   // pair: the iteration in which p_s / c_s / moved_s were last read
     constexpr int RB = 16 * NH;
-    // grid = items x KV heads in one dimension, the KV head varying fastest: workgroups are dispatched in the order of their
-    // index, so both heads' long row blocks come first
     const int nitems = gridDim.x / AKV, item = blockIdx.x / AKV;
     int rb = nitems - 1 - item;                                  // long rows first
     int part = 0, nparts = 1;
@@ -152,448 +162,33 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const bf16_t* __re
     const int kvh = blockIdx.x % AKV;
     const size_t slot = (size_t)kvh * nitems + (nitems - 1 - item);     // parts of a block: consecutive slots
     const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
-    const int h0 = kvh * (AH / AKV) + w;                         // this wavefront's head
-    const int r0 = rb * RB, row = r0 + n;                        // its 16 rows
+    const int pr = w & 3;                                        // pair; w >> 2: 0 = score, 1 = output wavefront
+    const int hq0 = NH == 2 ? 2 * (pr & 1) : pr;                  // this pair's first head within the KV group
+    const int h0 = kvh * (AH / AKV) + hq0;
+    const int r0 = rb * RB + (NH == 2 ? 16 * (pr >> 1) : 0), row = r0 + n;
     const bool row_ok = row < S;
     const int my_last = q_pos0 + row;                            // last key this query row may see
     const int kend = min(L, q_pos0 + min(rb * RB + RB - 1, S - 1) + 1);        // keys any row of the workgroup sees
     const int ntiles = (kend + KT - 1) / KT;
-    const int kend_w = r0 < S ? min(L, q_pos0 + min(r0 + 15, S - 1) + 1) : 0;  // keys any row of this wavefront sees
+    const int kend_w = r0 < S ? min(L, q_pos0 + min(r0 + 15, S - 1) + 1) : 0;  // keys any row of this pair sees
     const int ntiles_w = (kend_w + KT - 1) / KT;
-    // this workgroup's tiles [ta, tb); tw: where this wavefront's rows end
-    const int ta = part * tmax, tb = tmax > 0 ? min(ntiles, ta + tmax) : ntiles;
-    const int tw = min(ntiles_w, tb);
-
-    // Q^T as the B operand of the score MFMA: lane (row n, group g) holds q[row][32 kb + 8 g .. + 8], for both heads
-    bf16x8 bq[NH][8];
-#pragma unroll
-    for (int hh = 0; hh < NH; hh++) {
-        const u32x4* qr = reinterpret_cast<const u32x4*>(q + (size_t)(h0 + hh) * q_head_stride + (size_t)(row_ok ? row : 0) * AD);
-#pragma unroll
-        for (int kb = 0; kb < 8; kb++) {
-            u32x4 v = qr[kb * 4 + g];
-            if (!row_ok) v = u32x4{0, 0, 0, 0};
-            bq[hh][kb] = __builtin_bit_cast(bf16x8, v);
-        }
-    }
-    // tile loader: wavefront w issues direct-to-LDS loads i = 0..7 of K and of V; load 8 w + i fills rows 2 (8 w + i) and
-    // + 1 (one KiB): lane l lands at chunk position l & 31 of row 2 (8 w + i) + (l >> 5) and fetches chunk (l & 31) ^ (row & 15).
-    // The per-lane byte offsets within a tile do not change from tile to tile.  A tile that would run past the end of the
-    // sequence is shifted back to end at L (tile_row0): its first rows repeat keys of the tile before and are masked.  Only a
-    // sequence shorter than one tile repeats its last key instead (slow path, first tile only).
-    const char* kg = reinterpret_cast<const char*>(K + (size_t)kvh * kv_head_stride);
-    const char* vg = reinterpret_cast<const char*>(V + (size_t)kvh * kv_head_stride);
-    // byte offset of load 0 within a tile; load i differs by XOR with 1056 i (row bits 10..12, chunk bits 5..7)
-    const unsigned ld_off0 = (unsigned)(16 * w + (lane >> 5)) * (AD * 2) + ((unsigned)((lane & 31) ^ (lane >> 5)) << 4);
-    auto tile_row0 = [&](int t) { return max(0, min(t * KT, L - KT)); };
-    // a copy of ld_off0 the compiler cannot see through: the offsets of the eight loads are then recomputed where they are
-    // used (one XOR each) instead of living in registers the accumulators need
-    auto opaque_off0 = [&]() {
-        unsigned off0 = ld_off0;
-        asm volatile("" : "+v"(off0));
-        return off0;
-    };
-    // the row part of a load (2 i rows = 1024 i bytes) goes into the instruction's immediate offset, which moves the global
-    // address and the LDS destination alike (at most 4095: the upper four loads start 4 KiB further in both)
-    // (dst: LDS byte address of the tile buffer)
-    const unsigned w_lds = 8192u * w;                            // this wavefront's 8 KiB of a tile buffer
-    auto load_four = [&](const char* src, unsigned dst, int t, int half, unsigned off0) {   // loads 4 half .. 4 half + 3 of tile t
-        const char* base = src + (size_t)tile_row0(t) * (AD * 2) + 4096 * half;
-        const unsigned i0 = 4u * half;
-        lds_dma16x4(base, off0 ^ (32u * i0), off0 ^ (32u * (i0 + 1)), off0 ^ (32u * (i0 + 2)), off0 ^ (32u * (i0 + 3)),
-                    dst + w_lds + 4096u * half);
-    };
-    auto load_rows = [&](const char* src, unsigned dst, int t) {  // one K or V tile: this wavefront's eight direct loads
-        if (L >= KT) {
-            const unsigned off0 = opaque_off0();
-            load_four(src, dst, t, 0, off0);
-            load_four(src, dst, t, 1, off0);
-        } else {                                                 // t = 0: rows past the end repeat the last key; they are masked
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const unsigned o = ld_off0 ^ (1056u * i);
-                const unsigned off = (unsigned)min((int)(o >> 9), L - 1) * (AD * 2) + (o & 511u);
-                lds_dma16<0>(src, off, dst + w_lds + 1024u * i);
-            }
-        }
-    };
-
-    float m_run[NH];
-    f32x4 Lsum[NH];                                              // row sums of P, accumulated by MFMA against a block of ones
-    f32x4 O[NH][16];
-#pragma unroll
-    for (int hh = 0; hh < NH; hh++)
-#pragma unroll
-        for (int j = 0; j < 16; j++) O[hh][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int hh = 0; hh < NH; hh++) m_run[hh] = NEG, Lsum[hh] = f32x4{0.f, 0.f, 0.f, 0.f};
-    // A operand of the scores: row 16 kt + n of the tile, chunk (4 kb + g) ^ n
-    const int ka_row = n * AD;
-    // transposing load: within 16 lanes, lane 4q + i receives element i of the 8-byte chunks addressed by lanes q, q+4,
-    // q+8, q+12; lane n of group g points at key 4g + n/4, columns 4 (n%4).. of the block and receives keys 4g..4g+3 of column n
-    const int vrow = 4 * g + (n >> 2);                           // row within a 16-key block = its swizzle
-    const int va_row = vrow * AD + 4 * (n & 1), vc0 = (n & 3) >> 1;
-
-    // K fragment kb of sub-tile kt
-    auto k_frag = [&](const bf16_t* ka, int kt, int kb) {
-        // chunk (4 kb + g) ^ n; n < 16 leaves bit 4 alone, so fragments kb and kb + 4 share an address register
-        return *reinterpret_cast<const bf16x8*>(ka + 16 * kt * AD + (((4 * (kb & 3) + g) ^ n) << 3) + 128 * (kb >> 2));
-    };
-    // scores of tile 0, S^T = K_tile . Q^T: each K fragment multiplies the Q^T of both heads; the fragments of the next
-    // 16-key sub-tile are read while the MFMAs of the current one run
-    auto scores_first = [&](const bf16_t* ka, f32x4 (&acc)[NH][4]) {
-        bf16x8 Af[2][8];
-#pragma unroll
-        for (int kb = 0; kb < 8; kb++) Af[0][kb] = k_frag(ka, 0, kb);
-#pragma unroll
-        for (int kt = 0; kt < 4; kt++) {
-            __builtin_amdgcn_sched_barrier(0);
-            if (kt < 3) {
-#pragma unroll
-                for (int kb = 0; kb < 8; kb++) Af[(kt + 1) & 1][kb] = k_frag(ka, kt + 1, kb);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int hh = 0; hh < NH; hh++) acc[hh][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int kb = 0; kb < 8; kb++)
-#pragma unroll
-                for (int hh = 0; hh < NH; hh++)
-                    acc[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kt & 1][kb], bq[hh][kb], acc[hh][kt], 0, 0, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    f32x4 accs[2][NH][4];                                        // scores of tile t live in accs[t & 1]
-    // One tile, software-pipelined around ONE workgroup barrier X(t):
-    //     before X(t): the scores of tile t are in registers (computed during tile t - 1), P.V of tile t - 1 is done
-    //     at X(t):     K(t + 1) and V(t) have landed; K(t)'s buffer takes K(t + 2), V(t - 1)'s buffer takes V(t + 1)
-    //     after X(t):  the score MFMAs of tile t + 1 are interleaved, step by step, with the softmax VALU work of tile t
-    //                  (online softmax in base 2 on the raw products: p = 2^(c s - m), c = 256^-0.5 log2 e; every row sees
-    //                  key 0, so its maximum is finite from the first tile on and masked entries come out as 2^-huge = 0);
-    //                  then P.V(t)
-    // PAR = t & 1 picks the buffers at compile time.
-    auto tile = [&](const int t, auto par) {
-        constexpr int PAR = decltype(par)::value;
-        f32x4 (&acc)[NH][4] = accs[PAR];
-        f32x4 (&acc_next)[NH][4] = accs[PAR ^ 1];
-        const unsigned k_cur = lds_address(PAR ? k_s1 : k_s0);   // K(t): consumed already, refilled with K(t + 2)
-        const bf16_t* const k_nxt = PAR ? k_s0 : k_s1;           // K(t + 1)
-        const bf16_t* const v_cur = PAR ? v_s1 : v_s0;           // V(t)
-        const unsigned v_nxt = lds_address(PAR ? v_s0 : v_s1);   // V(t - 1): consumed, refilled with V(t + 1)
-        PHASE_FENCE();
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this wavefront's loads of K(t + 1), V(t) have landed in LDS
-        PHASE_FENCE();
-        __syncthreads();                                         // X(t)
-        // While scores of a further tile are due (then L > KT), this wavefront's 16 loads of K(t + 2) and V(t + 1) are spread
-        // over the steps below: a burst would stall on the memory pipeline's queue.  There a tile index past the end loads the
-        // last tile again, harmlessly: nothing reads that buffer any more.
-        const bool more = t + 1 < tw;                            // wavefront-uniform
-        const int tk = min(t + 2, tb - 1), tv = min(t + 1, tb - 1);
-        if (!more) {
-            if (t + 2 < tb) load_rows(kg, k_cur, t + 2);
-            if (t + 1 < tb) load_rows(vg, v_nxt, t + 1);
-        }
-        PHASE_FENCE();
-        if (t >= tw) return;                               // wavefront-uniform: the upper row block may see one tile more
-        // only tiles that touch the diagonal or the end of the sequence need the mask (wavefront-uniform)
-        if (t * KT + KT - 1 > q_pos0 + r0 || t * KT + KT > L) {
-#pragma unroll
-            for (int hh = 0; hh < NH; hh++)
-#pragma unroll
-                for (int kt = 0; kt < 4; kt++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int key = tile_row0(t) + 16 * kt + 4 * g + i;     // a shifted tile repeats keys below t * KT
-                        if (!(key >= t * KT && key <= my_last && key < L)) acc[hh][kt][i] = NEG;
-                    }
-        }
-        const bf16_t* ka = k_nxt + ka_row;
-        const bf16_t* va = v_cur + va_row;
-        auto v_frag = [&](int j, int q4) {
-            return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) s16x4*)(const_cast<bf16_t*>(va + (16 * q4) * AD + (((2 * (j & 7) + vc0) ^ vrow) << 3) +
-                                                                             128 * (j >> 3))));   // the swizzle (< 16) leaves bit 4 alone
-        };
-        s16x8 P[NH][2];
-        s16x4 Bf[3][4];
-        float mx[NH];
-        auto body = [&](auto with_scores) {
-            constexpr bool SC = decltype(with_scores)::value;
-            // K fragments: a ring, each read FRAG_AHEAD steps before the MFMAs that consume it (fragment f = 8 kt + kb)
-            bf16x8 Af[FRAG_AHEAD + 1];
-            if (SC) {
-#pragma unroll
-                for (int f = 0; f < FRAG_AHEAD; f++) Af[f] = k_frag(ka, f >> 3, f & 7);
-            }
-            // The exponentials are taken against the running reference point of each row at once, on the bet that no row's
-            // maximum grows by more than 2^LAZY in this tile (true for all but the first few tiles of a row block); the
-            // maxima are folded in beside them and the bet is checked after the steps (`grow` below).
-#pragma unroll
-            for (int hh = 0; hh < NH; hh++) mx[hh] = NEG;
-            PHASE_FENCE();
-            const unsigned step_off0 = SC ? opaque_off0() : 0u;
-            // 32 steps: two score MFMAs of tile t + 1 (one K fragment x both heads) and one softmax element of tile t
-            float pv_prev = 0.f;
-#pragma unroll
-            for (int st = 0; st < 32; st++) {
-                const int kt = st >> 3, kb = st & 7;
-                __builtin_amdgcn_sched_barrier(0);
-                if (SC && (st & 7) == 0) {
-                    if (st < 16)
-                        load_four(kg, k_cur, tk, st >> 3, step_off0);
-                    else
-                        load_four(vg, v_nxt, tv, (st >> 3) - 2, step_off0);
-                }
-                if (SC) {
-                    if (st + FRAG_AHEAD < 32)
-                        Af[(st + FRAG_AHEAD) % (FRAG_AHEAD + 1)] = k_frag(ka, (st + FRAG_AHEAD) >> 3, (st + FRAG_AHEAD) & 7);
-                    if (st >= 30) {                              // the first V fragments of P.V ride along with the last steps
-#pragma unroll
-                        for (int q4 = 0; q4 < 4; q4++) Bf[st - 30][q4] = v_frag(st - 30, q4);
-                    }
-#pragma unroll
-                    for (int hh = 0; hh < NH; hh++)
-                        acc_next[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            Af[st % (FRAG_AHEAD + 1)], bq[hh][kb], kb == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc_next[hh][kt], 0, 0, 0);
-                }
-                // softmax elements: NH * 16 of them over the 32 steps
-#pragma unroll
-                for (int e = (NH * 16 * st) / 32; e < (NH * 16 * (st + 1)) / 32; e++) {
-                    const int hh = e >> 4, kt2 = (e >> 2) & 3, i = e & 3;
-                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_run[hh]));
-                    mx[hh] = fmaxf(mx[hh], acc[hh][kt2][i]);
-                    if (i & 1) {
-                        const uint32_t pk = pack_bf(pv_prev, pv);
-                        P[hh][kt2 >> 1][(kt2 & 1) * 4 + i - 1] = (short)(pk & 0xffff);
-                        P[hh][kt2 >> 1][(kt2 & 1) * 4 + i] = (short)(pk >> 16);
-                    }
-                    pv_prev = pv;
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (!SC) {
-#pragma unroll
-                for (int q4 = 0; q4 < 4; q4++) {
-                    Bf[0][q4] = v_frag(0, q4);
-                    Bf[1][q4] = v_frag(1, q4);
-                }
-            }
-        };
-        if (more)
-            body(std::true_type{});
-        else
-            body(std::false_type{});
-        PHASE_FENCE();
-        // the reference point of a row only moves when its maximum has grown by more than 2^LAZY: until then p stays below
-        // 2^LAZY, which bf16 and the f32 sums hold as well as values below 1, and the accumulators are left alone
-        bool grow = false;
-#pragma unroll
-        for (int hh = 0; hh < NH; hh++) {
-            mx[hh] = max_over_groups(mx[hh]) * SCALE_LOG2E;
-            grow |= mx[hh] > m_run[hh] + LAZY;
-        }
-        if (__any(grow)) {                                       // wavefront-uniform and rare: the bet was lost for some row
-#pragma unroll
-            for (int hh = 0; hh < NH; hh++) {
-                const float m_new = mx[hh] > m_run[hh] + LAZY ? mx[hh] : m_run[hh];
-                const float corr = __builtin_amdgcn_exp2f(m_run[hh] - m_new);   // m_run = NEG initially: 2^-huge = 0
-                m_run[hh] = m_new;
-                c_s[w][hh][n] = corr;                            // all four groups store the same value: no divergent branch
-                // this tile's p again, against the new reference points (rows that did not move get the same bits)
-#pragma unroll
-                for (int kt2 = 0; kt2 < 4; kt2++)
-#pragma unroll
-                    for (int i = 0; i < 4; i += 2) {
-                        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i], SCALE_LOG2E, -m_new));
-                        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(acc[hh][kt2][i + 1], SCALE_LOG2E, -m_new));
-                        const uint32_t pk = pack_bf(p0, p1);
-                        P[hh][kt2 >> 1][(kt2 & 1) * 4 + i] = (short)(pk & 0xffff);
-                        P[hh][kt2 >> 1][(kt2 & 1) * 4 + i + 1] = (short)(pk >> 16);
-                        __builtin_amdgcn_sched_barrier(0);       // pair by pair: scheduled freely, the 32 values take registers
-                    }
-            }
-            wave_lds_sync();
-#pragma unroll
-            for (int hh = 0; hh < NH; hh++) {
-                const f32x4 c4 = *reinterpret_cast<const f32x4*>(&c_s[w][hh][4 * g]);
-#pragma unroll
-                for (int j = 0; j < 16; j++) {
-                    PIN_ACC(O[hh][j]);
-                    O[hh][j] *= c4;
-                    PIN_ACC(O[hh][j]);                           // and back at once: 128 products would not fit beside the rest
-                }
-                PIN_ACC(Lsum[hh]);
-                Lsum[hh] *= c4;
-                PIN_ACC(Lsum[hh]);
-            }
-            wave_lds_sync();                                     // c_s is rewritten by the next tile that moves a reference
-        }
-        PHASE_FENCE();
-        // P . V: the four transposed V fragments of a 16-column block are read two blocks ahead of their MFMAs and serve
-        // both heads; the row sums are one more column block, P . 1 (the sum of exactly the rounded values that multiply V)
-        {
-            s16x8 ones;
-#pragma unroll
-            for (int e = 0; e < 8; e++) ones[e] = (short)0x3f80;
-#pragma unroll
-            for (int pp = 0; pp < 2; pp++)
-#pragma unroll
-                for (int hh = 0; hh < NH; hh++)
-                    Lsum[hh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[hh][pp]),
-                                                                      __builtin_bit_cast(bf16x8, ones), Lsum[hh], 0, 0, 0);
-        }
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            __builtin_amdgcn_sched_barrier(0);
-            if (j + 2 < 16) {
-#pragma unroll
-                for (int q4 = 0; q4 < 4; q4++) Bf[(j + 2) % 3][q4] = v_frag(j + 2, q4);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int pp = 0; pp < 2; pp++) {
-                const s16x8 B = __builtin_shufflevector(Bf[j % 3][2 * pp], Bf[j % 3][2 * pp + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-                for (int hh = 0; hh < NH; hh++)
-                    O[hh][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[hh][pp]),
-                                                                      __builtin_bit_cast(bf16x8, B), O[hh][j], 0, 0, 0);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        PHASE_FENCE();
-    };
-
-    if (ta < tb) {                                               // (a part past the block's last tile is empty)
-        load_rows(kg, lds_address(k_s0), ta);
-        load_rows(vg, lds_address(v_s0), ta);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (tb - ta > 1) load_rows(kg, lds_address(k_s1), ta + 1);
-        if (tw > ta) scores_first(k_s0 + ka_row, accs[0]);
-        for (int t = ta; t < tb; t += 2) {
-            tile(t, std::integral_constant<int, 0>{});
-            if (t + 1 < tb) tile(t + 1, std::integral_constant<int, 1>{});
-        }
-    }
-    // The lane's coordinates for the epilogue are taken again here, from the lane number the hardware counts: kept from the
-    // prologue they would live through the tile loop, in two registers more than the wavefront has (the kernel then spills
-    // them to scratch memory; measured, that cost nothing below 4096 rows and 2 % there).
-    int zero = 0;
-    asm volatile("" : "+v"(zero));                               // (keeps the count below the loop)
-    const int lane_e = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));
-    const int n_e = lane_e & 15, g_e = lane_e >> 4, my_last_e = q_pos0 + r0 + n_e;
-    if (nparts > 1) {
-        // One part of several: leave O, m, l of this wavefront's heads as they are.  A row that sees no key of this part (its
-        // last key lies before the part's first) has exponentiated masked scores against a masked maximum: it is written as
-        // the neutral element (m = NEG, l = 0, O = 0).
-        const int first_key = ta * KT, lr0 = r0 - rb * RB;       // this wavefront's first row within the block
-#pragma unroll
-        for (int hh = 0; hh < NH; hh++) {
-            const int hq = w + hh;                               // head within the KV group
-            _Float16* po = part_o + (slot * 4 + hq) * (RB * AD);
-            float* pml = part_ml + (slot * 4 + hq) * (2 * RB);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int lr = lr0 + 4 * g_e + r;
-                const bool seen = q_pos0 + rb * RB + lr >= first_key;
-                const float inv = seen ? 1.0f / Lsum[hh][r] : 0.f;
-#pragma unroll
-                for (int j = 0; j < 16; j++) po[lr * AD + 16 * j + n_e] = (_Float16)(seen ? O[hh][j][r] * inv : 0.f);
-                if (n_e == 0) pml[RB + lr] = seen ? Lsum[hh][r] : 0.f;
-            }
-            if (g_e == 0) pml[lr0 + n_e] = my_last_e >= first_key ? m_run[hh] : NEG;
-        }
-        return;
-    }
-    // ---- normalise and store: lane (n_e, g_e) holds rows 4g .. 4g+3 of column 16 j + n_e, and of the row sums (any column)
-#pragma unroll
-    for (int hh = 0; hh < NH; hh++) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int orow = r0 + 4 * g_e + r;
-            if (orow < S) {
-                const float inv = 1.0f / Lsum[hh][r];
-                bf16_t* dst = out + (size_t)(h0 + hh) * q_head_stride + (size_t)orow * AD + n_e;
-#pragma unroll
-                for (int j = 0; j < 16; j++) dst[16 * j] = f2bf(O[hh][j][r] * inv);
-            }
-        }
-    }
-}
-
-// a word of LDS as a volatile object in the LDS address space (through a generic pointer, a volatile access is a flat
-// instruction, which is also counted, and waited for, as an access of global memory)
-__device__ __forceinline__ volatile __attribute__((address_space(3))) int* lds_word(int* shared_word) {
-    return (volatile __attribute__((address_space(3))) int*)shared_word;
-}
-
-// The tile loop with the two halves of a tile's work on different wavefronts.  A workgroup is 32 query rows x 4 heads on
-// eight wavefronts, two per SIMD: wavefront pr (0 .. 3, the "score" wavefront of pair pr) computes the scores and the softmax
-// of rows 16 (pr >> 1) .. + 16 for heads 2 (pr & 1), + 1, and wavefront 4 + pr (the pair's "output" wavefront) multiplies the
-// resulting P by V, one tile behind.  A wavefront's instructions issue one after the other (an MFMA holds its wavefront for
-// about as long as it holds the matrix unit, and every LDS read, exponential or wait comes on top), while two wavefronts
-// of a SIMD do overlap: one feeds the unit Q K^T while the other reads V fragments, and the softmax arithmetic of the one
-// runs beside the P V MFMAs of the other.  (All of it on one wavefront per SIMD, with these 32 rows x 4 heads, measures
-// 5 - 7 % slower; the compiler's order within the score wavefront, the softmax arithmetic as one block and then the MFMA
-// steps back to back, measures better than the same arithmetic tied into the steps.)  With eight wavefronts the 512 registers
-// of a SIMD lane are split in two, 256 per wavefront and no separate accumulation half: the score side holds Q^T (64
-// registers) and two tiles of scores (64), the output side O (128).
-//     iteration t (after barrier X(t): K(t + 1) and V(t - 1) are in LDS):
-//         score wavefront:  softmax of tile t (its scores are in registers since iteration t - 1) and the score MFMAs of
-//                           tile t + 1; then P(t), as packed A operands, and the rows' rescale factors go to LDS
-//         output wavefront: takes P(t - 1) and the factors from LDS, rescales O and the row sums if any row's reference
-//                           moved, O += P(t - 1) V(t - 1)
-//         all eight:        direct-to-LDS loads of K(t + 2) into K(t)'s buffer and of V(t) into V(t - 2)'s
-// P has one buffer per pair: the output wavefront reads it into registers first thing in an iteration and says so
-// (taken_s[pr] = t), and the score wavefront, which writes the next P a few thousand clocks later, looks at that word first.
-// The loader here has no path for fewer than 64 keys: the host picks this kernel from about 1500 query rows on.
-__global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ K,
-                                                              const bf16_t* __restrict__ V, bf16_t* __restrict__ out, int S, int L,
-                                                              int q_pos0, long q_head_stride, long kv_head_stride, int tmax,
-                                                              _Float16* __restrict__ part_o, float* __restrict__ part_ml) {
-    __shared__ __align__(1024) bf16_t kv_s[4 * TILE];            // K tiles of even / odd iterations, then the V tiles
-    __shared__ __align__(16) u32x4 p_s[4][2][2][64];             // [pair][head][32-key half][lane]: P as the lanes hold it
-    __shared__ __align__(16) float c_s[4][2][16];                // [pair][head][row]: factor of a row whose reference moved
-    __shared__ float m_s[4][2][16];                              // final reference points (only the parts' epilogue needs them)
-    __shared__ int moved_s[4];                                   // pair: did any reference move in the tile whose P lies in p_s
-    __shared__ int taken_s[4];                                   // pair: the iteration in which p_s / c_s / moved_s were last read
-    constexpr int RB = 32;
-    const int nitems = gridDim.x / AKV, item = blockIdx.x / AKV;
-    int rb = nitems - 1 - item;                                  // long rows first
-    int part = 0, nparts = 1;
-    if (tmax > 0) {                                              // items are parts (see attn_prefill_kernel)
-        const int c = (KT / RB) * tmax, p = (q_pos0 + RB - 1) / RB;
-        const long y = (long)rb + parts_upto(p, c);
-        int k = 0;
-        while ((long)c * ((k + 1) * (k + 2) / 2) <= y) k++;
-        const int nn = k * c + (int)((y - (long)c * (k * (k + 1) / 2)) / (k + 1));
-        part = (int)(y - parts_upto(nn, c));
-        nparts = k + 1;
-        rb = nn - p;
-    }
-    const int kvh = blockIdx.x % AKV;
-    const size_t slot = (size_t)kvh * nitems + (nitems - 1 - item);
-    const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n = lane & 15, g = lane >> 4;
-    const int pr = w & 3;                                        // pair; w >> 2: 0 = score, 1 = output wavefront
-    const int h0 = kvh * (AH / AKV) + 2 * (pr & 1);
-    const int r0 = rb * RB + 16 * (pr >> 1), row = r0 + n;
-    const bool row_ok = row < S;
-    const int my_last = q_pos0 + row;
-    const int kend = min(L, q_pos0 + min(rb * RB + RB - 1, S - 1) + 1);
-    const int ntiles = (kend + KT - 1) / KT;
-    const int kend_w = r0 < S ? min(L, q_pos0 + min(r0 + 15, S - 1) + 1) : 0;
-    const int ntiles_w = (kend_w + KT - 1) / KT;
+    // this workgroup's tiles [ta, tb); tw: where this pair's rows end (the upper rows of a block may see one tile more)
     const int ta = part * tmax, tb = tmax > 0 ? min(ntiles, ta + tmax) : ntiles;
     const int tw = min(ntiles_w, tb);
 
     // tile loader: wavefront w issues four direct-to-LDS loads of K and four of V per tile; load i fills rows 8 w + 2 i, + 1
-    // (one KiB): lane l lands at chunk l & 31 of row 8 w + 2 i + (l >> 5) and fetches chunk (l & 31) ^ (row & 15).  L >= KT here.
+    // (one KiB): lane l lands at chunk position l & 31 of row 8 w + 2 i + (l >> 5) and fetches chunk (l & 31) ^ (row & 15).  The
+    // per-lane byte offsets within a tile do not change from tile to tile: load i differs from load 0 by 2 i rows, which go into
+    // the instruction's immediate offset (it moves the global address and the LDS destination alike), and by an XOR of the
+    // chunk with 2 i.  A tile that would run past the end of the sequence is shifted back to end at L (tile_row0): its first
+    // rows repeat keys of the tile before and are masked.  Only a sequence shorter than one tile repeats its last key instead.
     const char* kg = reinterpret_cast<const char*>(K + (size_t)kvh * kv_head_stride);
     const char* vg = reinterpret_cast<const char*>(V + (size_t)kvh * kv_head_stride);
     const unsigned ld_row0 = 8u * w + (lane >> 5);
     const unsigned ld_off0 = ld_row0 * (AD * 2) + ((unsigned)((lane & 31) ^ (ld_row0 & 15u)) << 4);
     auto tile_row0 = [&](int t) { return max(0, min(t * KT, L - KT)); };
+    // a copy of ld_off0 the compiler cannot see through: the offsets of the four loads are then recomputed where they are
+    // used (one XOR each) instead of living in registers through the loop
     auto opaque_off0 = [&]() {
         unsigned off0 = ld_off0;
         asm volatile("" : "+v"(off0));
@@ -601,18 +196,31 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
     };
     const unsigned w_lds = 4096u * w;                            // this wavefront's 4 KiB of a tile buffer
     auto load_four = [&](const char* src, unsigned dst, int t, unsigned off0) {
-        const char* base = src + (size_t)tile_row0(t) * (AD * 2);
-        lds_dma16x4(base, off0, off0 ^ 32u, off0 ^ 64u, off0 ^ 96u, dst + w_lds);
+        if (L >= KT) {
+            const char* base = src + (size_t)tile_row0(t) * (AD * 2);
+            lds_dma16x4(base, off0, off0 ^ 32u, off0 ^ 64u, off0 ^ 96u, dst + w_lds);
+        } else {                                                 // t = 0: rows past the end repeat the last key; they are masked
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const unsigned o = (ld_off0 ^ (32u * i)) + 1024u * i;
+                lds_dma16<0>(src, (unsigned)min((int)(o >> 9), L - 1) * (AD * 2) + (o & 511u), dst + w_lds + 1024u * i);
+            }
+        }
     };
+    // A operand of the scores: row 16 kt + n of the tile, chunk (4 kb + g) ^ n
     const int ka_row = n * AD;
-    const int vrow = 4 * g + (n >> 2);
+    // transposing load: within 16 lanes, lane 4q + i receives element i of the 8-byte chunks addressed by lanes q, q+4,
+    // q+8, q+12; lane n of group g points at key 4g + n/4, columns 4 (n%4).. of the block and receives keys 4g..4g+3 of column n
+    const int vrow = 4 * g + (n >> 2);                           // row within a 16-key block = its swizzle
     const int va_row = vrow * AD + 4 * (n & 1), vc0 = (n & 3) >> 1;
+    // K fragment kb of sub-tile kt: chunk (4 kb + g) ^ n; n < 16 leaves bit 4 alone, so fragments kb and kb + 4 share an
+    // address register
     auto k_frag = [&](const bf16_t* ka, int kt, int kb) {
         return *reinterpret_cast<const bf16x8*>(ka + 16 * kt * AD + (((4 * (kb & 3) + g) ^ n) << 3) + 128 * (kb >> 2));
     };
 
     if (tid < 4) taken_s[tid] = -1, moved_s[tid] = 0;
-    if (tid < 128) (&m_s[0][0][0])[tid] = NEG;
+    if (tid < 4 * NH * 16) (&m_s[0][0][0])[tid] = NEG;
     if (ta < tb) {                                               // (a part past the block's last tile is empty)
         load_four(kg, lds_address(kv_s), ta, ld_off0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -623,9 +231,9 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
     if (w < 4) {
         // ------------------------------------------------------------------------------------------ score wavefront
         if (ta >= tb) return;
-        bf16x8 bq[2][8];
+        bf16x8 bq[NH][8];
 #pragma unroll
-        for (int hh = 0; hh < 2; hh++) {
+        for (int hh = 0; hh < NH; hh++) {
             const u32x4* qr = reinterpret_cast<const u32x4*>(q + (size_t)(h0 + hh) * q_head_stride + (size_t)(row_ok ? row : 0) * AD);
 #pragma unroll
             for (int kb = 0; kb < 8; kb++) {
@@ -634,8 +242,10 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
                 bq[hh][kb] = __builtin_bit_cast(bf16x8, v);
             }
         }
-        float m_run[2] = {NEG, NEG};
-        auto first_scores = [&](f32x4 (&acc0)[2][4]) {
+        float m_run[NH];
+#pragma unroll
+        for (int hh = 0; hh < NH; hh++) m_run[hh] = NEG;
+        auto first_scores = [&](f32x4 (&acc0)[NH][4]) {
             const bf16_t* ka = kv_s + ka_row;
             bf16x8 Af[2][8];
 #pragma unroll
@@ -649,16 +259,16 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++) acc0[hh][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                for (int hh = 0; hh < NH; hh++) acc0[hh][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kb = 0; kb < 8; kb++)
 #pragma unroll
-                    for (int hh = 0; hh < 2; hh++)
+                    for (int hh = 0; hh < NH; hh++)
                         acc0[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Af[kt & 1][kb], bq[hh][kb], acc0[hh][kt], 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         };
-        f32x4 acc[2][4] = {};                                    // scores of tile t
+        f32x4 acc[NH][4] = {};                                   // scores of tile t
         if (tw > ta) first_scores(acc);
         for (int t = ta; t <= tb; t++) {
             const unsigned par = (unsigned)(t - ta) & 1u;
@@ -679,34 +289,40 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
             }
             PHASE_FENCE();
             if (t >= tw) continue;
+            // only tiles that touch the diagonal or the end of the sequence need the mask (wavefront-uniform)
             if (t * KT + KT - 1 > q_pos0 + r0 || t * KT + KT > L) {
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++)
+                for (int hh = 0; hh < NH; hh++)
 #pragma unroll
                     for (int kt = 0; kt < 4; kt++)
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
-                            const int key = tile_row0(t) + 16 * kt + 4 * g + i;
+                            const int key = tile_row0(t) + 16 * kt + 4 * g + i;     // a shifted tile repeats keys below t * KT
                             if (!(key >= t * KT && key <= my_last && key < L)) acc[hh][kt][i] = NEG;
                         }
             }
             const bf16_t* ka = k_nxt + ka_row;
-            f32x4 acc_next[2][4];
-            // Tile t's softmax rides on the 32 score steps of tile t + 1.  The exponentials are taken against the running
-            // reference points on the bet that no row's maximum grows by more than 2^LAZY in this tile; the maxima are folded
-            // in beside them and the bet is checked in `publish`.
-            auto publish = [&](s16x8 (&P)[2][2], float (&mx)[2], int taken_early) {
+            f32x4 acc_next[NH][4];
+            // Online softmax in base 2 on the raw products: p = 2^(c s - m), c = 256^-0.5 log2 e; every row sees key 0, so its
+            // maximum is finite from the first tile on and masked entries come out as 2^-huge = 0.  The exponentials are taken
+            // against the running reference point of each row at once, on the bet that no row's maximum grows by more than
+            // 2^LAZY in this tile (true for all but the first few tiles of a row block); the maxima are folded in beside them
+            // and the bet is checked here.  A reference point only moves when the row's maximum has grown by more than 2^LAZY:
+            // until then p stays below 2^LAZY, which bf16 and the f32 sums hold as well as values below 1.
+            auto publish = [&](s16x8 (&P)[NH][2], float (&mx)[NH], int taken_early) {
                 bool grow = false;
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++) {
+                for (int hh = 0; hh < NH; hh++) {
                     mx[hh] = max_over_groups(mx[hh]) * SCALE_LOG2E;
                     grow |= mx[hh] > m_run[hh] + LAZY;
                 }
                 const bool any_grow = __any(grow);
-                float corr[2] = {1.f, 1.f};
+                float corr[NH];
+#pragma unroll
+                for (int hh = 0; hh < NH; hh++) corr[hh] = 1.f;
                 if (any_grow) {                                      // wavefront-uniform and rare
 #pragma unroll
-                    for (int hh = 0; hh < 2; hh++) {
+                    for (int hh = 0; hh < NH; hh++) {
                         const float m_new = mx[hh] > m_run[hh] + LAZY ? mx[hh] : m_run[hh];
                         corr[hh] = __builtin_amdgcn_exp2f(m_run[hh] - m_new);    // m_run = NEG initially: 2^-huge = 0
                         m_run[hh] = m_new;
@@ -734,23 +350,25 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
                 }
                 asm volatile("" ::: "memory");
                 if (any_grow) {
-                    c_s[pr][0][n] = corr[0];                         // all four groups store the same value
-                    c_s[pr][1][n] = corr[1];
+#pragma unroll
+                    for (int hh = 0; hh < NH; hh++) c_s[pr][hh][n] = corr[hh];    // all four groups store the same value
                 }
                 moved_s[pr] = any_grow ? 1 : 0;
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++)
+                for (int hh = 0; hh < NH; hh++)
 #pragma unroll
                     for (int pp = 0; pp < 2; pp++) p_s[pr][hh][pp][lane] = __builtin_bit_cast(u32x4, P[hh][pp]);
                 if (t == tw - 1) {
-                    m_s[pr][0][n] = m_run[0];
-                    m_s[pr][1][n] = m_run[1];
+#pragma unroll
+                    for (int hh = 0; hh < NH; hh++) m_s[pr][hh][n] = m_run[hh];
                 }
             };
             auto body = [&](auto with_scores) {
                 constexpr bool SC = decltype(with_scores)::value;
-                s16x8 P[2][2];
-                float mx[2] = {NEG, NEG};
+                s16x8 P[NH][2];
+                float mx[NH];
+#pragma unroll
+                for (int hh = 0; hh < NH; hh++) mx[hh] = NEG;
                 bf16x8 Af[FRAG_AHEAD + 1];
                 if (SC) {
 #pragma unroll
@@ -779,11 +397,11 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
                         if (st + FRAG_AHEAD < 32)
                             Af[(st + FRAG_AHEAD) % (FRAG_AHEAD + 1)] = k_frag(ka, (st + FRAG_AHEAD) >> 3, (st + FRAG_AHEAD) & 7);
 #pragma unroll
-                        for (int hh = 0; hh < 2; hh++)
+                        for (int hh = 0; hh < NH; hh++)
                             acc_next[hh][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                                 Af[st % (FRAG_AHEAD + 1)], bq[hh][kb], kb == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc_next[hh][kt], 0, 0, 0);
                     }
-                    if ((st & 1) == 0) softmax_pair(st >> 1);
+                    if (st % (4 / NH) == 0) softmax_pair(st / (4 / NH));       // 8 NH pairs over the 32 steps
                     if (st == 20) taken_early = *lds_word(&taken_s[pr]);   // (read early: its LDS latency passes under the steps)
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -796,7 +414,7 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
             PHASE_FENCE();
             if (more) {
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++)
+                for (int hh = 0; hh < NH; hh++)
 #pragma unroll
                     for (int kt = 0; kt < 4; kt++) acc[hh][kt] = acc_next[hh][kt];
             }
@@ -805,10 +423,10 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
         return;
     }
     // ---------------------------------------------------------------------------------------------- output wavefront
-    f32x4 O[2][16];
-    f32x4 Lsum[2];                                                   // row sums of P, accumulated by MFMA against a block of ones
+    f32x4 O[NH][16];
+    f32x4 Lsum[NH];                                                  // row sums of P, accumulated by MFMA against a block of ones
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
+    for (int hh = 0; hh < NH; hh++) {
         Lsum[hh] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 16; j++) O[hh][j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -834,16 +452,14 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
         PHASE_FENCE();
         __syncthreads();                                             // X(t)
         const int mv = __builtin_amdgcn_readfirstlane(moved_s[pr]);
-        s16x8 P[2][2];
+        s16x8 P[NH][2];
 #pragma unroll
-        for (int hh = 0; hh < 2; hh++)
+        for (int hh = 0; hh < NH; hh++)
 #pragma unroll
             for (int pp = 0; pp < 2; pp++) P[hh][pp] = __builtin_bit_cast(s16x8, p_s[pr][hh][pp][lane]);
-        f32x4 c4[2] = {f32x4{1.f, 1.f, 1.f, 1.f}, f32x4{1.f, 1.f, 1.f, 1.f}};
-        if (mv) {
-            c4[0] = *reinterpret_cast<const f32x4*>(&c_s[pr][0][4 * g]);
-            c4[1] = *reinterpret_cast<const f32x4*>(&c_s[pr][1][4 * g]);
-        }
+        f32x4 c4[NH];
+#pragma unroll
+        for (int hh = 0; hh < NH; hh++) c4[hh] = mv ? *reinterpret_cast<const f32x4*>(&c_s[pr][hh][4 * g]) : f32x4{1.f, 1.f, 1.f, 1.f};
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         *lds_word(&taken_s[pr]) = t;
         asm volatile("" ::: "memory");
@@ -860,7 +476,7 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
             for (int q4 = 0; q4 < 4; q4++) Bf[j][q4] = v_frag(j, q4);
         if (mv) {                                                    // a reference moved: rescale what is accumulated
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++) {
+            for (int hh = 0; hh < NH; hh++) {
 #pragma unroll
                 for (int j = 0; j < 16; j++) O[hh][j] *= c4[hh];
                 Lsum[hh] *= c4[hh];
@@ -874,7 +490,7 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
 #pragma unroll
             for (int pp = 0; pp < 2; pp++)
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++)
+                for (int hh = 0; hh < NH; hh++)
                     Lsum[hh] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[hh][pp]),
                                                                       __builtin_bit_cast(bf16x8, ones), Lsum[hh], 0, 0, 0);
         }
@@ -893,7 +509,7 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
             for (int pp = 0; pp < 2; pp++) {
                 const s16x8 B = __builtin_shufflevector(Bf[j % (V_FRAG_AHEAD + 1)][2 * pp], Bf[j % (V_FRAG_AHEAD + 1)][2 * pp + 1], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
-                for (int hh = 0; hh < 2; hh++)
+                for (int hh = 0; hh < NH; hh++)
                     O[hh][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, P[hh][pp]),
                                                                       __builtin_bit_cast(bf16x8, B), O[hh][j], 0, 0, 0);
             }
@@ -903,13 +519,15 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
     }
     if (ta < tb)
         for (int t = max(tw, ta) + 1; t <= tb; t++) idle_iter(t);
+    // ---- normalise and store: lane (n, g) holds rows 4g .. 4g+3 of column 16 j + n, and of the row sums (any column)
     if (nparts > 1) {
-        // one part of several (see attn_prefill_kernel): O / l, m, l of this pair's heads; rows that see no key of the part
-        // are written as the neutral element
+        // One part of several: leave O / l, m, l of this pair's heads as they are.  A row that sees no key of this part (its
+        // last key lies before the part's first) has exponentiated masked scores against a masked maximum: it is written as
+        // the neutral element (m = NEG, l = 0, O = 0).
         const int first_key = ta * KT, lr0 = r0 - rb * RB;
 #pragma unroll
-        for (int hh = 0; hh < 2; hh++) {
-            const int hq = 2 * (pr & 1) + hh;
+        for (int hh = 0; hh < NH; hh++) {
+            const int hq = hq0 + hh;
             _Float16* po = part_o + (slot * 4 + hq) * (RB * AD);
             float* pml = part_ml + (slot * 4 + hq) * (2 * RB);
 #pragma unroll
@@ -926,7 +544,7 @@ __global__ __launch_bounds__(512) void attn_prefill_ws_kernel(const bf16_t* __re
         return;
     }
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
+    for (int hh = 0; hh < NH; hh++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int orow = r0 + 4 * g + r;
@@ -1097,10 +715,10 @@ int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out
     _Float16* part_o = ks.tmax ? (_Float16*)workspace : nullptr;
     float* part_ml = ks.tmax ? reinterpret_cast<float*>(part_o + (size_t)ks.parts * AKV * part_o_floats(RB)) : nullptr;
     if (ks.nh == 2)
-        hipLaunchKernelGGL(attn_prefill_ws_kernel, grid, dim3(512), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
+        hipLaunchKernelGGL(attn_prefill_kernel<2>, grid, dim3(512), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
                            (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
     else
-        hipLaunchKernelGGL(attn_prefill_kernel, grid, dim3(256), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
+        hipLaunchKernelGGL(attn_prefill_kernel<1>, grid, dim3(512), 0, stream, (const bf16_t*)q, (const bf16_t*)K, (const bf16_t*)V,
                            (bf16_t*)out, S, L, q_pos0, q_head_stride, kv_head_stride, ks.tmax, part_o, part_ml);
     if (ks.tmax) {
         const dim3 mgrid((unsigned)ks.split_blocks, AKV, (AH / AKV) * ks.nh);

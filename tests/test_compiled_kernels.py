@@ -175,7 +175,7 @@ def test_no_kernel_spills_or_reaches_a_barrier_with_an_unwaited_lds_store(tmp_pa
         with open(out) as f:
             asm = f.read()
         if os.path.basename(src) == "gqa_prefill.hip":
-            for kernel in ("attn_prefill_kernel", "attn_prefill_ws_kernel"):
+            for kernel in ("attn_prefill_kernelILi1E", "attn_prefill_kernelILi2E"):
                 assert partial_lds_waits(asm, kernel) >= 50, f"{kernel}: the tile loop waits for every LDS read in full"
         return os.path.basename(src), asm.count("s_barrier"), unwaited_barriers(asm), scratch_users(asm)
 
