@@ -231,6 +231,7 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
     if (w < 4) {
         // ------------------------------------------------------------------------------------------ score wavefront
         if (ta >= tb) return;
+        // Q^T as the B operand of the score MFMA: lane (row n, group g) holds q[row][32 kb + 8 g .. + 8] of each head
         bf16x8 bq[NH][8];
 #pragma unroll
         for (int hh = 0; hh < NH; hh++) {
@@ -245,6 +246,8 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
         float m_run[NH];
 #pragma unroll
         for (int hh = 0; hh < NH; hh++) m_run[hh] = NEG;
+        // scores of the first tile, S^T = K_tile . Q^T: each K fragment multiplies the Q^T of every head of the pair; the fragments
+        // of the next 16-key sub-tile are read while the MFMAs of the current one run
         auto first_scores = [&](f32x4 (&acc0)[NH][4]) {
             const bf16_t* ka = kv_s + ka_row;
             bf16x8 Af[2][8];
@@ -281,7 +284,10 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             PHASE_FENCE();
             __syncthreads();                                         // X(t)
-            const bool more = t + 1 < tw;
+            // While scores of a further tile are due (then L > KT), this wavefront's loads of K(t + 2) and V(t) ride on the steps
+            // below: a burst would stall on the memory pipeline's queue.  There a tile index past the end loads the last tile
+            // again, harmlessly: nothing reads that buffer any more.
+            const bool more = t + 1 < tw;                            // wavefront-uniform
             const int tk = min(t + 2, tb - 1);
             if (!more) {
                 if (t + 2 < tb) load_four(kg, k_cur, t + 2, opaque_off0());
@@ -387,6 +393,9 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
                 PHASE_FENCE();
                 const unsigned step_off0 = SC ? opaque_off0() : 0u;
                 int taken_early = -1;
+                // 32 steps: one K fragment read (FRAG_AHEAD steps ahead, a ring) and its MFMAs, one per head.  The softmax
+                // pairs are written beside them, but nothing ties them to their step: the compiler gathers the arithmetic
+                // into one block beside the steps, which measures better than the same arithmetic held between the MFMAs.
 #pragma unroll
                 for (int st = 0; st < 32; st++) {
                     const int kt = st >> 3, kb = st & 7;
