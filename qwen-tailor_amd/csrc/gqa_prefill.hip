@@ -625,7 +625,7 @@ inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 288; }   /
 // The key split of a launch: tmax = 0 (none) or the tiles per part, parts = grid width, split_blocks = blocks with several parts.
 // Only launches that leave CUs without a workgroup are split (fewer than 2048 query rows: a short continuation of a long
 // prefix, a short prompt), and only as far as the idle CUs go: a part holds the smallest number of tiles (from the launch's
-// average per CU, at least 8) with which all parts are resident at once, and the split must shorten the longest workgroup
+// average per CU, at least 6) with which all parts are resident at once, and the split must shorten the longest workgroup
 // by six tiles or more to pay for the merge launch.  A workgroup costs
 // about 6 us beyond its tiles (dispatch, Q and first-tile latency, the output stores): measured at S = 2048 (256 workgroups,
 // 57 us unsplit) every part size from 4 to 32 tiles came out between 53 and 61 us before the parts were even merged.
@@ -648,10 +648,11 @@ KeySplit plan_split_nh(int S, int L, int q_pos0, int nh, int min_gain) {
         total += nt;
         longest = std::max(longest, nt);
     }
-    // the smallest part size (from the average per CU, at least 8 tiles) whose parts are all resident at once: a CU that has
-    // to run a second part pays the per-workgroup cost twice
+    // the smallest part size (from the average per CU, at least 6 tiles) whose parts are all resident at once: a CU that has
+    // to run a second part pays the per-workgroup cost twice.  (A floor of 6 against 8, us: 768 rows 18.1 / 20.7, 1536 rows
+    // 28.9 / 29.9, one row after 4095 keys 19.6 / 21.1, 64 rows after 8000 keys 29.4 / 27.6; 5 and 7 are worse on more shapes.)
     const long p = (q_pos0 + RB - 1) / RB, cpt = KT / RB;
-    int tmax = (int)std::max(8L, (total * AKV + cus - 1) / cus);
+    int tmax = (int)std::max(6L, (total * AKV + cus - 1) / cus);
     while (tmax < longest && (parts_upto(p + nb, cpt * tmax) - parts_upto(p, cpt * tmax)) * AKV > cus) tmax++;
     if (longest - tmax < min_gain) return ks;                    // the merge launch has to be earned
     const long c = cpt * tmax;
