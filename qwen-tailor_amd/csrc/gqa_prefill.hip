@@ -620,7 +620,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const _Float16*
 
 namespace {
 
-inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 288; }   // from 4577 rows on (4096: 127 / 142 us, 4608: 163 / 158 us)
+inline bool two_heads_per_wave(int S) { return (S + 31) / 32 * AKV >= 288; }   // from 4577 rows on: 32-row blocks unsplit
 
 // The key split of a launch: tmax = 0 (none) or the tiles per part, parts = grid width, split_blocks = blocks with several parts.
 // Only launches that leave CUs without a workgroup are split (fewer than 2048 query rows: a short continuation of a long
@@ -661,21 +661,21 @@ KeySplit plan_split_nh(int S, int L, int q_pos0, int nh, int min_gain) {
     ks.split_blocks = nb - (int)std::max(0L, c - p);
     return ks;
 }
-// The form of a launch, by measurement (us at q_pos0 = 0, one head per wavefront in its best form / two heads with the split:
-// S = 1280 30.6 / 35.7, 1536 39.4 / 37.7, 2048 57.5 / 47.0, 2560 70.2 / 64.6, 3072 84.4 / 88.5, 4096 130 / 132; after a prefix
-// two heads win by more: 1536 rows after 1000 keys 63.4 / 52.8, 2048 after 6000 201 / 174):
-//   from about 4600 rows on     two heads per wavefront, unsplit (enough 32-row blocks to balance themselves);
-//   from about 1500 rows on     two heads per wavefront with the key split, where the launch leaves room for it and, for a
-//                               whole prompt, up to about 2800 rows (a tile of a 32-row block costs 2.4 us against 2 x 1.6 -
-//                               2 us for two 16-row blocks, but its parts are twice the size);
-//   everything else             one head per wavefront, split if CUs would idle.
+// The form of a launch, by measurement (us at q_pos0 = 0, 16-row blocks (NH = 1) in their best form / 32-row blocks (NH = 2) with
+// the split: S = 1280 25.3 / 27.3, 1408 27.7 / 27.7, 1536 32.3 / 30.0, 2048 47.0 / 37.2, 2560 59.9 / 51.4, 2944 68.5 / 63.3,
+// 3072 71.0 / 69.8, 3200 76.3 / 75.5, 3328 79.3 / 82.5; unsplit 4096 108 / 114, 4608 138 / 131, 5120 167 / 149):
+//   from about 4600 rows on     NH = 2, unsplit (enough 32-row blocks to balance themselves);
+//   from about 1500 rows on     NH = 2 with the key split, where the launch leaves room for it and, for a whole prompt, up to
+//                               3200 rows (a tile of a 32-row block costs less than two tiles of 16-row blocks, but its parts
+//                               are twice the size); after a prefix NH = 2 wins by more;
+//   everything else             NH = 1, split if CUs would idle.
 KeySplit plan_split(int S, int L, int q_pos0) {
     if (two_heads_per_wave(S)) {                                 // (two heads: S >= 1472 in every case, so L >= one tile)
         KeySplit ks;
         ks.nh = 2;
         return ks;
     }
-    if (S >= 1472 && (q_pos0 > 0 || S <= 2816)) {
+    if (S >= 1472 && (q_pos0 > 0 || S <= 3200)) {
         const KeySplit ks = plan_split_nh(S, L, q_pos0, 2, 4);
         if (ks.tmax) return ks;
     }

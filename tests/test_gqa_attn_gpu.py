@@ -324,10 +324,10 @@ def test_prefill_causal_score_ranges(qt, dev, qscale):
                                          (1024, 3000, 1.0), (16, 5000, 1.0), (1, 4095, 1.0), (1000, 9, 40.0), (130, 2000, 0.05),
                                          # from about 1500 rows on: 32-row blocks, two heads per wavefront, with the split
                                          (1536, 0, 1.0), (2048, 0, 1.0), (1500, 23, 1.0), (2500, 7, 40.0), (1800, 5000, 1.0),
-                                         (2816, 0, 0.05), (2049, 2048, 1.0)])
+                                         (2816, 0, 0.05), (3200, 0, 1.0), (2049, 2048, 1.0)])
 def test_prefill_causal_key_split(qt, dev, S, P0, qscale):
     """Launches that leave half of the CUs idle are split along the keys (parts of a row block meet in a workspace and a second
-    kernel combines them): prompts of up to 2800 rows and continuations of a long prefix, positions that are no
+    kernel combines them): prompts of up to 3200 rows and continuations of a long prefix, positions that are no
     multiple of 16 (some rows of a block then see no key of the block's last part), rescaled and flat score ranges.  Checked
     against the float64 oracle on a sample of rows, and against the same launch without a workspace (unsplit)."""
     from qwen_tailor_amd import _lib as QL
