@@ -347,19 +347,26 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
                 }
                 // the pair's buffers are free once the output wavefront has read tile t - 1 out of them (it does so first
                 // thing in this iteration; the word was read some steps ago, so that its LDS latency is not waited for here).
-                // The wait is bounded: the word is always written, and a bound costs nothing.
+                // The wait is bounded (the word is always written, and a bound costs nothing); a wait that does run out must not
+                // pass in silence: the pair's rows are then rescaled by NaN, which every later stage carries to the output.
+                bool gave_up = false;
                 if (t > ta && __builtin_amdgcn_readfirstlane(taken_early) != t) {
-                    for (int spin = 0; spin < (1 << 16); spin++) {
-                        if (__builtin_amdgcn_readfirstlane(*lds_word(&taken_s[pr])) == t) break;
+                    gave_up = true;
+                    for (int spin = 0; spin < (1 << 20); spin++) {
+                        if (__builtin_amdgcn_readfirstlane(*lds_word(&taken_s[pr])) == t) {
+                            gave_up = false;
+                            break;
+                        }
                         __builtin_amdgcn_s_sleep(1);
                     }
                 }
                 asm volatile("" ::: "memory");
-                if (any_grow) {
+                if (any_grow || gave_up) {
 #pragma unroll
-                    for (int hh = 0; hh < NH; hh++) c_s[pr][hh][n] = corr[hh];    // all four groups store the same value
+                    for (int hh = 0; hh < NH; hh++)              // all four groups store the same value
+                        c_s[pr][hh][n] = gave_up ? __builtin_nanf("") : corr[hh];
                 }
-                moved_s[pr] = any_grow ? 1 : 0;
+                moved_s[pr] = any_grow || gave_up ? 1 : 0;
 #pragma unroll
                 for (int hh = 0; hh < NH; hh++)
 #pragma unroll
