@@ -271,9 +271,10 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
             }
             __builtin_amdgcn_sched_barrier(0);
         };
-        f32x4 acc[NH][4] = {};                                   // scores of tile t
-        if (tw > ta) first_scores(acc);
-        for (int t = ta; t <= tb; t++) {
+        // the scores of tile t live in accs[(t - ta) & 1]: two iterations in the source, so that both sets are registers
+        f32x4 accs[2][NH][4] = {};
+        if (tw > ta) first_scores(accs[0]);
+        auto s_iter = [&](const int t, f32x4 (&acc)[NH][4], f32x4 (&acc_next)[NH][4]) {
             const unsigned par = (unsigned)(t - ta) & 1u;
             const unsigned k_cur = lds_address(kv_s) + par * (2 * TILE);           // K(t): consumed, refilled with K(t + 2)
             const bf16_t* const k_nxt = kv_s + (par ^ 1u) * TILE;                  // K(t + 1)
@@ -294,7 +295,7 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
                 if (t < tb) load_four(vg, v_new, t, opaque_off0());
             }
             PHASE_FENCE();
-            if (t >= tw) continue;
+            if (t >= tw) return;
             // only tiles that touch the diagonal or the end of the sequence need the mask (wavefront-uniform)
             if (t * KT + KT - 1 > q_pos0 + r0 || t * KT + KT > L) {
 #pragma unroll
@@ -308,7 +309,6 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
                         }
             }
             const bf16_t* ka = k_nxt + ka_row;
-            f32x4 acc_next[NH][4];
             // Online softmax in base 2 on the raw products: p = 2^(c s - m), c = 256^-0.5 log2 e; every row sees key 0, so its
             // maximum is finite from the first tile on and masked entries come out as 2^-huge = 0.  The exponentials are taken
             // against the running reference point of each row at once, on the bet that no row's maximum grows by more than
@@ -428,13 +428,10 @@ __global__ __launch_bounds__(512) void attn_prefill_kernel(const bf16_t* __restr
             else
                 body(std::false_type{});
             PHASE_FENCE();
-            if (more) {
-#pragma unroll
-                for (int hh = 0; hh < NH; hh++)
-#pragma unroll
-                    for (int kt = 0; kt < 4; kt++) acc[hh][kt] = acc_next[hh][kt];
-            }
-            PHASE_FENCE();
+        };
+        for (int t = ta; t <= tb; t += 2) {
+            s_iter(t, accs[0], accs[1]);
+            if (t + 1 <= tb) s_iter(t + 1, accs[1], accs[0]);
         }
         return;
     }
