@@ -353,9 +353,11 @@ def bench_attn_glue(torch, qt, dev, R=2048, seed=5):
     pos = torch.zeros(1, dtype=torch.int32, device=dev)
     o = torch.randn((R, 8, 256), generator=g).to(bf).to(dev)
     t1 = time_graph(torch, lambda: qt.attention.qkv_prep(qkv, qn, kn, pos, M=R), reps=60, inner=3)
+    t1t = time_graph(torch, lambda: qt.attention.qkv_prep(qkv, qn, kn, pos, M=R, max_pos=R), reps=60, inner=3)   # rotary pairs from the table
     t2 = time_graph(torch, lambda: qt.attention.out_gate(o, qkv), reps=60, inner=3)
     b1, b2 = R * (3072 + 3072) * 2, R * (2048 * 3) * 2          # q, k, v columns in + out; o, gate in + out
-    return {"rows": R, "qkv_prep_us": t1 * 1e6, "qkv_prep_GBps": b1 / t1 / 1e9, "out_gate_us": t2 * 1e6, "out_gate_GBps": b2 / t2 / 1e9}
+    return {"rows": R, "qkv_prep_us": t1 * 1e6, "qkv_prep_GBps": b1 / t1 / 1e9, "qkv_prep_table_us": t1t * 1e6,
+            "out_gate_us": t2 * 1e6, "out_gate_GBps": b2 / t2 / 1e9}
 
 
 def bench_projections(torch, qt, dev, B=64, seed=9):

@@ -178,9 +178,14 @@ int qt_gqa_prefill_causal(const void* q, const void* K, const void* V, void* out
  * qwen35/model.py:154-169).  qkv [R,5120] bf16 = [(q_h[256] | gate_h[256]) for 8 heads | k[2][256] | v[2][256]].
  * qt_attn_qkv_prep: q [R,8,256], k [R,2,256] = rope(rms_norm(., q_norm / k_norm [256] bf16, eps), position), v [R,2,256] = v;
  * rotary embedding of the first 64 features, half-split pairing, theta 1e7; row r = b*M + j sits at position pos[b] + j.
+ * qt_attn_qkv_prep_table: the same (the same call of the reference, the same bits) with the (cos, sin) pairs of positions
+ * 0 .. table_positions - 1 read from rope_table (as for qt_gqa_attn_layer_decode above; may be null) instead of evaluated
+ * per row; rows at positions beyond the table evaluate their own.
  * qt_attn_out_gate: out [R,2048] = o [R,8,256] * sigmoid(gate). */
 int qt_attn_qkv_prep(const void* qkv, const void* q_norm, const void* k_norm, const int32_t* pos, void* q, void* k, void* v, long R,
                      int M, float eps, qt_stream_t stream);
+int qt_attn_qkv_prep_table(const void* qkv, const void* q_norm, const void* k_norm, const int32_t* pos, const void* rope_table,
+                           int table_positions, void* q, void* k, void* v, long R, int M, float eps, qt_stream_t stream);
 int qt_attn_out_gate(const void* o, const void* qkv, void* out, long R, qt_stream_t stream);
 
 /* The projections either side of the core at decode / verify time: the reference's fused_gemv (qwen35/kernels.py:80-319) on

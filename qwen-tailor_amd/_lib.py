@@ -39,6 +39,7 @@ _SIGS = {
     "qt_gdn_phase_a_conv": [_vp] * 13 + [_i, _vp],
     "qt_blit": [_vp, _vp, _i, _l, _l, _l, _l, _l, _l, _vp],
     "qt_attn_qkv_prep": [_vp] * 7 + [_l, _i, _f, _vp],
+    "qt_attn_qkv_prep_table": [_vp] * 5 + [_i] + [_vp] * 3 + [_l, _i, _f, _vp],
     "qt_attn_out_gate": [_vp, _vp, _vp, _l, _vp],
     "qt_blit_batch": [_vp, _vp, _vp, _i, _vp],
     "qt_rms_rows": [_vp, _vp, _vp, _i, _i, _f, _vp],

@@ -43,11 +43,14 @@ def scaled_dot_product_attention(q, k, v, *, scale: float, mask="causal"):
 QKV_W = 8 * 512 + 2 * 2 * 256
 
 
-def qkv_prep(qkv, q_norm, k_norm, pos, M=1, eps=1e-6):
+def qkv_prep(qkv, q_norm, k_norm, pos, M=1, eps=1e-6, max_pos=None):
     """The steps between the qkv projection and the attention kernel of a full-attention layer (qwen35/batch.py:505-512,
     qwen35/model.py:154-164): split the 5120-wide rows into q / gate / k / v, RMS-normalise q and k per head (weights [256]
     bf16), rotate their first 64 features to the row's position.  qkv [R,5120] bf16, pos int32 [R / M] (row b*M + j sits at
-    pos[b] + j).  Returns q [R,8,256], k [R,2,256], v [R,2,256] bf16; the gate stays in qkv (out_gate reads it there)."""
+    pos[b] + j).  Returns q [R,8,256], k [R,2,256], v [R,2,256] bf16; the gate stays in qkv (out_gate reads it there).
+    max_pos: a bound of the positions that the caller knows on the host (a prefill knows its key count): the rotary (cos,
+    sin) pairs then come from the device's table of positions 0 .. max_pos instead of being evaluated per row (same bits;
+    a row beyond the bound still evaluates its own)."""
     qkv = L.dev(qkv, BF16, "qkv", (None, QKV_W))
     R = qkv.shape[0]
     if M < 1 or R % M:
@@ -56,7 +59,12 @@ def qkv_prep(qkv, q_norm, k_norm, pos, M=1, eps=1e-6):
     qn, kn = L.dev(q_norm, BF16, "q_norm", (256,)), L.dev(k_norm, BF16, "k_norm", (256,))
     q = torch.empty((R, 8, 256), dtype=BF16, device=qkv.device)
     k, v = (torch.empty((R, 2, 256), dtype=BF16, device=qkv.device) for _ in range(2))
-    L.call("qt_attn_qkv_prep", L.ptr(qkv), L.ptr(qn), L.ptr(kn), L.ptr(pos), L.ptr(q), L.ptr(k), L.ptr(v), R, M, float(eps), L.stream())
+    if max_pos is None:
+        L.call("qt_attn_qkv_prep", L.ptr(qkv), L.ptr(qn), L.ptr(kn), L.ptr(pos), L.ptr(q), L.ptr(k), L.ptr(v), R, M, float(eps), L.stream())
+    else:
+        table, n_pos = L.rope_table(qkv.device, int(max_pos) + 1)
+        L.call("qt_attn_qkv_prep_table", L.ptr(qkv), L.ptr(qn), L.ptr(kn), L.ptr(pos), L.ptr(table), n_pos, L.ptr(q), L.ptr(k), L.ptr(v),
+               R, M, float(eps), L.stream())
     return q, k, v
 
 

@@ -25,13 +25,15 @@ __constant__ float rope_freq[ROPE_DIM / 2] = {
     2.54829683e-05f, 1.5399266e-05f, 9.3057206e-06f, 5.62341347e-06f, 3.39820826e-06f, 2.05352512e-06f,
     1.24093776e-06f, 7.49894184e-07f, 4.5315835e-07f, 2.73841977e-07f, 1.65481708e-07f};
 
-// One workgroup per row r = b * M + j (position pos[b] + j): threads 0..31 evaluate the row's 32 (cos, sin) pairs once
-// (double-precision libm, the expensive part) into LDS; then a wavefront takes one 256-wide vector at a time (lane l holds
-// elements 4l .. 4l+3) out of the row's 12: 0..7 = q heads, 8..9 = k heads, 10..11 = v heads.
+// One workgroup per row r = b * M + j (position pos[b] + j): threads 0..31 bring the row's 32 (cos, sin) pairs into LDS, from
+// the table of rope_table_kernel where it covers the position, else evaluated here (double-precision libm, the expensive part:
+// the same expression, so the same bits); then a wavefront takes one 256-wide vector at a time (lane l holds elements
+// 4l .. 4l+3) out of the row's 12: 0..7 = q heads, 8..9 = k heads, 10..11 = v heads.
 __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict__ q_norm,
                                                             const bf16_t* __restrict__ k_norm, const int* __restrict__ pos,
                                                             bf16_t* __restrict__ q, bf16_t* __restrict__ k, bf16_t* __restrict__ v,
-                                                            long R, int M, float eps) {
+                                                            long R, int M, float eps, const float2* __restrict__ table,
+                                                            int table_positions) {
     __shared__ float cs_s[2][ROPE_DIM / 2];
     const long r = blockIdx.x;
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -45,10 +47,16 @@ __global__ __launch_bounds__(256) void attn_qkv_prep_kernel(const bf16_t* __rest
     }
     const uint2 wq = reinterpret_cast<const uint2*>(q_norm)[lane], wk = reinterpret_cast<const uint2*>(k_norm)[lane];
     if (threadIdx.x < ROPE_DIM / 2) {
-        const float p = (float)(pos[r / M] + (int)(r % M));
-        const float th = __fmul_rn(p, rope_freq[threadIdx.x]);
-        cs_s[0][threadIdx.x] = (float)cos((double)th);
-        cs_s[1][threadIdx.x] = (float)sin((double)th);
+        const int ip = pos[r / M] + (int)(r % M);
+        if (ip >= 0 && ip < table_positions) {                   // (table_positions = 0 without a table)
+            const float2 cs = table[(size_t)ip * (ROPE_DIM / 2) + threadIdx.x];
+            cs_s[0][threadIdx.x] = cs.x;
+            cs_s[1][threadIdx.x] = cs.y;
+        } else {
+            const float th = __fmul_rn((float)ip, rope_freq[threadIdx.x]);
+            cs_s[0][threadIdx.x] = (float)cos((double)th);
+            cs_s[1][threadIdx.x] = (float)sin((double)th);
+        }
     }
     __syncthreads();
 #pragma unroll
@@ -124,17 +132,24 @@ __global__ __launch_bounds__(256) void attn_out_gate_kernel(const bf16_t* __rest
 
 extern "C" {
 
-int qt_attn_qkv_prep(const void* qkv, const void* q_norm, const void* k_norm, const int32_t* pos, void* q, void* k, void* v, long R,
-                     int M, float eps, hipStream_t stream) {
+// rope_table: null, or the (cos, sin) pairs of positions 0 .. table_positions - 1 as qt_rope_table_build writes them; rows at
+// positions beyond the table evaluate their pairs themselves, with the same bits
+int qt_attn_qkv_prep_table(const void* qkv, const void* q_norm, const void* k_norm, const int32_t* pos, const void* rope_table,
+                           int table_positions, void* q, void* k, void* v, long R, int M, float eps, hipStream_t stream) {
     if (!qkv || !q_norm || !k_norm || !pos || !q || !k || !v) return QT_ERR_NULL;
-    if (R < 0 || M < 1 || R % M) return QT_ERR_DIM;
+    if (R < 0 || M < 1 || R % M || table_positions < 0) return QT_ERR_DIM;
     if (R == 0) return QT_OK;
-    for (const void* p : {qkv, q_norm, k_norm, (const void*)q, (const void*)k, (const void*)v})
+    for (const void* p : {qkv, q_norm, k_norm, rope_table, (const void*)q, (const void*)k, (const void*)v})
         if (reinterpret_cast<uintptr_t>(p) & 7u) return QT_ERR_ALIGN;
     hipLaunchKernelGGL(attn_qkv_prep_kernel, dim3((unsigned)R), dim3(256), 0, stream, (const bf16_t*)qkv, (const bf16_t*)q_norm,
-                       (const bf16_t*)k_norm, pos, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, R, M, eps);
+                       (const bf16_t*)k_norm, pos, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v, R, M, eps, (const float2*)rope_table,
+                       rope_table ? table_positions : 0);
     QT_CHECK_LAUNCH();
     return QT_OK;
+}
+int qt_attn_qkv_prep(const void* qkv, const void* q_norm, const void* k_norm, const int32_t* pos, void* q, void* k, void* v, long R,
+                     int M, float eps, hipStream_t stream) {
+    return qt_attn_qkv_prep_table(qkv, q_norm, k_norm, pos, nullptr, 0, q, k, v, R, M, eps, stream);
 }
 
 int qt_rope_table_build(void* table, int n_pos, hipStream_t stream) {

@@ -64,6 +64,8 @@ def test_null_and_dimension_errors_from_the_c_abi():
     assert lib.qt_blit(p16, p16, 2, 0, 0, 0, 1, 0, 0, z) == 0                        # nothing to copy: no launch
     assert lib.qt_attn_qkv_prep(p16, p16, p16, p16, p16, p16, p16, 6, 4, 1e-6, z) == -1      # M must divide the rows
     assert lib.qt_attn_qkv_prep(p16, p16, p16, z, p16, p16, p16, 4, 4, 1e-6, z) == -3
+    assert lib.qt_attn_qkv_prep_table(p16, p16, p16, p16, z, 0, p16, p16, p16, 6, 4, 1e-6, z) == -1
+    assert lib.qt_attn_qkv_prep_table(p16, p16, p16, p16, p16, -1, p16, p16, p16, 4, 4, 1e-6, z) == -1
     assert lib.qt_attn_out_gate(p16, ctypes.c_void_p(8), p16, 1, z) == -2
     assert lib.qt_gdn_phase_a_conv(p16, p16, p16, p16, p16, p16, p16, z, z, z, p16, p16, p16, 64, z) == -3   # q without k, v
     assert lib.qt_gdn_phase_a_conv(p16, p16, p16, p16, p16, p16, z, z, z, p16, p16, p16, p16, 64, z) == -4   # conv_out aliases conv_state

@@ -427,6 +427,11 @@ def test_qkv_prep_and_out_gate_bit_exact(qt, dev, R, M):
     check_equal("q", to_np(q), oq)
     check_equal("k", to_np(k), ok)
     check_equal("v", to_np(v), ov)
+    # the same with the rotary pairs read from the device's table: every position inside it, and a table that ends below
+    # most positions (those rows evaluate their own pairs): the same bits either way
+    for bound in (int(pos.max()) + M, 1000):
+        qt_, kt_, vt_ = qt.attention.qkv_prep(dq, to_dev(qn, dev, BF16), to_dev(kn, dev, BF16), to_dev(pos, dev), M, max_pos=bound)
+        assert torch.equal(qt_, q) and torch.equal(kt_, k) and torch.equal(vt_, v), f"table up to {bound}"
     o = bf(rng.standard_normal((R, 8, 256)))
     if R >= 256:                                                 # tiny, huge, zero and -0 gates among the ordinary ones
         special = bf(np.array([1e-7, -3e-6, 200.0, -150.0, 0.0, -0.0, 127.5, -1e-30]))
